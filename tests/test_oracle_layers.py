@@ -1,0 +1,247 @@
+"""Pins the CPU oracle's layer arithmetic against things it did not come from:
+torch autograd on an independently written float64 model, central finite
+differences, brute-force attention rows, scipy/torch special functions and
+algebraic invariants."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from jaxpp_amd.model import LayerSpec, init_layer_params
+from oracle import layers as L
+
+torch.set_num_threads(4)
+
+SPECS = {
+    "bert": LayerSpec("bert", 32, 4, 64, 8, 2, eps=1e-12),
+    "bert_tanh": LayerSpec("bert", 32, 4, 64, 8, 2, eps=1e-6, gelu_tanh=True),
+    "llama": LayerSpec("llama", 32, 4, 48, 8, 2, n_kv_heads=2, head_dim=8, causal=True,
+                       rope_theta=1e4, eps=1e-5),
+    "llama_mha": LayerSpec("llama", 32, 4, 48, 6, 1, n_kv_heads=4, head_dim=8, causal=True,
+                           rope_theta=5e5, eps=1e-5),
+    "mixtral": LayerSpec("mixtral", 32, 4, 24, 8, 2, n_kv_heads=2, head_dim=8, causal=True,
+                         rope_theta=1e4, eps=1e-5, n_experts=4, top_k=2),
+}
+
+
+def cfg_of(spec):
+    return L.LayerCfg(**spec.as_dict())
+
+
+# ---------------------------------------------------------------------------
+# an independent torch model (autograd supplies every gradient)
+# ---------------------------------------------------------------------------
+def torch_layer(spec, p, x):
+    T, h, d, B, S = spec.tokens, spec.hidden, spec.d, spec.batch, spec.seq
+    Hq, Hkv = spec.n_heads, spec.kvh
+
+    def attn(q, k, v):
+        q = q.view(B, S, Hq, d).permute(0, 2, 1, 3)
+        k = k.view(B, S, Hkv, d).permute(0, 2, 1, 3).repeat_interleave(Hq // Hkv, 1)
+        v = v.view(B, S, Hkv, d).permute(0, 2, 1, 3).repeat_interleave(Hq // Hkv, 1)
+        s = q @ k.transpose(-1, -2) / math.sqrt(d)
+        if spec.causal:
+            s = s.masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool), 1), float("-inf"))
+        return (torch.softmax(s, -1) @ v).permute(0, 2, 1, 3).reshape(T, Hq * d)
+
+    def rope(t, H):
+        t = t.view(B, S, H, d)
+        inv = spec.rope_theta ** (-torch.arange(0, d // 2, dtype=torch.float64) * 2 / d)
+        ang = torch.arange(S, dtype=torch.float64)[:, None] * inv[None]
+        z = torch.complex(t[..., :d // 2], t[..., d // 2:]) * torch.polar(
+            torch.ones_like(ang), ang)[None, :, None, :]
+        return torch.cat([z.real, z.imag], -1).reshape(T, H * d)
+
+    if spec.family == "bert":
+        qkv = x @ p["Wqkv"] + p["bqkv"]
+        q, k, v = qkv.split(h, -1)
+        a = attn(q, k, v) @ p["Wo"] + p["bo"] + x
+        x1 = torch.nn.functional.layer_norm(a, (h,), p["ln1_g"], p["ln1_b"], spec.eps)
+        g = torch.nn.functional.gelu(x1 @ p["W1"] + p["b1"],
+                                     approximate="tanh" if spec.gelu_tanh else "none")
+        c = g @ p["W2"] + p["b2"] + x1
+        return torch.nn.functional.layer_norm(c, (h,), p["ln2_g"], p["ln2_b"], spec.eps)
+
+    def rms(t, g):
+        return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + spec.eps) * g
+
+    n1 = rms(x, p["rms1_g"])
+    q, k, v = (n1 @ p["Wqkv"]).split([Hq * d, Hkv * d, Hkv * d], -1)
+    h1 = attn(rope(q, Hq), rope(k, Hkv), v) @ p["Wo"] + x
+    n2 = rms(h1, p["rms2_g"])
+    f = spec.ffn
+    if spec.family == "llama":
+        gu = n2 @ p["Wgu"]
+        return (torch.nn.functional.silu(gu[:, :f]) * gu[:, f:]) @ p["Wd"] + h1
+    logits = n2 @ p["Wr"]
+    top, ids = torch.topk(logits, spec.top_k, -1)
+    gates = torch.softmax(top, -1)
+    y = h1
+    for e in range(spec.n_experts):
+        gu = n2 @ p["Wgu"][e]
+        eo = (torch.nn.functional.silu(gu[:, :f]) * gu[:, f:]) @ p["Wd"][e]
+        w = (gates * (ids == e)).sum(-1, keepdim=True)
+        y = y + w * eo
+    return y
+
+
+def oracle_grads(spec, params, x, dy, nm):
+    cfg = cfg_of(spec)
+    y, st = L.layer_fwd(cfg, params, x, nm)
+    dx, wst, small = L.layer_bwd_i(cfg, params, st, dy, nm)
+    grads = dict(small)
+    grads.update(L.layer_bwd_w(cfg, st, wst, nm))
+    return y, dx, grads
+
+
+@pytest.mark.parametrize("name", list(SPECS))
+def test_layer_matches_torch_autograd(name):
+    spec = SPECS[name]
+    rng = np.random.default_rng(3)
+    params = {k: v.astype(np.float64) * (5.0 if v.ndim >= 2 else 1.0)
+              for k, v in init_layer_params(spec, 7, 0, perturb=True).items()}
+    x = rng.standard_normal((spec.tokens, spec.hidden))
+    dy = rng.standard_normal((spec.tokens, spec.hidden))
+    y, dx, grads = oracle_grads(spec, params, x, dy, L.Numerics.f64())
+
+    tp = {k: torch.tensor(v, requires_grad=True) for k, v in params.items()}
+    tx = torch.tensor(x, requires_grad=True)
+    ty = torch_layer(spec, tp, tx)
+    ty.backward(torch.tensor(dy))
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-9, atol=1e-10)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-8, atol=1e-10)
+    assert set(grads) == set(params)
+    for k in params:
+        np.testing.assert_allclose(grads[k], tp[k].grad.numpy(), rtol=1e-8, atol=1e-10,
+                                   err_msg=k)
+
+
+@pytest.mark.parametrize("name", ["bert", "llama", "mixtral"])
+def test_layer_finite_differences(name):
+    spec = SPECS[name]
+    cfg = cfg_of(spec)
+    nm = L.Numerics.f64()
+    rng = np.random.default_rng(11)
+    params = {k: v.astype(np.float64) * (5.0 if v.ndim >= 2 else 1.0)
+              for k, v in init_layer_params(spec, 5, 1, perturb=True).items()}
+    x = rng.standard_normal((spec.tokens, spec.hidden))
+    dy = rng.standard_normal((spec.tokens, spec.hidden))
+    _, dx, grads = oracle_grads(spec, params, x, dy, nm)
+
+    def loss(pp, xx):
+        return float((L.layer_fwd(cfg, pp, xx, nm)[0] * dy).sum())
+
+    eps = 1e-6
+    for k in list(params) + ["x"]:
+        base = x if k == "x" else params[k]
+        direction = rng.standard_normal(base.shape)
+        direction /= np.linalg.norm(direction)
+
+        def at(t):
+            if k == "x":
+                return loss(params, x + t * direction)
+            return loss({**params, k: params[k] + t * direction}, x)
+
+        fd = (at(eps) - at(-eps)) / (2 * eps)
+        an = float(((dx if k == "x" else grads[k]) * direction).sum())
+        assert abs(fd - an) <= 1e-5 * max(1.0, abs(an)), (k, fd, an)
+
+
+def test_bf16_rounding_matches_torch():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(4096).astype(np.float32) * 37.0,
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895e38, 1e-40,
+                                  np.inf, -np.inf], np.float32)])
+    want = torch.tensor(x).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(L.bf16_round(x), want)
+    bits = L.f32_to_bf16_bits(x)
+    np.testing.assert_array_equal(L.bf16_bits_to_f32(bits), want)
+    assert np.isnan(L.bf16_round(np.array([np.nan], np.float32)))[0]
+
+
+def test_gelu_and_silu_against_library_routines():
+    u = np.linspace(-6, 6, 1001)
+    tu = torch.tensor(u, requires_grad=True)
+    for tanh in (False, True):
+        g = torch.nn.functional.gelu(tu, approximate="tanh" if tanh else "none")
+        np.testing.assert_allclose(L.gelu(u, tanh), g.detach().numpy(), rtol=1e-12, atol=1e-14)
+        (gr,) = torch.autograd.grad(g.sum(), tu)
+        np.testing.assert_allclose(L.gelu_grad(u, tanh), gr.numpy(), rtol=1e-10, atol=1e-12)
+    gu = np.stack([u, u[::-1]], 0).reshape(1, -1)   # gate | up
+    f = u.size
+    s = torch.nn.functional.silu(torch.tensor(u)) * torch.tensor(u[::-1].copy())
+    np.testing.assert_allclose(L.swiglu(gu, f)[0], s.numpy(), rtol=1e-12)
+
+
+def test_attention_against_brute_force_rows():
+    from scipy.special import logsumexp
+    rng = np.random.default_rng(5)
+    B, S, Hq, Hkv, d = 2, 7, 4, 2, 8
+    q = rng.standard_normal((B, S, Hq, d))
+    k = rng.standard_normal((B, S, Hkv, d))
+    v = rng.standard_normal((B, S, Hkv, d))
+    for causal in (False, True):
+        o, lse = L.attention_fwd(q, k, v, causal, np.float64)
+        for b in range(B):
+            for hq in range(Hq):
+                hk = hq // (Hq // Hkv)
+                for i in range(S):
+                    hi = i + 1 if causal else S
+                    sc = np.array([q[b, i, hq] @ k[b, j, hk] for j in range(hi)]) / math.sqrt(d)
+                    w = np.exp(sc - sc.max())
+                    w /= w.sum()
+                    want = sum(w[j] * v[b, j, hk] for j in range(hi))
+                    np.testing.assert_allclose(o[b, i, hq], want, rtol=1e-12)
+                    np.testing.assert_allclose(lse[b, hq, i], logsumexp(sc), rtol=1e-12)
+
+
+def test_rope_is_a_rotation():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((2, 16, 3, 8))
+    cos, sin = L.rope_tables(16, 8, 1e4)
+    y = L.rope_apply(x, cos, sin)
+    np.testing.assert_allclose(np.linalg.norm(y, axis=-1), np.linalg.norm(x, axis=-1), rtol=1e-12)
+    np.testing.assert_allclose(L.rope_apply(y, cos, sin, inverse=True), x, atol=1e-12)
+    np.testing.assert_allclose(y[:, 0], x[:, 0], atol=0)          # position 0: identity
+    # relative-position property: <rope(q,m), rope(k,n)> depends on m-n only
+    q = rng.standard_normal(8)
+    kk = rng.standard_normal(8)
+    Q = L.rope_apply(np.broadcast_to(q, (1, 16, 1, 8)), cos, sin)[0, :, 0]
+    K = L.rope_apply(np.broadcast_to(kk, (1, 16, 1, 8)), cos, sin)[0, :, 0]
+    np.testing.assert_allclose(Q[5] @ K[2], Q[9] @ K[6], rtol=1e-10)
+
+
+def test_norms_against_torch():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((5, 16))
+    g, b = rng.standard_normal(16), rng.standard_normal(16)
+    y, mean, rstd = L.layernorm_fwd(x, g, b, 1e-5, np.float64)
+    want = torch.nn.functional.layer_norm(torch.tensor(x), (16,), torch.tensor(g),
+                                          torch.tensor(b), 1e-5).numpy()
+    np.testing.assert_allclose(y, want, rtol=1e-12)
+    np.testing.assert_allclose(mean, x.mean(-1), rtol=1e-12)
+    y, rstd = L.rmsnorm_fwd(x, g, 1e-5, np.float64)
+    np.testing.assert_allclose(rstd, 1 / np.sqrt((x ** 2).mean(-1) + 1e-5), rtol=1e-12)
+
+
+def test_moe_route_ties_and_gates():
+    logits = np.array([[1.0, 3.0, 3.0, 0.0], [2.0, 2.0, 2.0, 2.0], [0.0, -1.0, 5.0, 4.0]])
+    ids, gates = L.moe_route(logits, 2)
+    np.testing.assert_array_equal(ids, [[1, 2], [0, 1], [2, 3]])
+    np.testing.assert_allclose(gates[0], [0.5, 0.5])
+    np.testing.assert_allclose(gates[2], np.exp([5.0, 4.0]) / np.exp([5.0, 4.0]).sum())
+    np.testing.assert_allclose(gates.sum(-1), 1.0)
+
+
+def test_bf16_mode_stays_close_to_f32():
+    spec = SPECS["llama"]
+    params = init_layer_params(spec, 1, 0, perturb=True)
+    pb = {k: L.bf16_round(v) for k, v in params.items()}
+    rng = np.random.default_rng(4)
+    x = L.bf16_round(rng.standard_normal((spec.tokens, spec.hidden)).astype(np.float32))
+    dy = L.bf16_round(rng.standard_normal((spec.tokens, spec.hidden)).astype(np.float32))
+    y32, dx32, g32 = oracle_grads(spec, pb, x, dy, L.Numerics.f32())
+    y16, dx16, g16 = oracle_grads(spec, pb, x, dy, L.Numerics.bf16())
+    for a, b in [(y16, y32), (dx16, dx32)] + [(g16[k], g32[k]) for k in g32]:
+        assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max() + 1e-6

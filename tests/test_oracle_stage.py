@@ -1,0 +1,142 @@
+"""The oracle's loop executor: any valid schedule gives results bit-identical
+to the sequential ``treduce`` loop (the invariant the reference asserts in
+tests/test_transformations.py:187-191), split backward equals whole backward,
+and residual lifetimes follow the table."""
+import numpy as np
+import pytest
+
+from jaxpp_amd import schedules as S
+from jaxpp_amd.model import LayerSpec, boundary_tensor, init_layer_params
+from oracle import layers as L
+from oracle import stage as O
+
+SPEC = LayerSpec("bert", 16, 2, 32, 4, 2, eps=1e-12)
+LLAMA = LayerSpec("llama", 16, 2, 24, 4, 2, n_kv_heads=1, head_dim=8, causal=True, eps=1e-5)
+
+
+def build(spec, n_stages, layers_per_stage=1):
+    return [[init_layer_params(spec, 1, s * layers_per_stage + l, perturb=True)
+             for l in range(layers_per_stage)] for s in range(n_stages)]
+
+
+def xs_for(spec, n):
+    return [boundary_tensor("x", 0, m, (spec.tokens, spec.hidden)) for m in range(n)]
+
+
+GRID = [  # the reference's grid, tests/test_transformations.py:140-155
+    (1, 4, S.Std1F1B(num_stages=1)),
+    (2, 4, S.Std1F1B(num_stages=2)),
+    (3, 5, S.Eager1F1B(num_stages=3)),
+    (1, 1, S.Interleaved1F1B(num_stages=1, mpmd_dim=1)),
+    (8, 1, S.Interleaved1F1B(num_stages=8, mpmd_dim=4)),
+    (8, 1, S.KimiK2(num_stages=8, mpmd_dim=4, fuse_steady_state=True)),
+    (4, 12, S.Interleaved1F1B(num_stages=4, mpmd_dim=2)),
+    (4, 4, S.ZeroBubble(num_stages=4)),
+    (4, 8, S.ZeroBubble(num_stages=4)),
+    (6, 6, S.DualPipeV(num_stages=6, mpmd_dim=3)),
+    (6, 10, S.DualPipeV(num_stages=6, mpmd_dim=3)),
+    (3, 5, S.GPipe(num_stages=3)),
+]
+
+
+@pytest.mark.parametrize("n_stages,n,sched", GRID, ids=lambda v: str(v))
+@pytest.mark.parametrize("spec", [SPEC, LLAMA], ids=["bert", "llama"])
+def test_schedule_equals_sequential_bitwise(spec, n_stages, n, sched):
+    cfg = L.LayerCfg(**spec.as_dict())
+    nm = L.Numerics.f32()
+    stages = build(spec, n_stages)
+    xs = xs_for(spec, n)
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, xs, nm)
+    rows = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)
+    owner = [int(sched.get_mpmd_idx(s)) for s in range(n_stages)]
+    loss, acc, _ = O.run_pipeline(cfg, stages, rows, owner, xs, nm)
+    np.testing.assert_array_equal(loss, want_loss)
+    for s in range(n_stages):
+        for li, layer in enumerate(want_acc[s]):
+            for k, v in layer.items():
+                np.testing.assert_array_equal(acc[s][li][k], v, err_msg=f"{s}/{li}/{k}")
+
+
+def test_treduce_closed_form():
+    """losses are concatenated, gradients are the sum of per-microbatch ones."""
+    cfg = L.LayerCfg(**SPEC.as_dict())
+    nm = L.Numerics.f64()
+    stages = build(SPEC, 2)
+    xs = [x.astype(np.float64) for x in xs_for(SPEC, 3)]
+    loss, acc = O.treduce_sequential(cfg, stages, xs, nm)
+    tot = None
+    for m, x in enumerate(xs):
+        l1, a1 = O.treduce_sequential(cfg, stages, [x], nm)
+        np.testing.assert_allclose(loss[m], l1[0] / 3, rtol=1e-6)
+        g = a1[0][0]["Wqkv"] / 3
+        tot = g if tot is None else tot + g
+    np.testing.assert_allclose(acc[0][0]["Wqkv"], tot, rtol=1e-5, atol=1e-9)
+
+
+def test_mse_loss_gradient():
+    rng = np.random.default_rng(0)
+    a, b = rng.standard_normal((6, 5)), rng.standard_normal((6, 5))
+    loss, d = L.mse_loss(a, b, 8, np.float64)
+    assert np.isclose(loss, ((a - b) ** 2).mean() / 8)
+    e = np.zeros_like(a)
+    e[2, 3] = 1e-6
+    fd = (L.mse_loss(a + e, b, 8, np.float64)[0] - L.mse_loss(a - e, b, 8, np.float64)[0]) / 2e-6
+    assert np.isclose(fd, d[2, 3], rtol=1e-6)
+
+
+@pytest.mark.parametrize("sched,rank,n,peak", [
+    (S.Std1F1B(4), 0, 16, 4), (S.Std1F1B(4), 3, 16, 1),
+    (S.Interleaved1F1B(8, 4), 0, 8, 11), (S.ZeroBubble(4), 1, 8, 4),
+])
+def test_rank_row_with_synthetic_boundaries(sched, rank, n, peak):
+    """One rank alone, boundary tensors supplied from outside: the scheduled
+    row and the plain per-stage loop agree bit for bit, and the peak number
+    of live residual sets is what the table implies."""
+    spec = SPEC
+    cfg = L.LayerCfg(**spec.as_dict())
+    nm = L.Numerics.bf16()
+    row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
+    mine = [s for s in range(sched.num_stages) if int(sched.get_mpmd_idx(s)) == rank]
+    chunks = {s: [{k: L.bf16_round(v) for k, v in init_layer_params(spec, 2, s, True).items()}]
+              for s in mine}
+    shape = (spec.tokens, spec.hidden)
+    x_in = lambda s, m: L.bf16_round(boundary_tensor("x", s, m, shape))
+    dy_in = lambda s, m: L.bf16_round(boundary_tensor("dy", s, m, shape))
+    ro = O.RankOracle(cfg, chunks, nm)
+    ys, dxs = ro.run_row(row, x_in, dy_in)
+    assert ro.peak_live == peak
+    plain = O.RankOracle(cfg, chunks, nm)
+    for s in mine:
+        for m in range(n):
+            y = plain.fwd(s, m, x_in(s, m))
+            dx = plain.bwd(s, m, dy_in(s, m))
+            np.testing.assert_array_equal(ys[s, m], y)
+            np.testing.assert_array_equal(dxs[s, m], dx)
+    for s in mine:
+        for k, v in plain.acc[s][0].items():
+            np.testing.assert_array_equal(ro.acc[s][0][k], v)
+
+
+def test_invalid_table_raises():
+    cfg = L.LayerCfg(**SPEC.as_dict())
+    stages = build(SPEC, 2)
+    rows = S.preprocess_schedule_tasks(S.Std1F1B(2).tasks(2), 0, False)
+    rows[1] = rows[1][::-1]          # backward before forward on the last stage
+    with pytest.raises(AssertionError, match="does not honor data dependencies"):
+        O.run_pipeline(cfg, stages, rows, [0, 1], xs_for(SPEC, 2), L.Numerics.f32())
+
+
+def test_adam_step_matches_torch():
+    import torch
+    rng = np.random.default_rng(1)
+    p = {"w": rng.standard_normal((4, 3)).astype(np.float32)}
+    tp = torch.nn.Parameter(torch.tensor(p["w"]))
+    opt = torch.optim.Adam([tp], lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+    m = {"w": np.zeros_like(p["w"])}
+    v = {"w": np.zeros_like(p["w"])}
+    for step in (1, 2, 3):
+        g = rng.standard_normal((4, 3)).astype(np.float32)
+        tp.grad = torch.tensor(g)
+        opt.step()
+        p = O.adam_step(p, {"w": g}, m, v, step)
+        np.testing.assert_allclose(p["w"], tp.detach().numpy(), rtol=2e-6, atol=1e-7)
