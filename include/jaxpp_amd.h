@@ -1,0 +1,208 @@
+/* jaxpp_amd -- C ABI of the MI355X stage executor and its kernels.
+ *
+ * The reference (NVIDIA/jaxpp, Python on JAX/XLA) has no native interface for
+ * this path; what this library replaces is
+ *   - the op seam: the XLA executable a stage task compiles to
+ *     (src/jaxpp/jax_primitives.py:704-730, `callable_task` / `apply_task`),
+ *     i.e. the GEMM / attention / norm / activation / accumulate kernels; and
+ *   - the task seam: `task_impl` dispatching one (stage, kind, microbatch)
+ *     task on device buffers (src/jaxpp/jax_primitives.py:776-859).
+ * Each entry point below names the reference construct it stands in for.
+ *
+ * Conventions
+ *   - plain C, POD arguments, device pointers owned by the caller unless
+ *     stated; nothing here takes or returns framework tensor types;
+ *   - every function returns 0 (JPP_OK) or a negative jpp_status and never
+ *     throws or aborts; jpp_last_error() returns the thread's last message;
+ *   - kernels are enqueued on the given HIP stream and never synchronise;
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - bf16 tensors are raw uint16 bit patterns, row-major, leading dimension
+ *     in elements.
+ */
+#ifndef JAXPP_AMD_H_
+#define JAXPP_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  JPP_OK = 0,
+  JPP_ERR_INVALID = -1, /* shape / alignment / argument violation, found on host */
+  JPP_ERR_HIP = -2,     /* a HIP runtime call or launch failed */
+  JPP_ERR_STATE = -3    /* task order violates residual lifetimes */
+} jpp_status;
+
+/* TaskType of the reference (src/jaxpp/types.py:79-96); same integer values. */
+typedef enum { JPP_FWD = 1, JPP_BWD = 2, JPP_BWD_I = 3, JPP_BWD_W = 4 } jpp_task_kind;
+
+typedef enum { JPP_FAMILY_BERT = 0, JPP_FAMILY_LLAMA = 1, JPP_FAMILY_MIXTRAL = 2 } jpp_family;
+
+const char* jpp_last_error(void);
+int jpp_version(void);
+
+/* ---- device plumbing for hosts that have no GPU runtime of their own ------
+ * (a ctypes / FFI host; under JAX, XLA owns buffers and streams instead) */
+int jpp_device_count(int* count);
+int jpp_set_device(int device);
+int jpp_malloc(void** ptr, size_t bytes);
+int jpp_free(void* ptr);
+int jpp_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int jpp_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int jpp_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream);
+int jpp_fill_u32(void* dst, uint32_t value, size_t count, void* stream);
+int jpp_stream_create(void** stream);
+int jpp_stream_destroy(void* stream);
+int jpp_stream_sync(void* stream);
+int jpp_device_sync(void);
+int jpp_event_create(void** event);
+int jpp_event_destroy(void* event);
+int jpp_event_record(void* event, void* stream);
+int jpp_event_sync(void* event);
+int jpp_event_elapsed_ms(void* start, void* stop, float* ms);
+int jpp_mem_info(size_t* free_bytes, size_t* total_bytes);
+
+/* ---- GEMM: stands in for the `dot_general`s of a stage task ----------------
+ * C[M,N] = epilogue( sum_k Aop[m,k] * Bop[n,k] ), bf16 operands, fp32 MFMA
+ * accumulation.
+ *   trans_a = 0: A is [M,K] (lda >= K);  1: A is [K,M] (lda >= M)
+ *   trans_b = 0: B is [N,K] (ldb >= K);  1: B is [K,N] (ldb >= N)
+ * so  y = x W      -> trans_a 0, trans_b 1   (W stored [in,out])
+ *     dx = dy W^T  -> trans_a 0, trans_b 0
+ *     dW = x^T dy  -> trans_a 1, trans_b 1
+ * M and N must be multiples of 128, K of 64; all pointers 16-byte aligned and
+ * leading dimensions multiples of 8. */
+typedef enum {
+  JPP_EPI_BF16 = 0,    /* C(bf16) = acc [+ bias[n]] [+ resid[m,n]]                     */
+  JPP_EPI_GELU = 1,    /* u = acc + bias;  C = u,  C2 = gelu(u)   (both bf16)          */
+  JPP_EPI_DGELU = 2,   /* C(bf16) = acc * gelu'(aux[m,n])                              */
+  JPP_EPI_ACC_F32 = 3, /* C(f32) += acc      (the `add prev_acc g` of a backward task) */
+  JPP_EPI_F32 = 4      /* C(f32) = acc                                                 */
+} jpp_epilogue;
+
+typedef struct {
+  const void* a;
+  const void* b;
+  void* c;
+  void* c2;          /* second output (JPP_EPI_GELU) */
+  const void* bias;  /* bf16 [N] or NULL */
+  const void* resid; /* bf16 [M,N] or NULL */
+  const void* aux;   /* bf16 [M,N] (JPP_EPI_DGELU) */
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc, ldc2, ldresid, ldaux;
+  int trans_a, trans_b;
+  int epilogue;      /* jpp_epilogue */
+  int gelu_tanh;     /* 0: erf form, 1: tanh approximation */
+  int tile;          /* 0: choose; 1: 128x128; 2: 256x128; 3: 256x256 (tuning/tests) */
+} jpp_gemm_args;
+
+int jpp_gemm_bf16(void* stream, const jpp_gemm_args* args);
+
+/* ---- fused attention (softmax(QK^T/sqrt(d)) V), forward and backward -------
+ * q: [batch*seq, *] with head h at columns h*head_dim (row stride ldq); k, v
+ * likewise with n_kv_heads heads; query head h reads kv head h / (n_heads /
+ * n_kv_heads).  lse: f32 [batch, n_heads, seq], natural-log sum-exp of the
+ * scaled scores.  head_dim 64 or 128; seq a multiple of 128. */
+typedef struct {
+  const void* q; const void* k; const void* v;
+  void* o;                  /* fwd: out; bwd: in */
+  float* lse;               /* fwd: out; bwd: in */
+  const void* d_o;          /* bwd */
+  void* dq; void* dk; void* dv;
+  float* delta;             /* bwd scratch, f32 [batch, n_heads, seq] */
+  int64_t ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv;
+  int batch, seq, n_heads, n_kv_heads, head_dim, causal;
+} jpp_attn_args;
+
+int jpp_attn_fwd(void* stream, const jpp_attn_args* args);
+int jpp_attn_bwd(void* stream, const jpp_attn_args* args);
+
+/* ---- row-wise norms ---------------------------------------------------------
+ * x, y, dy, dx: bf16 [rows, cols]; gamma/beta bf16 [cols]; mean/rstd f32
+ * [rows].  The backward adds `resid` (bf16, may be NULL) to dx, and
+ * accumulates the parameter gradients into the f32 arrays dgamma / dbeta
+ * (`+=`, fixed summation order) using `partial` (f32 [2 * JPP_NORM_PARTIALS *
+ * cols]) as scratch.  beta == NULL and mean == NULL select RMSNorm. */
+#define JPP_NORM_PARTIALS 256
+typedef struct {
+  const void* x; const void* gamma; const void* beta;
+  void* y; float* mean; float* rstd;
+  const void* dy; const void* resid; void* dx;
+  float* dgamma; float* dbeta; float* partial;
+  int64_t rows, cols;
+  float eps;
+} jpp_norm_args;
+
+int jpp_norm_fwd(void* stream, const jpp_norm_args* args);
+int jpp_norm_bwd(void* stream, const jpp_norm_args* args);
+
+/* ---- elementwise ------------------------------------------------------------ */
+/* s[t,j] = silu(gu[t,j]) * gu[t,f+j]; backward writes dgu [T,2f]. */
+int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f);
+int jpp_swiglu_bwd(void* stream, const void* gu, const void* ds, void* dgu, int64_t rows,
+                   int64_t f);
+/* Half-split rotary embedding applied in place to the first n_rot_heads heads
+ * of each row (q and k heads are adjacent in a packed qkv row); cos/sin: f32
+ * [seq, head_dim/2]; inverse != 0 rotates by the negative angle (backward). */
+int jpp_rope(void* stream, void* x, int64_t ld, const float* cos_tab, const float* sin_tab,
+             int batch, int seq, int n_rot_heads, int head_dim, int inverse);
+/* acc[i] += g[i]; g is bf16 (g_is_f32 == 0) or f32.  The gradient accumulation
+ * of `treduce`'s Add (src/jaxpp/training.py:112-123) as a standalone pass. */
+int jpp_grad_accum_f32(void* stream, float* acc, const void* g, int64_t count, int g_is_f32);
+/* acc[j] += sum_t x[t,j] (bias gradients); partial: f32 [JPP_NORM_PARTIALS*cols]. */
+int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int64_t cols,
+                     float* acc, float* partial);
+int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count);
+int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count);
+
+/* ---- stage executor: stands in for `task_impl` on one pipeline rank ----------
+ * A stage object holds this rank's chunks (the stages the schedule places on
+ * it), their bf16 parameters, the f32 gradient accumulators (the loop carry of
+ * `treduce`), and a ring of residual slots sized for the schedule's peak
+ * number of live microbatches (src/jaxpp/core.py:1732-1890 decides the same
+ * lifetimes by donation and explicit deletes). */
+typedef struct jpp_stage jpp_stage;
+
+typedef struct {
+  int family;            /* jpp_family */
+  int hidden, n_heads, n_kv_heads, head_dim, ffn, seq, batch;
+  int causal;
+  float rope_theta;
+  float eps;
+  int gelu_tanh;
+  int n_experts, top_k;
+  int n_chunks;          /* stages held by this rank */
+  int layers_per_chunk;
+  int max_live;          /* residual slots */
+  int split_backward;    /* 1: BWD_I / BWD_W tasks will be issued separately */
+  int fused_wgrad_accum; /* 1: accumulate in the weight-gradient GEMM epilogue;
+                            0: bf16 gradient then jpp_grad_accum_f32 */
+} jpp_stage_desc;
+
+int jpp_stage_create(const jpp_stage_desc* desc, jpp_stage** out);
+int jpp_stage_destroy(jpp_stage* stage);
+/* Parameters of one layer, in a fixed order per family. */
+int jpp_stage_n_params(const jpp_stage* stage);
+int jpp_stage_param_info(const jpp_stage* stage, int index, const char** name, int64_t* rows,
+                         int64_t* cols);
+/* bf16 parameter / f32 accumulator storage of (chunk, layer, index). */
+int jpp_stage_param_ptr(jpp_stage* stage, int chunk, int layer, int index, void** ptr);
+int jpp_stage_grad_ptr(jpp_stage* stage, int chunk, int layer, int index, float** ptr);
+int jpp_stage_zero_grads(jpp_stage* stage, void* stream);
+size_t jpp_stage_bytes(const jpp_stage* stage);
+/* One task.  `in` is the incoming boundary activation (FWD) or cotangent
+ * (BWD, BWD_I), `out` receives the outgoing activation / cotangent; both are
+ * bf16 [batch*seq, hidden] and may be reused by the caller once the call has
+ * returned (stream order).  BWD_W takes neither.  A BWD_I that is never
+ * followed by BWD_W leaves its slot occupied. */
+int jpp_stage_run_task(jpp_stage* stage, int kind, int chunk, int mubatch, const void* in,
+                       void* out, void* stream);
+int jpp_stage_live_slots(const jpp_stage* stage);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JAXPP_AMD_H_ */

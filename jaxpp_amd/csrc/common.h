@@ -1,0 +1,145 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/jaxpp_amd.h"
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits as stored in HBM
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// -- error plumbing ---------------------------------------------------------
+// Every entry point returns 0 or a negative jpp_status and leaves a message
+// that jpp_last_error() hands back (thread local).
+int jpp_set_error(int code, const char* fmt, ...);
+
+#define JPP_CHECK_HIP(expr)                                                     \
+  do {                                                                          \
+    hipError_t e_ = (expr);                                                     \
+    if (e_ != hipSuccess)                                                       \
+      return jpp_set_error(JPP_ERR_HIP, "%s failed: %s (%s:%d)", #expr,         \
+                           hipGetErrorString(e_), __FILE__, __LINE__);          \
+  } while (0)
+
+#define JPP_REQUIRE(cond, ...)                                                  \
+  do {                                                                          \
+    if (!(cond)) return jpp_set_error(JPP_ERR_INVALID, __VA_ARGS__);            \
+  } while (0)
+
+#define JPP_LAUNCH_CHECK()                                                      \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess)                                                       \
+      return jpp_set_error(JPP_ERR_HIP, "kernel launch failed: %s (%s:%d)",     \
+                           hipGetErrorString(e_), __FILE__, __LINE__);          \
+  } while (0)
+
+// -- bf16 <-> f32 -------------------------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(bf16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) {
+  return __uint_as_float(w & 0xffff0000u);
+}
+// round to nearest even
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// -- LDS operand slabs ----------------------------------------------------------
+// A slab is [rows][64] bf16 (128 B per row, no padding).  The eight 16-byte
+// chunks of a row are XOR-swizzled with the row index so that both the MFMA
+// operand reads (32 consecutive rows, one chunk) and the transposing stores
+// (rows 8 apart, one chunk) spread over the LDS banks.
+__device__ __forceinline__ int slab_swz(int row) { return (row ^ (row >> 3)) & 7; }
+__device__ __forceinline__ int slab_off(int row, int chunk) {
+  return row * 128 + ((chunk ^ slab_swz(row)) << 4);
+}
+
+// MFMA operand fragment for v_mfma_f32_32x32x16_bf16: lane l supplies the row
+// (l & 31) and the 8 contraction elements of chunk 2*kstep + (l >> 5).
+__device__ __forceinline__ bf16x8 slab_frag(const uint8_t* slab, int row0, int kstep, int lane) {
+  int row = row0 + (lane & 31);
+  return *(const bf16x8*)(slab + slab_off(row, kstep * 2 + (lane >> 5)));
+}
+
+// Swap bits 2 and 3 of a contraction index.  An operand built straight from
+// MFMA accumulator registers enumerates its contraction index in the order
+// (reg/4, lane/32, reg%4); storing the LDS-side operand with those two bits
+// swapped makes both sides agree while keeping 16-byte fragment reads.
+__device__ __forceinline__ int swap_bits23(int k) {
+  return (k & ~0xC) | ((k & 4) << 1) | ((k & 8) >> 1);
+}
+
+// Cooperative loader of a (64 x ROWS) or (ROWS x 64) bf16 tile for 256 threads.
+//  TRANS = false: memory holds [ROWS][64..] with the contraction index
+//                 contiguous; a thread moves ROWS/32 16-byte chunks.
+//  TRANS = true : memory holds [64][ROWS..] (contraction index is the slow
+//                 one); a thread reads a (ROWS/32 x 8) block, transposes it in
+//                 registers and writes 8 short runs of contraction elements.
+//  KPERM        : store contraction index k at position swap_bits23(k).
+template <int ROWS, bool TRANS, bool KPERM = false>
+struct TileLoader {
+  static constexpr int NV = ROWS / 32;
+  static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "ROWS");
+  static_assert(!KPERM || (TRANS && NV <= 4), "KPERM needs short transposed runs");
+  typedef uint4 Regs[NV];
+
+  static __device__ __forceinline__ void load(Regs& r, const bf16_t* __restrict__ src, long ld,
+                                              int tid) {
+    if constexpr (!TRANS) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+        r[i] = *(const uint4*)(src + (long)((tid >> 3) + 32 * i) * ld + (tid & 7) * 8);
+    } else {
+      const int rb = tid % (ROWS / 8), kb = tid / (ROWS / 8);
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+        r[j] = *(const uint4*)(src + (long)(kb * NV + j) * ld + rb * 8);
+    }
+  }
+
+  static __device__ __forceinline__ void store(const Regs& r, uint8_t* slab, int tid) {
+    if constexpr (!TRANS) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        int row = (tid >> 3) + 32 * i;
+        *(uint4*)(slab + slab_off(row, tid & 7)) = r[i];
+      }
+    } else {
+      const int rb = tid % (ROWS / 8), kb = tid / (ROWS / 8);
+      int k0 = kb * NV;
+      if constexpr (KPERM) k0 = swap_bits23(k0);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int row = rb * 8 + c;
+        uint32_t w[NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+          const uint4 v = r[j];
+          w[j] = (c >> 1) == 0 ? v.x : (c >> 1) == 1 ? v.y : (c >> 1) == 2 ? v.z : v.w;
+        }
+        uint32_t o[NV / 2];
+#pragma unroll
+        for (int q = 0; q < NV / 2; ++q)
+          o[q] = (c & 1) ? ((w[2 * q] >> 16) | (w[2 * q + 1] & 0xffff0000u))
+                         : ((w[2 * q] & 0xffffu) | (w[2 * q + 1] << 16));
+        uint8_t* dst = slab + slab_off(row, k0 >> 3) + (k0 & 7) * 2;
+        if constexpr (NV == 8) {
+          *(uint4*)dst = make_uint4(o[0], o[1], o[2], o[3]);
+        } else if constexpr (NV == 4) {
+          *(uint2*)dst = make_uint2(o[0], o[1]);
+        } else {
+          *(uint32_t*)dst = o[0];
+        }
+      }
+    }
+  }
+};

@@ -1,0 +1,525 @@
+// HBM-bound kernels of a stage task: LayerNorm / RMSNorm forward and
+// backward, SwiGLU, rotary embedding, gradient accumulation, bias-gradient
+// column sums and dtype casts.  All move 16 bytes per lane per access and keep
+// statistics in fp32.  Parameter gradients are reduced in a fixed order
+// (per-block partial sums, then one ordered pass) so results do not depend on
+// scheduling.
+#include <math.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kMaxChunksPerLane = 16;  // a wave holds one row of <= 8192 columns
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+  f[0] = bf16lo_to_f32(v.x); f[1] = bf16hi_to_f32(v.x);
+  f[2] = bf16lo_to_f32(v.y); f[3] = bf16hi_to_f32(v.y);
+  f[4] = bf16lo_to_f32(v.z); f[5] = bf16hi_to_f32(v.z);
+  f[6] = bf16lo_to_f32(v.w); f[7] = bf16hi_to_f32(v.w);
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+  return make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                    pack_bf16x2(f[6], f[7]));
+}
+
+// ---------------------------------------------------------------------------
+// norm forward: one wave per row, the row cached in registers
+// ---------------------------------------------------------------------------
+template <bool LN, int NCH>
+__global__ __launch_bounds__(256) void norm_fwd_kernel(const bf16_t* __restrict__ x,
+                                                       const bf16_t* __restrict__ gamma,
+                                                       const bf16_t* __restrict__ beta,
+                                                       bf16_t* __restrict__ y,
+                                                       float* __restrict__ mean_out,
+                                                       float* __restrict__ rstd_out, long rows,
+                                                       int cols, float eps) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nchunk = cols >> 3;
+  const uint4* xr = (const uint4*)(x + row * cols);
+  uint4 v[NCH];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + 64 * i;
+    v[i] = c < nchunk ? xr[c] : make_uint4(0, 0, 0, 0);
+    float f[8];
+    unpack8(v[i], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += LN ? f[e] : f[e] * f[e];
+  }
+  s = wave_sum(s);
+  float mean = 0.f, var;
+  if (LN) {
+    mean = s / cols;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      if (lane + 64 * i < nchunk) {
+        float f[8];
+        unpack8(v[i], f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) q += (f[e] - mean) * (f[e] - mean);
+      }
+    }
+    var = wave_sum(q) / cols;
+  } else {
+    var = s / cols;
+  }
+  const float rstd = 1.0f / sqrtf(var + eps);
+  if (lane == 0) {
+    rstd_out[row] = rstd;
+    if (LN) mean_out[row] = mean;
+  }
+  uint4* yr = (uint4*)(y + row * cols);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + 64 * i;
+    if (c < nchunk) {
+      float f[8], g[8], b[8];
+      unpack8(v[i], f);
+      unpack8(((const uint4*)gamma)[c], g);
+      if (LN) unpack8(((const uint4*)beta)[c], b);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = (f[e] - mean) * rstd * g[e] + (LN ? b[e] : 0.f);
+      yr[c] = pack8(f);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// norm backward: dx per row, and per-block partial sums of dgamma / dbeta
+// ---------------------------------------------------------------------------
+template <bool LN, int NCH>
+__global__ __launch_bounds__(256) void norm_bwd_kernel(
+    const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x, const float* __restrict__ mean_in,
+    const float* __restrict__ rstd_in, const bf16_t* __restrict__ gamma,
+    const bf16_t* __restrict__ resid, bf16_t* __restrict__ dx, float* __restrict__ partial,
+    long rows, int cols) {
+  __shared__ float red[4][64 * 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nchunk = cols >> 3;
+  const long stride = (long)gridDim.x * 4;
+  float pg[NCH][8], pb[LN ? NCH : 1][8];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pg[i][e] = 0.f;
+      if (LN) pb[i][e] = 0.f;
+    }
+  for (long row = (long)blockIdx.x * 4 + wave; row < rows; row += stride) {
+    const float rstd = rstd_in[row];
+    const float mean = LN ? mean_in[row] : 0.f;
+    const uint4* xr = (const uint4*)(x + row * cols);
+    const uint4* dyr = (const uint4*)(dy + row * cols);
+    uint4 vx[NCH], vd[NCH];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = lane + 64 * i;
+      if (c < nchunk) {
+        vx[i] = xr[c];
+        vd[i] = dyr[c];
+        float fx[8], fd[8], g[8];
+        unpack8(vx[i], fx);
+        unpack8(vd[i], fd);
+        unpack8(((const uint4*)gamma)[c], g);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xh = (fx[e] - mean) * rstd;
+          const float dg = fd[e] * g[e];
+          s1 += dg;
+          s2 += dg * xh;
+          pg[i][e] += fd[e] * xh;
+          if (LN) pb[i][e] += fd[e];
+        }
+      }
+    }
+    s2 = wave_sum(s2) / cols;
+    s1 = LN ? wave_sum(s1) / cols : 0.f;
+    uint4* dxr = (uint4*)(dx + row * cols);
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = lane + 64 * i;
+      if (c < nchunk) {
+        float fx[8], fd[8], g[8], r[8];
+        unpack8(vx[i], fx);
+        unpack8(vd[i], fd);
+        unpack8(((const uint4*)gamma)[c], g);
+        if (resid) unpack8(((const uint4*)(resid + row * cols))[c], r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xh = (fx[e] - mean) * rstd;
+          float o = (fd[e] * g[e] - s1 - xh * s2) * rstd;
+          if (resid) o += r[e];
+          fx[e] = o;
+        }
+        dxr[c] = pack8(fx);
+      }
+    }
+  }
+  // combine the 4 waves of the block in a fixed order, one chunk column at a time
+  float* pgam = partial + (long)blockIdx.x * cols;
+  float* pbet = partial + ((long)gridDim.x + blockIdx.x) * cols;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + 64 * i;
+#pragma unroll
+    for (int pass = 0; pass < (LN ? 2 : 1); ++pass) {
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[wave][lane * 8 + e] = pass ? pb[LN ? i : 0][e] : pg[i][e];
+      __syncthreads();
+      if (wave == 0 && c < nchunk) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float t = ((red[0][lane * 8 + e] + red[1][lane * 8 + e]) + red[2][lane * 8 + e]) +
+                          red[3][lane * 8 + e];
+          (pass ? pbet : pgam)[c * 8 + e] = t;
+        }
+      }
+    }
+  }
+}
+
+// acc[j] += sum_b partial[b][j], b ascending
+__global__ __launch_bounds__(256) void partial_reduce_kernel(const float* __restrict__ partial,
+                                                             int nblocks, int cols,
+                                                             float* __restrict__ acc) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= cols) return;
+  float s = 0.f;
+  for (int b = 0; b < nblocks; ++b) s += partial[(long)b * cols + j];
+  acc[j] += s;
+}
+
+// ---------------------------------------------------------------------------
+// column sums (bias gradients): block b sums rows b, b+nb, ... of a 2048-wide
+// column panel
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const bf16_t* __restrict__ x, long ld,
+                                                             long rows, int cols,
+                                                             float* __restrict__ partial) {
+  const int c = blockIdx.y * 256 + threadIdx.x;  // 8-column chunk
+  if (c * 8 >= cols) return;
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (long row = blockIdx.x; row < rows; row += gridDim.x) {
+    float f[8];
+    unpack8(*(const uint4*)(x + row * ld + c * 8), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[e] += f[e];
+  }
+  float* dst = partial + (long)blockIdx.x * cols + c * 8;
+  *(float4*)dst = make_float4(s[0], s[1], s[2], s[3]);
+  *(float4*)(dst + 4) = make_float4(s[4], s[5], s[6], s[7]);
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restrict__ gu,
+                                                         bf16_t* __restrict__ s, long rows,
+                                                         int f) {
+  const int fc = f >> 3;
+  const long total = rows * fc;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long t = i / fc;
+    const int c = (int)(i - t * fc);
+    float a[8], b[8];
+    unpack8(*(const uint4*)(gu + t * 2 * f + c * 8), a);
+    unpack8(*(const uint4*)(gu + t * 2 * f + f + c * 8), b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[e] = a[e] / (1.0f + __expf(-a[e])) * b[e];
+    *(uint4*)(s + t * f + c * 8) = pack8(a);
+  }
+}
+
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restrict__ gu,
+                                                         const bf16_t* __restrict__ ds,
+                                                         bf16_t* __restrict__ dgu, long rows,
+                                                         int f) {
+  const int fc = f >> 3;
+  const long total = rows * fc;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long t = i / fc;
+    const int c = (int)(i - t * fc);
+    float a[8], b[8], d[8];
+    unpack8(*(const uint4*)(gu + t * 2 * f + c * 8), a);
+    unpack8(*(const uint4*)(gu + t * 2 * f + f + c * 8), b);
+    unpack8(*(const uint4*)(ds + t * f + c * 8), d);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sg = 1.0f / (1.0f + __expf(-a[e]));
+      const float da = d[e] * b[e] * sg * (1.0f + a[e] * (1.0f - sg));
+      const float db = d[e] * a[e] * sg;
+      a[e] = da;
+      b[e] = db;
+    }
+    *(uint4*)(dgu + t * 2 * f + c * 8) = pack8(a);
+    *(uint4*)(dgu + t * 2 * f + f + c * 8) = pack8(b);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// rotary embedding, half-split layout, in place
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rope_kernel(bf16_t* __restrict__ x, long ld,
+                                                   const float* __restrict__ cos_tab,
+                                                   const float* __restrict__ sin_tab, long rows,
+                                                   int seq, int heads, int d, int inverse) {
+  const int hc = d >> 4;  // 8-element chunks in half a head
+  const long total = rows * heads * hc;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const int c = (int)(i % hc);
+    const long th = i / hc;
+    const int hh = (int)(th % heads);
+    const long t = th / heads;
+    const int pos = (int)(t % seq);
+    bf16_t* p = x + t * ld + hh * d + c * 8;
+    float a[8], b[8];
+    unpack8(*(const uint4*)p, a);
+    unpack8(*(const uint4*)(p + d / 2), b);
+    const float* ct = cos_tab + (long)pos * (d / 2) + c * 8;
+    const float* st = sin_tab + (long)pos * (d / 2) + c * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float cs = ct[e], sn = inverse ? -st[e] : st[e];
+      const float o1 = a[e] * cs - b[e] * sn, o2 = b[e] * cs + a[e] * sn;
+      a[e] = o1;
+      b[e] = o2;
+    }
+    *(uint4*)p = pack8(a);
+    *(uint4*)(p + d / 2) = pack8(b);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gradient accumulation and casts
+// ---------------------------------------------------------------------------
+template <bool G_F32>
+__global__ __launch_bounds__(256) void grad_accum_kernel(float* __restrict__ acc,
+                                                         const void* __restrict__ g, long n8) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n8; i += (long)gridDim.x * 256) {
+    float4 a0 = ((float4*)acc)[2 * i], a1 = ((float4*)acc)[2 * i + 1];
+    if (G_F32) {
+      const float4 g0 = ((const float4*)g)[2 * i], g1 = ((const float4*)g)[2 * i + 1];
+      a0.x += g0.x; a0.y += g0.y; a0.z += g0.z; a0.w += g0.w;
+      a1.x += g1.x; a1.y += g1.y; a1.z += g1.z; a1.w += g1.w;
+    } else {
+      float f[8];
+      unpack8(((const uint4*)g)[i], f);
+      a0.x += f[0]; a0.y += f[1]; a0.z += f[2]; a0.w += f[3];
+      a1.x += f[4]; a1.y += f[5]; a1.z += f[6]; a1.w += f[7];
+    }
+    ((float4*)acc)[2 * i] = a0;
+    ((float4*)acc)[2 * i + 1] = a1;
+  }
+}
+
+template <bool G_F32>
+__global__ void grad_accum_tail_kernel(float* acc, const void* g, long start, long count) {
+  const long i = start + blockIdx.x * 256 + threadIdx.x;
+  if (i < count) acc[i] += G_F32 ? ((const float*)g)[i] : bf16_to_f32(((const bf16_t*)g)[i]);
+}
+
+__global__ __launch_bounds__(256) void cast_f32_bf16_kernel(const float* __restrict__ src,
+                                                            bf16_t* __restrict__ dst, long n) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+    dst[i] = f32_to_bf16(src[i]);
+}
+__global__ __launch_bounds__(256) void cast_bf16_f32_kernel(const bf16_t* __restrict__ src,
+                                                            float* __restrict__ dst, long n) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+    dst[i] = bf16_to_f32(src[i]);
+}
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* dst, uint32_t v, long n) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+    dst[i] = v;
+}
+
+int grid_for(long items, int per_block = 256, int cap = 256 * 32) {
+  long g = (items + per_block - 1) / per_block;
+  return (int)(g < 1 ? 1 : (g > cap ? cap : g));
+}
+
+template <bool LN>
+int launch_norm_fwd(hipStream_t st, const jpp_norm_args* a) {
+  const int blocks = (int)((a->rows + 3) / 4);
+  const int nch = (int)((a->cols / 8 + 63) / 64);
+#define JPP_NF(N)                                                                            \
+  hipLaunchKernelGGL((norm_fwd_kernel<LN, N>), dim3(blocks), dim3(256), 0, st,               \
+                     (const bf16_t*)a->x, (const bf16_t*)a->gamma, (const bf16_t*)a->beta,   \
+                     (bf16_t*)a->y, a->mean, a->rstd, (long)a->rows, (int)a->cols, a->eps)
+  if (nch <= 1) JPP_NF(1);
+  else if (nch <= 2) JPP_NF(2);
+  else if (nch <= 4) JPP_NF(4);
+  else if (nch <= 8) JPP_NF(8);
+  else JPP_NF(16);
+#undef JPP_NF
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+template <bool LN>
+int launch_norm_bwd(hipStream_t st, const jpp_norm_args* a) {
+  const int nch = (int)((a->cols / 8 + 63) / 64);
+  const int blocks = JPP_NORM_PARTIALS;
+#define JPP_NB(N)                                                                             \
+  hipLaunchKernelGGL((norm_bwd_kernel<LN, N>), dim3(blocks), dim3(256), 0, st,                \
+                     (const bf16_t*)a->dy, (const bf16_t*)a->x, a->mean, a->rstd,             \
+                     (const bf16_t*)a->gamma, (const bf16_t*)a->resid, (bf16_t*)a->dx,        \
+                     a->partial, (long)a->rows, (int)a->cols)
+  if (nch <= 1) JPP_NB(1);
+  else if (nch <= 2) JPP_NB(2);
+  else if (nch <= 4) JPP_NB(4);
+  else if (nch <= 8) JPP_NB(8);
+  else JPP_NB(16);
+#undef JPP_NB
+  JPP_LAUNCH_CHECK();
+  const int cb = (int)((a->cols + 255) / 256);
+  hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb), dim3(256), 0, st, a->partial, blocks,
+                     (int)a->cols, a->dgamma);
+  if (LN)
+    hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb), dim3(256), 0, st,
+                       a->partial + (long)blocks * a->cols, blocks, (int)a->cols, a->dbeta);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int jpp_norm_fwd(void* stream, const jpp_norm_args* a) {
+  JPP_REQUIRE(a && a->x && a->gamma && a->y && a->rstd, "norm_fwd: null operand");
+  JPP_REQUIRE(a->rows > 0 && a->cols > 0 && a->cols % 8 == 0 &&
+                  a->cols <= 8 * 64 * kMaxChunksPerLane,
+              "norm_fwd: cols must be a multiple of 8 and at most %d, got %ld",
+              8 * 64 * kMaxChunksPerLane, (long)a->cols);
+  JPP_REQUIRE((a->beta == nullptr) == (a->mean == nullptr),
+              "norm_fwd: beta and mean are both given (LayerNorm) or both NULL (RMSNorm)");
+  return a->beta ? launch_norm_fwd<true>((hipStream_t)stream, a)
+                 : launch_norm_fwd<false>((hipStream_t)stream, a);
+}
+
+int jpp_norm_bwd(void* stream, const jpp_norm_args* a) {
+  JPP_REQUIRE(a && a->x && a->gamma && a->dy && a->dx && a->rstd && a->dgamma && a->partial,
+              "norm_bwd: null operand");
+  JPP_REQUIRE(a->rows > 0 && a->cols > 0 && a->cols % 8 == 0 &&
+                  a->cols <= 8 * 64 * kMaxChunksPerLane,
+              "norm_bwd: cols must be a multiple of 8 and at most %d, got %ld",
+              8 * 64 * kMaxChunksPerLane, (long)a->cols);
+  const bool ln = a->mean != nullptr;
+  JPP_REQUIRE(!ln || a->dbeta, "norm_bwd: LayerNorm needs dbeta");
+  return ln ? launch_norm_bwd<true>((hipStream_t)stream, a)
+            : launch_norm_bwd<false>((hipStream_t)stream, a);
+}
+
+int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f) {
+  JPP_REQUIRE(gu && s && rows > 0 && f > 0 && f % 8 == 0, "swiglu_fwd: bad arguments");
+  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid_for(rows * (f / 8))), dim3(256), 0,
+                     (hipStream_t)stream, (const bf16_t*)gu, (bf16_t*)s, (long)rows, (int)f);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_swiglu_bwd(void* stream, const void* gu, const void* ds, void* dgu, int64_t rows,
+                   int64_t f) {
+  JPP_REQUIRE(gu && ds && dgu && rows > 0 && f > 0 && f % 8 == 0, "swiglu_bwd: bad arguments");
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid_for(rows * (f / 8))), dim3(256), 0,
+                     (hipStream_t)stream, (const bf16_t*)gu, (const bf16_t*)ds, (bf16_t*)dgu,
+                     (long)rows, (int)f);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_rope(void* stream, void* x, int64_t ld, const float* cos_tab, const float* sin_tab,
+             int batch, int seq, int n_rot_heads, int head_dim, int inverse) {
+  JPP_REQUIRE(x && cos_tab && sin_tab, "rope: null operand");
+  JPP_REQUIRE(batch > 0 && seq > 0 && n_rot_heads > 0 && head_dim % 16 == 0 && ld % 8 == 0 &&
+                  ld >= (int64_t)n_rot_heads * head_dim,
+              "rope: bad shape");
+  const long rows = (long)batch * seq;
+  hipLaunchKernelGGL(rope_kernel, dim3(grid_for(rows * n_rot_heads * (head_dim / 16))), dim3(256),
+                     0, (hipStream_t)stream, (bf16_t*)x, (long)ld, cos_tab, sin_tab, rows, seq,
+                     n_rot_heads, head_dim, inverse);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_grad_accum_f32(void* stream, float* acc, const void* g, int64_t count, int g_is_f32) {
+  JPP_REQUIRE(acc && g && count >= 0, "grad_accum: bad arguments");
+  JPP_REQUIRE((uintptr_t)acc % 16 == 0 && (uintptr_t)g % 16 == 0,
+              "grad_accum: operands must be 16-byte aligned");
+  if (count == 0) return JPP_OK;
+  const long n8 = count / 8;
+  hipStream_t st = (hipStream_t)stream;
+  if (n8) {
+    if (g_is_f32)
+      hipLaunchKernelGGL(grad_accum_kernel<true>, dim3(grid_for(n8)), dim3(256), 0, st, acc, g, n8);
+    else
+      hipLaunchKernelGGL(grad_accum_kernel<false>, dim3(grid_for(n8)), dim3(256), 0, st, acc, g, n8);
+  }
+  if (count % 8) {
+    if (g_is_f32)
+      hipLaunchKernelGGL(grad_accum_tail_kernel<true>, dim3(1), dim3(256), 0, st, acc, g, n8 * 8,
+                         (long)count);
+    else
+      hipLaunchKernelGGL(grad_accum_tail_kernel<false>, dim3(1), dim3(256), 0, st, acc, g, n8 * 8,
+                         (long)count);
+  }
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int64_t cols,
+                     float* acc, float* partial) {
+  JPP_REQUIRE(x && acc && partial && rows > 0 && cols > 0 && cols % 8 == 0 && ld % 8 == 0 &&
+                  ld >= cols,
+              "colsum: bad arguments");
+  hipStream_t st = (hipStream_t)stream;
+  const int nb = (int)(rows < JPP_NORM_PARTIALS ? rows : JPP_NORM_PARTIALS);
+  const int panels = (int)((cols / 8 + 255) / 256);
+  hipLaunchKernelGGL(colsum_partial_kernel, dim3(nb, panels), dim3(256), 0, st, (const bf16_t*)x,
+                     (long)ld, (long)rows, (int)cols, partial);
+  hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 255) / 256)), dim3(256), 0, st,
+                     partial, nb, (int)cols, acc);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count) {
+  JPP_REQUIRE(src && dst && count > 0, "cast: bad arguments");
+  hipLaunchKernelGGL(cast_f32_bf16_kernel, dim3(grid_for(count)), dim3(256), 0,
+                     (hipStream_t)stream, src, (bf16_t*)dst, (long)count);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count) {
+  JPP_REQUIRE(src && dst && count > 0, "cast: bad arguments");
+  hipLaunchKernelGGL(cast_bf16_f32_kernel, dim3(grid_for(count)), dim3(256), 0,
+                     (hipStream_t)stream, (const bf16_t*)src, dst, (long)count);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_fill_u32(void* dst, uint32_t value, size_t count, void* stream) {
+  JPP_REQUIRE(dst || count == 0, "fill: null destination");
+  if (count == 0) return JPP_OK;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for((long)count)), dim3(256), 0,
+                     (hipStream_t)stream, (uint32_t*)dst, value, (long)count);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,275 @@
+// bf16 GEMM on gfx950 matrix cores (v_mfma_f32_32x32x16_bf16), LDS
+// double-buffered, with the epilogues a pipeline stage needs.
+//
+//   C[m,n] = epilogue( sum_k Aop[m,k] * Bop[n,k] )
+//
+// A workgroup of 256 threads (4 waves, 2 x 2) owns a BM x BN output tile and
+// walks K in steps of 64.  Both operands live in LDS as swizzled [rows][64]
+// slabs with the contraction index contiguous, whatever their layout in HBM:
+// an operand whose contraction index is the slow one in memory (the weights
+// in a forward GEMM, both operands of a weight-gradient GEMM) is transposed in
+// registers on its way into LDS (TileLoader<.., TRANS=true>).  The next K-step
+// is fetched from HBM into registers while the current one is multiplied.
+//
+// The weight operand is fed to the MFMA "A" port and the activation operand to
+// the "B" port, so a lane ends up holding 4 consecutive n for one m and the
+// epilogue writes 8-byte (bf16) or 16-byte (f32) runs.
+#include <math.h>
+
+#include "common.h"
+
+namespace {
+
+struct GemmParams {
+  const bf16_t* a;
+  const bf16_t* b;
+  void* c;
+  void* c2;
+  const bf16_t* bias;
+  const bf16_t* resid;
+  const bf16_t* aux;
+  int m, n, k;
+  long lda, ldb, ldc, ldc2, ldresid, ldaux;
+  int gelu_tanh;
+  int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ float gelu_f(float u, int tanh_form) {
+  if (tanh_form) {
+    float t = tanhf(0.7978845608028654f * (u + 0.044715f * u * u * u));
+    return 0.5f * u * (1.0f + t);
+  }
+  return 0.5f * u * (1.0f + erff(u * 0.7071067811865476f));
+}
+
+__device__ __forceinline__ float gelu_grad_f(float u, int tanh_form) {
+  if (tanh_form) {
+    float t = tanhf(0.7978845608028654f * (u + 0.044715f * u * u * u));
+    return 0.5f * (1.0f + t) +
+           0.5f * u * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * u * u);
+  }
+  return 0.5f * (1.0f + erff(u * 0.7071067811865476f)) +
+         u * __expf(-0.5f * u * u) * 0.3989422804014327f;
+}
+
+// Output tile of a workgroup.  Consecutive workgroup ids land on different
+// XCDs (8 of them, each with its own L2); give every XCD a contiguous range of
+// tiles, and inside a range walk GROUP tile-rows at a time so the B panels in
+// flight stay L2 resident.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int nwg = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  if ((nwg & 7) == 0) pid = (pid & 7) * (nwg >> 3) + (pid >> 3);
+  constexpr int GROUP = 8;
+  const int width = GROUP * tiles_n;
+  const int group = pid / width;
+  const int first = group * GROUP;
+  const int gsize = min(tiles_m - first, GROUP);
+  tm = first + (pid % width) % gsize;
+  tn = (pid % width) / gsize;
+}
+
+template <int BM, int BN, bool TA, bool TB, int EPI>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 MFMA tiles per wave
+  extern __shared__ __align__(16) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_of_block(p.tiles_m, p.tiles_n, tm, tn);
+  const long m0 = (long)tm * BM, n0 = (long)tn * BN;
+
+  const bf16_t* a_src = TA ? p.a + m0 : p.a + m0 * p.lda;
+  const bf16_t* b_src = TB ? p.b + n0 : p.b + n0 * p.ldb;
+  const long a_step = TA ? 64 * p.lda : 64;
+  const long b_step = TB ? 64 * p.ldb : 64;
+
+  using LA = TileLoader<BM, TA>;
+  using LB = TileLoader<BN, TB>;
+  typename LA::Regs ra;
+  typename LB::Regs rb;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int kt_n = p.k / 64;
+  LA::load(ra, a_src, p.lda, tid);
+  LB::load(rb, b_src, p.ldb, tid);
+  LA::store(ra, smem, tid);
+  LB::store(rb, smem + A_BYTES, tid);
+  __syncthreads();
+
+  for (int kt = 0; kt < kt_n; ++kt) {
+    const uint8_t* sa = smem + (kt & 1) * STAGE;
+    const uint8_t* sb = sa + A_BYTES;
+    // fetch the next K-step (the last iteration re-reads its own, unused)
+    const int kn = min(kt + 1, kt_n - 1);
+    LA::load(ra, a_src + (long)kn * a_step, p.lda, tid);
+    LB::load(rb, b_src + (long)kn * b_step, p.ldb, tid);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      bf16x8 fw[TN], fx[TM];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fw[j] = slab_frag(sb, wn * (BN / 2) + j * 32, ks, lane);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fx[i] = slab_frag(sa, wm * (BM / 2) + i * 32, ks, lane);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fx[i], acc[i][j], 0, 0, 0);
+    }
+    uint8_t* da = smem + ((kt + 1) & 1) * STAGE;
+    LA::store(ra, da, tid);
+    LB::store(rb, da + A_BYTES, tid);
+    __syncthreads();
+  }
+
+  // epilogue: lane holds m = base_m + (lane & 31), and for g = 0..3 the four
+  // columns base_n + 8 g + 4 (lane >> 5) + {0,1,2,3}
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const long m = m0 + wm * (BM / 2) + i * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const long n = n0 + wn * (BN / 2) + j * 32 + g * 8 + (lane >> 5) * 4;
+        float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
+        float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
+        if constexpr (EPI == JPP_EPI_ACC_F32) {
+          float4* dst = (float4*)((float*)p.c + m * p.ldc + n);
+          float4 o = *dst;
+          o.x += v0; o.y += v1; o.z += v2; o.w += v3;
+          *dst = o;
+        } else if constexpr (EPI == JPP_EPI_F32) {
+          *(float4*)((float*)p.c + m * p.ldc + n) = make_float4(v0, v1, v2, v3);
+        } else {
+          if (p.bias) {
+            const uint2 bb = *(const uint2*)(p.bias + n);
+            v0 += bf16lo_to_f32(bb.x); v1 += bf16hi_to_f32(bb.x);
+            v2 += bf16lo_to_f32(bb.y); v3 += bf16hi_to_f32(bb.y);
+          }
+          if constexpr (EPI == JPP_EPI_BF16) {
+            if (p.resid) {
+              const uint2 rr = *(const uint2*)(p.resid + m * p.ldresid + n);
+              v0 += bf16lo_to_f32(rr.x); v1 += bf16hi_to_f32(rr.x);
+              v2 += bf16lo_to_f32(rr.y); v3 += bf16hi_to_f32(rr.y);
+            }
+          } else if constexpr (EPI == JPP_EPI_GELU) {
+            *(uint2*)((bf16_t*)p.c2 + m * p.ldc2 + n) =
+                make_uint2(pack_bf16x2(gelu_f(v0, p.gelu_tanh), gelu_f(v1, p.gelu_tanh)),
+                           pack_bf16x2(gelu_f(v2, p.gelu_tanh), gelu_f(v3, p.gelu_tanh)));
+          } else if constexpr (EPI == JPP_EPI_DGELU) {
+            const uint2 uu = *(const uint2*)(p.aux + m * p.ldaux + n);
+            v0 *= gelu_grad_f(bf16lo_to_f32(uu.x), p.gelu_tanh);
+            v1 *= gelu_grad_f(bf16hi_to_f32(uu.x), p.gelu_tanh);
+            v2 *= gelu_grad_f(bf16lo_to_f32(uu.y), p.gelu_tanh);
+            v3 *= gelu_grad_f(bf16hi_to_f32(uu.y), p.gelu_tanh);
+          }
+          *(uint2*)((bf16_t*)p.c + m * p.ldc + n) =
+              make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, bool TA, bool TB, int EPI>
+int launch(hipStream_t stream, GemmParams& p) {
+  constexpr int SMEM = 2 * (BM + BN) * 128;
+  auto kern = gemm_kernel<BM, BN, TA, TB, EPI>;
+  static bool configured = false;  // per instantiation; attribute is sticky
+  if (!configured) {
+    JPP_CHECK_HIP(hipFuncSetAttribute((const void*)kern,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, SMEM));
+    configured = true;
+  }
+  p.tiles_m = p.m / BM;
+  p.tiles_n = p.n / BN;
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), SMEM, stream, p);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+template <bool TA, bool TB, int EPI>
+int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
+  switch (tile) {
+    case 1: return launch<128, 128, TA, TB, EPI>(stream, p);
+    case 2: return launch<256, 128, TA, TB, EPI>(stream, p);
+    default: return launch<256, 256, TA, TB, EPI>(stream, p);
+  }
+}
+
+// Largest tile that still gives every CU work: 256 CUs, one 256x256 or two
+// 128x128 workgroups resident per CU.
+int choose_tile(long m, long n) {
+  const long t256 = (m % 256 == 0 && n % 256 == 0) ? (m / 256) * (n / 256) : 0;
+  const long t2 = (m % 256 == 0) ? (m / 256) * (n / 128) : 0;
+  if (t256 >= 256) return 3;
+  if (t2 >= 256) return 2;
+  return 1;
+}
+
+}  // namespace
+
+extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
+  hipStream_t stream = (hipStream_t)stream_;
+  JPP_REQUIRE(a && a->a && a->b && a->c, "gemm: null operand");
+  JPP_REQUIRE(a->m > 0 && a->n > 0 && a->k > 0, "gemm: empty problem %ldx%ldx%ld", (long)a->m,
+              (long)a->n, (long)a->k);
+  JPP_REQUIRE(a->m % 128 == 0 && a->n % 128 == 0 && a->k % 64 == 0,
+              "gemm: M,N must be multiples of 128 and K of 64, got %ldx%ldx%ld", (long)a->m,
+              (long)a->n, (long)a->k);
+  JPP_REQUIRE(a->lda >= (a->trans_a ? a->m : a->k) && a->ldb >= (a->trans_b ? a->n : a->k) &&
+                  a->ldc >= a->n,
+              "gemm: leading dimension too small");
+  JPP_REQUIRE(a->lda % 8 == 0 && a->ldb % 8 == 0 && a->ldc % 4 == 0,
+              "gemm: leading dimensions must keep 16-byte alignment");
+  JPP_REQUIRE(((uintptr_t)a->a | (uintptr_t)a->b | (uintptr_t)a->c) % 16 == 0,
+              "gemm: operands must be 16-byte aligned");
+  JPP_REQUIRE(a->m < (1L << 31) && a->n < (1L << 31) && a->k < (1L << 31), "gemm: too large");
+  GemmParams p;
+  p.a = (const bf16_t*)a->a;
+  p.b = (const bf16_t*)a->b;
+  p.c = a->c;
+  p.c2 = a->c2;
+  p.bias = (const bf16_t*)a->bias;
+  p.resid = (const bf16_t*)a->resid;
+  p.aux = (const bf16_t*)a->aux;
+  p.m = (int)a->m; p.n = (int)a->n; p.k = (int)a->k;
+  p.lda = a->lda; p.ldb = a->ldb; p.ldc = a->ldc;
+  p.ldc2 = a->ldc2; p.ldresid = a->ldresid; p.ldaux = a->ldaux;
+  p.gelu_tanh = a->gelu_tanh;
+  if (a->epilogue == JPP_EPI_GELU)
+    JPP_REQUIRE(a->c2 && a->ldc2 >= a->n && a->ldc2 % 4 == 0, "gemm: GELU epilogue needs c2");
+  if (a->epilogue == JPP_EPI_DGELU)
+    JPP_REQUIRE(a->aux && a->ldaux >= a->n && a->ldaux % 4 == 0, "gemm: dGELU epilogue needs aux");
+  if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
+  int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
+  if (tile >= 2 && a->m % 256) tile = 1;
+  if (tile == 3 && a->n % 256) tile = 2;
+  JPP_REQUIRE(tile >= 1 && tile <= 3, "gemm: unknown tile %d", tile);
+
+  const int ta = a->trans_a != 0, tb = a->trans_b != 0, e = a->epilogue;
+#define JPP_GEMM_CASE(TA_, TB_, E_) \
+  if (ta == TA_ && tb == TB_ && e == E_) return launch_tiled<TA_, TB_, E_>(stream, p, tile)
+  JPP_GEMM_CASE(0, 1, JPP_EPI_BF16);     // forward
+  JPP_GEMM_CASE(0, 1, JPP_EPI_GELU);     // forward + GELU
+  JPP_GEMM_CASE(0, 1, JPP_EPI_F32);      // forward, f32 out (router logits)
+  JPP_GEMM_CASE(0, 0, JPP_EPI_BF16);     // input gradient
+  JPP_GEMM_CASE(0, 0, JPP_EPI_DGELU);    // input gradient through GELU
+  JPP_GEMM_CASE(1, 1, JPP_EPI_ACC_F32);  // weight gradient, accumulated
+  JPP_GEMM_CASE(1, 1, JPP_EPI_BF16);     // weight gradient, bf16
+  JPP_GEMM_CASE(1, 1, JPP_EPI_F32);      // weight gradient, f32
+#undef JPP_GEMM_CASE
+  return jpp_set_error(JPP_ERR_INVALID, "gemm: unsupported combination trans_a=%d trans_b=%d epilogue=%d",
+                       ta, tb, e);
+}

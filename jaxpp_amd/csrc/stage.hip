@@ -1,0 +1,607 @@
+// Stage executor: runs the FWD / BWD / BWD_I / BWD_W tasks of one pipeline
+// rank on one GPU, in whatever order the schedule's table dictates.
+//
+// Plays the part of `task_impl` in the reference
+// (src/jaxpp/jax_primitives.py:776-859) for the stages one rank owns:
+//   * a forward task runs the stage's layers and leaves a residual set
+//     ("stash") in a slot of a fixed ring; the slot is released by the task
+//     that last reads it - BWD, or BWD_W when the backward is split - which is
+//     the lifetime the reference derives with `infer_donation` / `add_deletes`
+//     (src/jaxpp/core.py:1732-1890);
+//   * with a split backward, BWD_I runs the input-gradient chain plus the
+//     small non-matmul parameter gradients (bias column sums, norm scale /
+//     shift), and BWD_W runs the weight-gradient GEMMs, exactly the partition
+//     `partition_eqns(memory_scarce=True)` makes (src/jaxpp/jaxpr_utils.py:105-169);
+//   * gradients are accumulated in fp32 in place: the loop carry of `treduce`
+//     with `Add` (src/jaxpp/training.py:112-123).
+#include <math.h>
+#include <string.h>
+
+#include <algorithm>
+#include <map>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+struct ParamInfo {
+  const char* name;
+  int64_t rows, cols;
+};
+
+struct Buf {  // a carved piece of a slot / scratch allocation
+  size_t off = 0, bytes = 0;
+};
+
+struct Carver {
+  size_t total = 0;
+  Buf take(size_t bytes) {
+    Buf b;
+    b.off = total;
+    b.bytes = bytes;
+    total += (bytes + 255) & ~(size_t)255;
+    return b;
+  }
+};
+
+// Residuals of one layer for one microbatch (offsets into a slot).
+struct LayerStash {
+  // common
+  Buf x, qkv, ctx, lse;
+  // bert
+  Buf a, mean1, rstd1, x1, u, g, c, mean2, rstd2;
+  // llama
+  Buf n1, h1, n2, gu, s;
+  // cotangents kept for the weight-gradient task
+  Buf dc, du, da, dqkv;   // bert (dqkv shared with llama)
+  Buf dyin, dgu, dh1;     // llama
+};
+
+}  // namespace
+
+struct jpp_stage {
+  jpp_stage_desc d;
+  int64_t T, h, f, qkvw, ctxw, hd;
+  std::vector<ParamInfo> pinfo;
+  std::vector<size_t> poff;        // element offset of parameter i inside a layer block
+  size_t layer_elems = 0;
+  bf16_t* params = nullptr;        // [chunk][layer][layer_elems] bf16
+  float* grads = nullptr;          // same shape, f32
+  std::vector<LayerStash> lay;     // per layer of a chunk, offsets into a slot
+  size_t slot_bytes = 0;
+  std::vector<uint8_t*> slots;
+  std::vector<int> free_slots;
+  std::map<std::pair<int, int>, int> live;  // (chunk, mubatch) -> slot
+  std::map<std::pair<int, int>, int> phase; // 1: forward done, 2: BWD_I done
+  // scratch shared by all tasks (stream ordered)
+  uint8_t* scratch = nullptr;
+  size_t scratch_bytes = 0;
+  LayerStash wshared;              // cotangent buffers when the backward is not split
+  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_delta, s_wg, s_cos, s_sin;
+  size_t total_bytes = 0;
+
+  bf16_t* P(int chunk, int layer, int i) {
+    return params + ((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i];
+  }
+  float* G(int chunk, int layer, int i) {
+    return grads + ((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i];
+  }
+  template <class T_ = void>
+  T_* S(const Buf& b) { return (T_*)(scratch + b.off); }
+};
+
+namespace {
+
+enum BertP { B_Wqkv, B_bqkv, B_Wo, B_bo, B_ln1g, B_ln1b, B_W1, B_b1, B_W2, B_b2, B_ln2g, B_ln2b };
+enum LlamaP { L_rms1, L_Wqkv, L_Wo, L_rms2, L_Wgu, L_Wd };
+
+int gemm(hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int64_t ldb, int tb,
+         void* c, int64_t ldc, int64_t m, int64_t n, int64_t k, int epi, const void* bias = nullptr,
+         const void* resid = nullptr, int64_t ldr = 0, const void* aux = nullptr,
+         int64_t ldaux = 0, void* c2 = nullptr, int64_t ldc2 = 0, int gelu_tanh = 0) {
+  jpp_gemm_args g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.c = c; g.c2 = c2; g.bias = bias; g.resid = resid; g.aux = aux;
+  g.m = m; g.n = n; g.k = k;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldc2 = ldc2; g.ldresid = ldr; g.ldaux = ldaux;
+  g.trans_a = ta; g.trans_b = tb; g.epilogue = epi; g.gelu_tanh = gelu_tanh;
+  return jpp_gemm_bf16(st, &g);
+}
+
+#define RC(expr)            \
+  do {                      \
+    int rc_ = (expr);       \
+    if (rc_) return rc_;    \
+  } while (0)
+
+// dW[rows, cols] (+)= X^T dY, X: [T, rows], dY: [T, cols]
+int wgrad(jpp_stage* s, hipStream_t st, const void* x, int64_t ldx, const void* dy, int64_t lddy,
+          float* acc, int64_t rows, int64_t cols) {
+  if (s->d.fused_wgrad_accum)
+    return gemm(st, x, ldx, 1, dy, lddy, 1, acc, cols, rows, cols, s->T, JPP_EPI_ACC_F32);
+  void* g = s->S<>(s->s_wg);
+  RC(gemm(st, x, ldx, 1, dy, lddy, 1, g, cols, rows, cols, s->T, JPP_EPI_BF16));
+  return jpp_grad_accum_f32(st, acc, g, rows * cols, 0);
+}
+
+int norm_f(jpp_stage* s, hipStream_t st, const void* x, const void* gamma, const void* beta,
+           void* y, float* mean, float* rstd) {
+  jpp_norm_args a;
+  memset(&a, 0, sizeof(a));
+  a.x = x; a.gamma = gamma; a.beta = beta; a.y = y; a.mean = mean; a.rstd = rstd;
+  a.rows = s->T; a.cols = s->h; a.eps = s->d.eps;
+  return jpp_norm_fwd(st, &a);
+}
+
+int norm_b(jpp_stage* s, hipStream_t st, const void* dy, const void* x, const float* mean,
+           const float* rstd, const void* gamma, const void* resid, void* dx, float* dgamma,
+           float* dbeta) {
+  jpp_norm_args a;
+  memset(&a, 0, sizeof(a));
+  a.dy = dy; a.x = x; a.mean = (float*)mean; a.rstd = (float*)rstd; a.gamma = gamma;
+  a.resid = resid; a.dx = dx; a.dgamma = dgamma; a.dbeta = dbeta;
+  a.partial = s->S<float>(s->s_partial);
+  a.rows = s->T; a.cols = s->h; a.eps = s->d.eps;
+  return jpp_norm_bwd(st, &a);
+}
+
+void attn_args(jpp_stage* s, jpp_attn_args& a, uint8_t* slot, const LayerStash& L) {
+  memset(&a, 0, sizeof(a));
+  bf16_t* qkv = (bf16_t*)(slot + L.qkv.off);
+  a.q = qkv;
+  a.k = qkv + (int64_t)s->d.n_heads * s->hd;
+  a.v = qkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd;
+  a.ldq = a.ldk = a.ldv = s->qkvw;
+  a.o = slot + L.ctx.off;
+  a.ldo = s->ctxw;
+  a.lse = (float*)(slot + L.lse.off);
+  a.batch = s->d.batch; a.seq = s->d.seq; a.n_heads = s->d.n_heads;
+  a.n_kv_heads = s->d.n_kv_heads; a.head_dim = (int)s->hd; a.causal = s->d.causal;
+}
+
+// ---- one layer, forward ----------------------------------------------------
+int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, void* y) {
+  const LayerStash& L = s->lay[li];
+  const int64_t T = s->T, h = s->h, f = s->f;
+  auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
+  jpp_attn_args aa;
+  if (s->d.family == JPP_FAMILY_BERT) {
+    RC(gemm(st, at(L.x), h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 1, at(L.qkv), 3 * h, T, 3 * h, h,
+            JPP_EPI_BF16, s->P(chunk, li, B_bqkv)));
+    attn_args(s, aa, slot, L);
+    RC(jpp_attn_fwd(st, &aa));
+    RC(gemm(st, at(L.ctx), h, 0, s->P(chunk, li, B_Wo), h, 1, at(L.a), h, T, h, h, JPP_EPI_BF16,
+            s->P(chunk, li, B_bo), at(L.x), h));
+    RC(norm_f(s, st, at(L.a), s->P(chunk, li, B_ln1g), s->P(chunk, li, B_ln1b), at(L.x1),
+              (float*)at(L.mean1), (float*)at(L.rstd1)));
+    RC(gemm(st, at(L.x1), h, 0, s->P(chunk, li, B_W1), f, 1, at(L.u), f, T, f, h, JPP_EPI_GELU,
+            s->P(chunk, li, B_b1), nullptr, 0, nullptr, 0, at(L.g), f, s->d.gelu_tanh));
+    RC(gemm(st, at(L.g), f, 0, s->P(chunk, li, B_W2), h, 1, at(L.c), h, T, h, f, JPP_EPI_BF16,
+            s->P(chunk, li, B_b2), at(L.x1), h));
+    RC(norm_f(s, st, at(L.c), s->P(chunk, li, B_ln2g), s->P(chunk, li, B_ln2b), y,
+              (float*)at(L.mean2), (float*)at(L.rstd2)));
+    return JPP_OK;
+  }
+  // llama
+  RC(norm_f(s, st, at(L.x), s->P(chunk, li, L_rms1), nullptr, at(L.n1), nullptr,
+            (float*)at(L.rstd1)));
+  RC(gemm(st, at(L.n1), h, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 1, at(L.qkv), s->qkvw, T, s->qkvw,
+          h, JPP_EPI_BF16));
+  RC(jpp_rope(st, at(L.qkv), s->qkvw, s->S<float>(s->s_cos), s->S<float>(s->s_sin), s->d.batch,
+              s->d.seq, s->d.n_heads + s->d.n_kv_heads, (int)s->hd, 0));
+  attn_args(s, aa, slot, L);
+  RC(jpp_attn_fwd(st, &aa));
+  RC(gemm(st, at(L.ctx), s->ctxw, 0, s->P(chunk, li, L_Wo), h, 1, at(L.h1), h, T, h, s->ctxw,
+          JPP_EPI_BF16, nullptr, at(L.x), h));
+  RC(norm_f(s, st, at(L.h1), s->P(chunk, li, L_rms2), nullptr, at(L.n2), nullptr,
+            (float*)at(L.rstd2)));
+  RC(gemm(st, at(L.n2), h, 0, s->P(chunk, li, L_Wgu), 2 * f, 1, at(L.gu), 2 * f, T, 2 * f, h,
+          JPP_EPI_BF16));
+  RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), T, f));
+  RC(gemm(st, at(L.s), f, 0, s->P(chunk, li, L_Wd), h, 1, y, h, T, h, f, JPP_EPI_BF16, nullptr,
+          at(L.h1), h));
+  return JPP_OK;
+}
+
+// ---- one layer, input-gradient half -------------------------------------------
+// `w` holds the cotangents the weight-gradient half will read: the slot itself
+// when the backward is split, the shared scratch set otherwise.
+int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, uint8_t* wbase,
+                const LayerStash& W, const void* dy, void* dx) {
+  const LayerStash& L = s->lay[li];
+  const int64_t T = s->T, h = s->h, f = s->f;
+  auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
+  auto wt = [&](const Buf& b) { return (void*)(wbase + b.off); };
+  float* partial = s->S<float>(s->s_partial);
+  jpp_attn_args aa;
+  if (s->d.family == JPP_FAMILY_BERT) {
+    void* dx1 = s->S<>(s->s_t1);
+    void* dctx = s->S<>(s->s_t2);
+    RC(norm_b(s, st, dy, at(L.c), (float*)at(L.mean2), (float*)at(L.rstd2),
+              s->P(chunk, li, B_ln2g), nullptr, wt(W.dc), s->G(chunk, li, B_ln2g),
+              s->G(chunk, li, B_ln2b)));
+    RC(gemm(st, wt(W.dc), h, 0, s->P(chunk, li, B_W2), h, 0, wt(W.du), f, T, f, h, JPP_EPI_DGELU,
+            nullptr, nullptr, 0, at(L.u), f, nullptr, 0, s->d.gelu_tanh));
+    RC(gemm(st, wt(W.du), f, 0, s->P(chunk, li, B_W1), f, 0, dx1, h, T, h, f, JPP_EPI_BF16, nullptr,
+            wt(W.dc), h));
+    RC(norm_b(s, st, dx1, at(L.a), (float*)at(L.mean1), (float*)at(L.rstd1),
+              s->P(chunk, li, B_ln1g), nullptr, wt(W.da), s->G(chunk, li, B_ln1g),
+              s->G(chunk, li, B_ln1b)));
+    RC(gemm(st, wt(W.da), h, 0, s->P(chunk, li, B_Wo), h, 0, dctx, h, T, h, h, JPP_EPI_BF16));
+    attn_args(s, aa, slot, L);
+    bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
+    aa.d_o = dctx; aa.lddo = h;
+    aa.dq = dqkv; aa.dk = dqkv + h; aa.dv = dqkv + 2 * h;
+    aa.lddq = aa.lddk = aa.lddv = 3 * h;
+    aa.delta = s->S<float>(s->s_delta);
+    RC(jpp_attn_bwd(st, &aa));
+    RC(gemm(st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dx, h, T, h, 3 * h,
+            JPP_EPI_BF16, nullptr, wt(W.da), h));
+    RC(jpp_colsum_accum(st, wt(W.dc), h, T, h, s->G(chunk, li, B_b2), partial));
+    RC(jpp_colsum_accum(st, wt(W.du), f, T, f, s->G(chunk, li, B_b1), partial));
+    RC(jpp_colsum_accum(st, wt(W.da), h, T, h, s->G(chunk, li, B_bo), partial));
+    RC(jpp_colsum_accum(st, dqkv, 3 * h, T, 3 * h, s->G(chunk, li, B_bqkv), partial));
+    return JPP_OK;
+  }
+  // llama
+  void* ds = s->S<>(s->s_t1);
+  void* dn = s->S<>(s->s_t2);   // dn2, later dn1
+  void* dctx = s->S<>(s->s_t3);
+  RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, ds, f, T, f, h, JPP_EPI_BF16));
+  RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), T, f));
+  RC(gemm(st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
+          JPP_EPI_BF16));
+  RC(norm_b(s, st, dn, at(L.h1), nullptr, (float*)at(L.rstd2), s->P(chunk, li, L_rms2), dy,
+            wt(W.dh1), s->G(chunk, li, L_rms2), nullptr));
+  RC(gemm(st, wt(W.dh1), h, 0, s->P(chunk, li, L_Wo), h, 0, dctx, s->ctxw, T, s->ctxw, h,
+          JPP_EPI_BF16));
+  attn_args(s, aa, slot, L);
+  bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
+  aa.d_o = dctx; aa.lddo = s->ctxw;
+  aa.dq = dqkv;
+  aa.dk = dqkv + (int64_t)s->d.n_heads * s->hd;
+  aa.dv = dqkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd;
+  aa.lddq = aa.lddk = aa.lddv = s->qkvw;
+  aa.delta = s->S<float>(s->s_delta);
+  RC(jpp_attn_bwd(st, &aa));
+  RC(jpp_rope(st, dqkv, s->qkvw, s->S<float>(s->s_cos), s->S<float>(s->s_sin), s->d.batch,
+              s->d.seq, s->d.n_heads + s->d.n_kv_heads, (int)s->hd, 1));
+  RC(gemm(st, dqkv, s->qkvw, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 0, dn, h, T, h, s->qkvw,
+          JPP_EPI_BF16));
+  RC(norm_b(s, st, dn, at(L.x), nullptr, (float*)at(L.rstd1), s->P(chunk, li, L_rms1), wt(W.dh1),
+            dx, s->G(chunk, li, L_rms1), nullptr));
+  return JPP_OK;
+}
+
+// ---- one layer, weight-gradient half --------------------------------------------
+int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, uint8_t* wbase,
+                const LayerStash& W, const void* dy) {
+  const LayerStash& L = s->lay[li];
+  const int64_t h = s->h, f = s->f;
+  auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
+  auto wt = [&](const Buf& b) { return (void*)(wbase + b.off); };
+  if (s->d.family == JPP_FAMILY_BERT) {
+    RC(wgrad(s, st, at(L.g), f, wt(W.dc), h, s->G(chunk, li, B_W2), f, h));
+    RC(wgrad(s, st, at(L.x1), h, wt(W.du), f, s->G(chunk, li, B_W1), h, f));
+    RC(wgrad(s, st, at(L.ctx), h, wt(W.da), h, s->G(chunk, li, B_Wo), h, h));
+    RC(wgrad(s, st, at(L.x), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
+    return JPP_OK;
+  }
+  RC(wgrad(s, st, at(L.s), f, dy, h, s->G(chunk, li, L_Wd), f, h));
+  RC(wgrad(s, st, at(L.n2), h, wt(W.dgu), 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f));
+  RC(wgrad(s, st, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, L_Wo), s->ctxw, h));
+  RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, L_Wqkv), h, s->qkvw));
+  return JPP_OK;
+}
+
+void carve_layer(jpp_stage* s, Carver& c, LayerStash& L, bool with_w) {
+  const size_t T = s->T, h = s->h, f = s->f, e = 2;
+  const size_t stat = (size_t)s->d.batch * s->d.n_heads * s->d.seq * 4;
+  L.x = c.take(T * h * e);
+  L.qkv = c.take(T * s->qkvw * e);
+  L.ctx = c.take(T * s->ctxw * e);
+  L.lse = c.take(stat);
+  if (s->d.family == JPP_FAMILY_BERT) {
+    L.a = c.take(T * h * e);
+    L.mean1 = c.take(T * 4); L.rstd1 = c.take(T * 4);
+    L.x1 = c.take(T * h * e);
+    L.u = c.take(T * f * e);
+    L.g = c.take(T * f * e);
+    L.c = c.take(T * h * e);
+    L.mean2 = c.take(T * 4); L.rstd2 = c.take(T * 4);
+  } else {
+    L.rstd1 = c.take(T * 4); L.rstd2 = c.take(T * 4);
+    L.n1 = c.take(T * h * e);
+    L.h1 = c.take(T * h * e);
+    L.n2 = c.take(T * h * e);
+    L.gu = c.take(T * 2 * f * e);
+    L.s = c.take(T * f * e);
+  }
+  if (with_w) {
+    // carved by the caller through carve_w
+  }
+}
+
+void carve_w(jpp_stage* s, Carver& c, LayerStash& L) {
+  const size_t T = s->T, h = s->h, f = s->f, e = 2;
+  L.dqkv = c.take(T * s->qkvw * e);
+  if (s->d.family == JPP_FAMILY_BERT) {
+    L.dc = c.take(T * h * e);
+    L.du = c.take(T * f * e);
+    L.da = c.take(T * h * e);
+  } else {
+    L.dyin = c.take(T * h * e);
+    L.dgu = c.take(T * 2 * f * e);
+    L.dh1 = c.take(T * h * e);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
+  JPP_REQUIRE(d && out, "stage_create: null");
+  *out = nullptr;
+  JPP_REQUIRE(d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_LLAMA,
+              "stage_create: family %d is not built", d->family);
+  JPP_REQUIRE(d->hidden > 0 && d->n_heads > 0 && d->ffn > 0 && d->seq > 0 && d->batch > 0,
+              "stage_create: bad shape");
+  JPP_REQUIRE(d->n_chunks > 0 && d->layers_per_chunk > 0 && d->max_live > 0,
+              "stage_create: n_chunks, layers_per_chunk and max_live must be positive");
+  const int kvh = d->n_kv_heads > 0 ? d->n_kv_heads : d->n_heads;
+  const int hd = d->head_dim > 0 ? d->head_dim : d->hidden / d->n_heads;
+  JPP_REQUIRE(hd == 64 || hd == 128, "stage_create: head_dim must be 64 or 128, got %d", hd);
+  JPP_REQUIRE(d->n_heads % kvh == 0, "stage_create: n_heads %% n_kv_heads != 0");
+  const int64_t T = (int64_t)d->batch * d->seq;
+  JPP_REQUIRE(T % 128 == 0 && d->seq % 128 == 0, "stage_create: seq must be a multiple of 128");
+  JPP_REQUIRE(d->hidden % 128 == 0 && d->ffn % 128 == 0 && ((d->n_heads + 2 * kvh) * hd) % 128 == 0,
+              "stage_create: hidden, ffn and qkv width must be multiples of 128");
+  JPP_REQUIRE(d->hidden <= 8192, "stage_create: hidden > 8192 not supported by the norm kernels");
+  if (d->family == JPP_FAMILY_BERT)
+    JPP_REQUIRE(kvh == d->n_heads && d->n_heads * hd == d->hidden && !d->causal,
+                "stage_create: the BERT layer needs n_heads*head_dim == hidden, no GQA, no mask");
+
+  jpp_stage* s = new jpp_stage();
+  s->d = *d;
+  s->d.n_kv_heads = kvh;
+  s->d.head_dim = hd;
+  s->T = T; s->h = d->hidden; s->f = d->ffn; s->hd = hd;
+  s->qkvw = (int64_t)(d->n_heads + 2 * kvh) * hd;
+  s->ctxw = (int64_t)d->n_heads * hd;
+  const int64_t h = s->h, f = s->f;
+  if (d->family == JPP_FAMILY_BERT)
+    s->pinfo = {{"Wqkv", h, 3 * h}, {"bqkv", 1, 3 * h}, {"Wo", h, h}, {"bo", 1, h},
+                {"ln1_g", 1, h}, {"ln1_b", 1, h}, {"W1", h, f}, {"b1", 1, f},
+                {"W2", f, h}, {"b2", 1, h}, {"ln2_g", 1, h}, {"ln2_b", 1, h}};
+  else
+    s->pinfo = {{"rms1_g", 1, h}, {"Wqkv", h, s->qkvw}, {"Wo", s->ctxw, h},
+                {"rms2_g", 1, h}, {"Wgu", h, 2 * f}, {"Wd", f, h}};
+  size_t off = 0;
+  for (auto& p : s->pinfo) {
+    s->poff.push_back(off);
+    off += (size_t)((p.rows * p.cols + 127) / 128 * 128);  // keep 256-byte alignment
+  }
+  s->layer_elems = off;
+
+  // residual slots
+  Carver slot;
+  s->lay.resize(d->layers_per_chunk);
+  for (auto& L : s->lay) {
+    carve_layer(s, slot, L, false);
+    if (d->split_backward) carve_w(s, slot, L);
+  }
+  s->slot_bytes = slot.total;
+
+  // scratch
+  Carver sc;
+  if (!d->split_backward) carve_w(s, sc, s->wshared);
+  const size_t e = 2;
+  s->s_dx[0] = sc.take(T * h * e);
+  s->s_dx[1] = sc.take(T * h * e);
+  s->s_t1 = sc.take(T * (d->family == JPP_FAMILY_BERT ? h : f) * e);
+  s->s_t2 = sc.take(T * h * e);
+  s->s_t3 = sc.take(T * s->ctxw * e);
+  const size_t widest = (size_t)std::max<int64_t>(std::max<int64_t>(s->qkvw, 2 * f), h);
+  s->s_partial = sc.take((size_t)2 * JPP_NORM_PARTIALS * widest * 4);
+  s->s_delta = sc.take((size_t)d->batch * d->n_heads * d->seq * 4);
+  size_t max_w = 0;
+  for (auto& p : s->pinfo) max_w = std::max(max_w, (size_t)(p.rows * p.cols));
+  s->s_wg = sc.take(d->fused_wgrad_accum ? 256 : max_w * e);
+  s->s_cos = sc.take((size_t)d->seq * (hd / 2) * 4);
+  s->s_sin = sc.take((size_t)d->seq * (hd / 2) * 4);
+  s->scratch_bytes = sc.total;
+
+  const size_t n_layers = (size_t)d->n_chunks * d->layers_per_chunk;
+  hipError_t e1 = hipMalloc((void**)&s->params, n_layers * s->layer_elems * 2);
+  hipError_t e2 = e1 == hipSuccess ? hipMalloc((void**)&s->grads, n_layers * s->layer_elems * 4)
+                                   : e1;
+  hipError_t e3 = e2 == hipSuccess ? hipMalloc((void**)&s->scratch, s->scratch_bytes) : e2;
+  hipError_t e4 = e3;
+  if (e3 == hipSuccess) {
+    for (int i = 0; i < d->max_live; ++i) {
+      uint8_t* p = nullptr;
+      e4 = hipMalloc((void**)&p, s->slot_bytes);
+      if (e4 != hipSuccess) break;
+      s->slots.push_back(p);
+      s->free_slots.push_back(d->max_live - 1 - i);
+    }
+  }
+  if (e4 != hipSuccess) {
+    jpp_stage_destroy(s);
+    return jpp_set_error(JPP_ERR_HIP, "stage_create: allocation failed: %s",
+                         hipGetErrorString(e4));
+  }
+  s->total_bytes = n_layers * s->layer_elems * 6 + s->scratch_bytes + s->slot_bytes * d->max_live;
+  hipMemset(s->params, 0, n_layers * s->layer_elems * 2);
+  hipMemset(s->grads, 0, n_layers * s->layer_elems * 4);
+
+  if (d->family != JPP_FAMILY_BERT) {
+    // cos/sin of pos * theta^(-2i/d): evaluated in double, stored as f32
+    const int half = hd / 2;
+    std::vector<float> c((size_t)d->seq * half), sn((size_t)d->seq * half);
+    for (int pos = 0; pos < d->seq; ++pos)
+      for (int i = 0; i < half; ++i) {
+        const double ang = (double)pos * pow((double)d->rope_theta, -2.0 * i / hd);
+        c[(size_t)pos * half + i] = (float)cos(ang);
+        sn[(size_t)pos * half + i] = (float)sin(ang);
+      }
+    hipMemcpy(s->S<>(s->s_cos), c.data(), c.size() * 4, hipMemcpyHostToDevice);
+    hipMemcpy(s->S<>(s->s_sin), sn.data(), sn.size() * 4, hipMemcpyHostToDevice);
+  }
+  hipError_t e5 = hipDeviceSynchronize();
+  if (e5 != hipSuccess) {
+    jpp_stage_destroy(s);
+    return jpp_set_error(JPP_ERR_HIP, "stage_create: %s", hipGetErrorString(e5));
+  }
+  *out = s;
+  return JPP_OK;
+}
+
+int jpp_stage_destroy(jpp_stage* s) {
+  if (!s) return JPP_OK;
+  hipDeviceSynchronize();
+  for (auto p : s->slots) hipFree(p);
+  if (s->scratch) hipFree(s->scratch);
+  if (s->grads) hipFree(s->grads);
+  if (s->params) hipFree(s->params);
+  delete s;
+  return JPP_OK;
+}
+
+int jpp_stage_n_params(const jpp_stage* s) { return s ? (int)s->pinfo.size() : 0; }
+
+int jpp_stage_param_info(const jpp_stage* s, int i, const char** name, int64_t* rows,
+                         int64_t* cols) {
+  JPP_REQUIRE(s && i >= 0 && i < (int)s->pinfo.size(), "param_info: bad index %d", i);
+  if (name) *name = s->pinfo[i].name;
+  if (rows) *rows = s->pinfo[i].rows;
+  if (cols) *cols = s->pinfo[i].cols;
+  return JPP_OK;
+}
+
+static int check_pli(const jpp_stage* s, int chunk, int layer, int i) {
+  JPP_REQUIRE(s, "stage: null");
+  JPP_REQUIRE(chunk >= 0 && chunk < s->d.n_chunks && layer >= 0 && layer < s->d.layers_per_chunk &&
+                  i >= 0 && i < (int)s->pinfo.size(),
+              "stage: (chunk %d, layer %d, param %d) out of range", chunk, layer, i);
+  return JPP_OK;
+}
+
+int jpp_stage_param_ptr(jpp_stage* s, int chunk, int layer, int i, void** ptr) {
+  RC(check_pli(s, chunk, layer, i));
+  *ptr = s->P(chunk, layer, i);
+  return JPP_OK;
+}
+
+int jpp_stage_grad_ptr(jpp_stage* s, int chunk, int layer, int i, float** ptr) {
+  RC(check_pli(s, chunk, layer, i));
+  *ptr = s->G(chunk, layer, i);
+  return JPP_OK;
+}
+
+int jpp_stage_zero_grads(jpp_stage* s, void* stream) {
+  JPP_REQUIRE(s, "stage: null");
+  const size_t n = (size_t)s->d.n_chunks * s->d.layers_per_chunk * s->layer_elems;
+  return jpp_fill_u32(s->grads, 0u, n, stream);
+}
+
+size_t jpp_stage_bytes(const jpp_stage* s) { return s ? s->total_bytes : 0; }
+int jpp_stage_live_slots(const jpp_stage* s) { return s ? (int)s->live.size() : 0; }
+
+int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in, void* out,
+                       void* stream) {
+  JPP_REQUIRE(s, "run_task: null stage");
+  JPP_REQUIRE(chunk >= 0 && chunk < s->d.n_chunks, "run_task: chunk %d out of range", chunk);
+  hipStream_t st = (hipStream_t)stream;
+  const int nl = s->d.layers_per_chunk;
+  const size_t act = (size_t)s->T * s->h * 2;
+  const auto key = std::make_pair(chunk, mb);
+
+  if (kind == JPP_FWD) {
+    JPP_REQUIRE(in && out, "run_task(FWD): needs in and out");
+    if (s->live.count(key))
+      return jpp_set_error(JPP_ERR_STATE, "run_task(FWD): (chunk %d, mubatch %d) is already live",
+                           chunk, mb);
+    if (s->free_slots.empty())
+      return jpp_set_error(JPP_ERR_STATE,
+                           "run_task(FWD): all %d residual slots are live; the schedule needs a "
+                           "larger max_live", s->d.max_live);
+    const int slot_i = s->free_slots.back();
+    s->free_slots.pop_back();
+    s->live[key] = slot_i;
+    s->phase[key] = 1;
+    uint8_t* slot = s->slots[slot_i];
+    JPP_CHECK_HIP(hipMemcpyAsync(slot + s->lay[0].x.off, in, act, hipMemcpyDeviceToDevice, st));
+    for (int li = 0; li < nl; ++li) {
+      void* y = li + 1 < nl ? (void*)(slot + s->lay[li + 1].x.off) : out;
+      RC(layer_fwd(s, st, chunk, li, slot, y));
+    }
+    return JPP_OK;
+  }
+
+  auto it = s->live.find(key);
+  if (it == s->live.end())
+    return jpp_set_error(JPP_ERR_STATE, "run_task: no forward residuals for (chunk %d, mubatch %d)",
+                         chunk, mb);
+  uint8_t* slot = s->slots[it->second];
+  const int ph = s->phase[key];
+  const bool split = s->d.split_backward != 0;
+
+  if (kind == JPP_BWD || kind == JPP_BWD_I) {
+    JPP_REQUIRE(in && out, "run_task(BWD): needs in and out");
+    if (ph != 1)
+      return jpp_set_error(JPP_ERR_STATE, "run_task: backward of (chunk %d, mubatch %d) ran twice",
+                           chunk, mb);
+    if (kind == JPP_BWD_I && !split)
+      return jpp_set_error(JPP_ERR_STATE,
+                           "run_task(BWD_I): stage was created without split_backward");
+    const void* dy = in;
+    for (int li = nl - 1; li >= 0; --li) {
+      uint8_t* wbase = split ? slot : s->scratch;
+      const LayerStash& W = split ? s->lay[li] : s->wshared;
+      void* dx;
+      if (li == 0) dx = out;
+      else if (split && s->d.family != JPP_FAMILY_BERT) dx = slot + s->lay[li - 1].dyin.off;
+      else dx = s->S<>(s->s_dx[li & 1]);
+      if (split && s->d.family != JPP_FAMILY_BERT && li == nl - 1) {
+        // the weight-gradient task reads the incoming cotangent again later
+        JPP_CHECK_HIP(hipMemcpyAsync(slot + s->lay[li].dyin.off, in, act,
+                                     hipMemcpyDeviceToDevice, st));
+        dy = slot + s->lay[li].dyin.off;
+      }
+      RC(layer_bwd_i(s, st, chunk, li, slot, wbase, W, dy, dx));
+      if (kind == JPP_BWD) RC(layer_bwd_w(s, st, chunk, li, slot, wbase, W, dy));
+      dy = dx;
+    }
+    if (kind == JPP_BWD) {
+      s->free_slots.push_back(it->second);
+      s->live.erase(it);
+      s->phase.erase(key);
+    } else {
+      s->phase[key] = 2;
+    }
+    return JPP_OK;
+  }
+
+  if (kind == JPP_BWD_W) {
+    if (!split)
+      return jpp_set_error(JPP_ERR_STATE,
+                           "run_task(BWD_W): stage was created without split_backward");
+    if (ph != 2)
+      return jpp_set_error(JPP_ERR_STATE, "run_task(BWD_W): BWD_I of (chunk %d, mubatch %d) has not run",
+                           chunk, mb);
+    for (int li = nl - 1; li >= 0; --li)
+      RC(layer_bwd_w(s, st, chunk, li, slot, slot, s->lay[li], slot + s->lay[li].dyin.off));
+    s->free_slots.push_back(it->second);
+    s->live.erase(it);
+    s->phase.erase(key);
+    return JPP_OK;
+  }
+  return jpp_set_error(JPP_ERR_INVALID, "run_task: unknown task kind %d", kind);
+}
+
+}  // extern "C"

@@ -1,0 +1,351 @@
+"""ctypes binding of ``libjaxpp_amd.so`` (the C ABI in include/jaxpp_amd.h).
+
+This is the host side for a process that has no GPU runtime of its own: it
+owns device buffers through the library's allocation helpers and drives the
+stage executor.  There is no CPU fallback: without the built library or
+without a GPU every call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Iterable
+
+import numpy as np
+
+from jaxpp_amd.types import TaskType
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libjaxpp_amd.so")
+_lib = None
+
+
+class JppError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"jaxpp_amd error {code}: {msg}")
+        self.code = code
+
+
+class GemmArgs(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p), ("c2", C.c_void_p),
+                ("bias", C.c_void_p), ("resid", C.c_void_p), ("aux", C.c_void_p),
+                ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64),
+                ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64),
+                ("ldc2", C.c_int64), ("ldresid", C.c_int64), ("ldaux", C.c_int64),
+                ("trans_a", C.c_int), ("trans_b", C.c_int), ("epilogue", C.c_int),
+                ("gelu_tanh", C.c_int), ("tile", C.c_int)]
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
+                ("lse", C.c_void_p), ("d_o", C.c_void_p), ("dq", C.c_void_p),
+                ("dk", C.c_void_p), ("dv", C.c_void_p), ("delta", C.c_void_p),
+                ("ldq", C.c_int64), ("ldk", C.c_int64), ("ldv", C.c_int64), ("ldo", C.c_int64),
+                ("lddo", C.c_int64), ("lddq", C.c_int64), ("lddk", C.c_int64),
+                ("lddv", C.c_int64),
+                ("batch", C.c_int), ("seq", C.c_int), ("n_heads", C.c_int),
+                ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("causal", C.c_int)]
+
+
+class NormArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("gamma", C.c_void_p), ("beta", C.c_void_p),
+                ("y", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p),
+                ("dy", C.c_void_p), ("resid", C.c_void_p), ("dx", C.c_void_p),
+                ("dgamma", C.c_void_p), ("dbeta", C.c_void_p), ("partial", C.c_void_p),
+                ("rows", C.c_int64), ("cols", C.c_int64), ("eps", C.c_float)]
+
+
+class StageDesc(C.Structure):
+    _fields_ = [("family", C.c_int), ("hidden", C.c_int), ("n_heads", C.c_int),
+                ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("ffn", C.c_int),
+                ("seq", C.c_int), ("batch", C.c_int), ("causal", C.c_int),
+                ("rope_theta", C.c_float), ("eps", C.c_float), ("gelu_tanh", C.c_int),
+                ("n_experts", C.c_int), ("top_k", C.c_int), ("n_chunks", C.c_int),
+                ("layers_per_chunk", C.c_int), ("max_live", C.c_int),
+                ("split_backward", C.c_int), ("fused_wgrad_accum", C.c_int)]
+
+
+EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32 = range(5)
+NORM_PARTIALS = 256
+FAMILY = {"bert": 0, "llama": 1, "mixtral": 2}
+
+# every symbol include/jaxpp_amd.h declares
+EXPORTS = [
+    "jpp_last_error", "jpp_version", "jpp_device_count", "jpp_set_device", "jpp_malloc",
+    "jpp_free", "jpp_memcpy_h2d", "jpp_memcpy_d2h", "jpp_memcpy_d2d_async", "jpp_fill_u32",
+    "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_device_sync",
+    "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
+    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
+    "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
+    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
+    "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
+    "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_bytes",
+    "jpp_stage_run_task", "jpp_stage_live_slots",
+]
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load():
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(
+            f"{_LIB_PATH} is missing: build it with `python -m jaxpp_amd.build` "
+            "(there is no fallback path)")
+    lib = C.CDLL(_LIB_PATH)
+    lib.jpp_last_error.restype = C.c_char_p
+    lib.jpp_stage_bytes.restype = C.c_size_t
+    lib.jpp_stage_bytes.argtypes = [C.c_void_p]
+    lib.jpp_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    lib.jpp_free.argtypes = [C.c_void_p]
+    lib.jpp_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.jpp_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.jpp_memcpy_d2d_async.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    lib.jpp_fill_u32.argtypes = [C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]
+    lib.jpp_stream_create.argtypes = [C.POINTER(C.c_void_p)]
+    lib.jpp_stream_destroy.argtypes = [C.c_void_p]
+    lib.jpp_stream_sync.argtypes = [C.c_void_p]
+    lib.jpp_event_create.argtypes = [C.POINTER(C.c_void_p)]
+    lib.jpp_event_destroy.argtypes = [C.c_void_p]
+    lib.jpp_event_record.argtypes = [C.c_void_p, C.c_void_p]
+    lib.jpp_event_sync.argtypes = [C.c_void_p]
+    lib.jpp_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
+    lib.jpp_mem_info.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    lib.jpp_gemm_bf16.argtypes = [C.c_void_p, C.POINTER(GemmArgs)]
+    lib.jpp_attn_fwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
+    lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
+    lib.jpp_norm_fwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
+    lib.jpp_norm_bwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
+    lib.jpp_swiglu_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]
+    lib.jpp_swiglu_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                   C.c_int64]
+    lib.jpp_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int,
+                             C.c_int, C.c_int, C.c_int, C.c_int]
+    lib.jpp_grad_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+    lib.jpp_colsum_accum.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                     C.c_void_p, C.c_void_p]
+    lib.jpp_cast_f32_to_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
+    lib.jpp_cast_bf16_to_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
+    lib.jpp_stage_create.argtypes = [C.POINTER(StageDesc), C.POINTER(C.c_void_p)]
+    lib.jpp_stage_destroy.argtypes = [C.c_void_p]
+    lib.jpp_stage_n_params.argtypes = [C.c_void_p]
+    lib.jpp_stage_param_info.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_char_p),
+                                         C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+    lib.jpp_stage_param_ptr.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                        C.POINTER(C.c_void_p)]
+    lib.jpp_stage_grad_ptr.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                       C.POINTER(C.c_void_p)]
+    lib.jpp_stage_zero_grads.argtypes = [C.c_void_p, C.c_void_p]
+    lib.jpp_stage_run_task.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                       C.c_void_p, C.c_void_p]
+    lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
+    _lib = lib
+    return lib
+
+
+def check(rc: int):
+    if rc != 0:
+        raise JppError(rc, load().jpp_last_error().decode(errors="replace"))
+
+
+def device_count() -> int:
+    n = C.c_int(0)
+    rc = load().jpp_device_count(C.byref(n))
+    return n.value if rc == 0 else 0
+
+
+def require_gpu():
+    if device_count() < 1:
+        raise RuntimeError("jaxpp_amd needs a GPU: no HIP device is visible")
+
+
+# ---------------------------------------------------------------------------
+# bf16 <-> float32 on the host (round to nearest even), numpy only
+# ---------------------------------------------------------------------------
+def to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    r = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    return r.astype(np.uint16)
+
+
+def from_bf16_bits(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(
+        np.float32)
+
+
+class DeviceBuffer:
+    """A device allocation owned by this object."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        check(load().jpp_malloc(C.byref(p), self.nbytes))
+        self.ptr = p.value or 0
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        buf = cls(a.nbytes)
+        buf.upload(a)
+        return buf
+
+    @classmethod
+    def from_f32_as_bf16(cls, a: np.ndarray) -> "DeviceBuffer":
+        return cls.from_numpy(to_bf16_bits(a))
+
+    def upload(self, a: np.ndarray, offset: int = 0):
+        a = np.ascontiguousarray(a)
+        assert offset + a.nbytes <= self.nbytes
+        check(load().jpp_memcpy_h2d(self.ptr + offset, a.ctypes.data, a.nbytes))
+
+    def download(self, dtype, shape, offset: int = 0) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        check(load().jpp_memcpy_d2h(out.ctypes.data, self.ptr + offset, out.nbytes))
+        return out
+
+    def download_bf16(self, shape) -> np.ndarray:
+        return from_bf16_bits(self.download(np.uint16, shape))
+
+    def zero(self, stream=None):
+        check(load().jpp_fill_u32(self.ptr, 0, self.nbytes // 4, stream))
+
+    def free(self):
+        if self.ptr:
+            load().jpp_free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def upload_ptr(ptr: int, a: np.ndarray):
+    a = np.ascontiguousarray(a)
+    check(load().jpp_memcpy_h2d(ptr, a.ctypes.data, a.nbytes))
+
+
+def download_ptr(ptr: int, dtype, shape) -> np.ndarray:
+    out = np.empty(shape, dtype=dtype)
+    check(load().jpp_memcpy_d2h(out.ctypes.data, ptr, out.nbytes))
+    return out
+
+
+def sync():
+    check(load().jpp_device_sync())
+
+
+class Event:
+    def __init__(self):
+        p = C.c_void_p()
+        check(load().jpp_event_create(C.byref(p)))
+        self.ptr = p.value
+
+    def record(self, stream=None):
+        check(load().jpp_event_record(self.ptr, stream))
+
+    def sync(self):
+        check(load().jpp_event_sync(self.ptr))
+
+    def elapsed_ms(self, later: "Event") -> float:
+        ms = C.c_float()
+        check(load().jpp_event_elapsed_ms(self.ptr, later.ptr, C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                load().jpp_event_destroy(self.ptr)
+        except Exception:
+            pass
+
+
+# ---------------------------------------------------------------------------
+# kernel wrappers (thin: arguments are device pointers)
+# ---------------------------------------------------------------------------
+def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, bias=None,
+         resid=None, ldresid=0, aux=None, ldaux=0, c2=None, ldc2=0, gelu_tanh=0, tile=0,
+         stream=None):
+    g = GemmArgs(a, b, c, c2, bias, resid, aux, m, n, k, lda, ldb, ldc, ldc2, ldresid, ldaux,
+                 int(trans_a), int(trans_b), epilogue, gelu_tanh, tile)
+    check(load().jpp_gemm_bf16(stream, C.byref(g)))
+
+
+class StageExecutor:
+    """One pipeline rank on one GPU: parameters, fp32 gradient accumulators,
+    residual slots, and the FWD / BWD / BWD_I / BWD_W tasks."""
+
+    def __init__(self, spec, n_chunks: int, layers_per_chunk: int, max_live: int,
+                 split_backward: bool = False, fused_wgrad_accum: bool = True):
+        require_gpu()
+        self.spec = spec
+        self.n_chunks, self.layers_per_chunk = n_chunks, layers_per_chunk
+        d = StageDesc(FAMILY[spec.family], spec.hidden, spec.n_heads, spec.kvh, spec.d, spec.ffn,
+                      spec.seq, spec.batch, int(spec.causal), spec.rope_theta, spec.eps,
+                      int(spec.gelu_tanh), spec.n_experts, spec.top_k, n_chunks,
+                      layers_per_chunk, max_live, int(split_backward), int(fused_wgrad_accum))
+        h = C.c_void_p()
+        check(load().jpp_stage_create(C.byref(d), C.byref(h)))
+        self.handle = h.value
+        self.params = []
+        for i in range(load().jpp_stage_n_params(self.handle)):
+            name, r, c = C.c_char_p(), C.c_int64(), C.c_int64()
+            check(load().jpp_stage_param_info(self.handle, i, C.byref(name), C.byref(r),
+                                              C.byref(c)))
+            self.params.append((name.value.decode(), r.value, c.value))
+        self.index = {n: i for i, (n, _, _) in enumerate(self.params)}
+
+    @property
+    def nbytes(self) -> int:
+        return load().jpp_stage_bytes(self.handle)
+
+    def _ptr(self, fn, chunk, layer, name):
+        p = C.c_void_p()
+        check(fn(self.handle, chunk, layer, self.index[name], C.byref(p)))
+        return p.value
+
+    def set_params(self, chunk: int, layer: int, params: dict):
+        """Upload float32 host arrays as bf16 device parameters."""
+        for name, rows, cols in self.params:
+            a = np.asarray(params[name], dtype=np.float32)
+            assert a.size == rows * cols, (name, a.shape, rows, cols)
+            upload_ptr(self._ptr(load().jpp_stage_param_ptr, chunk, layer, name),
+                       to_bf16_bits(a))
+
+    def get_grads(self, chunk: int, layer: int) -> dict:
+        out = {}
+        for name, rows, cols in self.params:
+            shape = (cols,) if rows == 1 and not name.startswith("W") else (rows, cols)
+            out[name] = download_ptr(self._ptr(load().jpp_stage_grad_ptr, chunk, layer, name),
+                                     np.float32, shape)
+        return out
+
+    def zero_grads(self, stream=None):
+        check(load().jpp_stage_zero_grads(self.handle, stream))
+
+    def run_task(self, kind: TaskType, chunk: int, mubatch: int, inp=None, out=None,
+                 stream=None):
+        check(load().jpp_stage_run_task(self.handle, kind.value, chunk, mubatch,
+                                        inp, out, stream))
+
+    def live_slots(self) -> int:
+        return load().jpp_stage_live_slots(self.handle)
+
+    def close(self):
+        if getattr(self, "handle", None):
+            load().jpp_stage_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,46 @@
+"""The C-ABI library: it is built, loads without a GPU, and exports every
+symbol include/jaxpp_amd.h declares (no compute calls here)."""
+import ctypes
+import os
+import re
+
+from jaxpp_amd import runtime as rt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "jaxpp_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(jpp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(rt.lib_path()):
+        from jaxpp_amd.build import build
+        build(verbose=False)
+    lib = ctypes.CDLL(rt.lib_path())
+    names = declared_symbols()
+    assert len(names) >= 40
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert sorted(rt.EXPORTS) == names, "runtime.EXPORTS and the header disagree"
+
+
+def test_error_convention_without_gpu():
+    lib = rt.load()
+    assert lib.jpp_version() == 100
+    # argument checks happen on the host, before anything touches a device
+    assert lib.jpp_gemm_bf16(None, None) == -1
+    assert b"null operand" in lib.jpp_last_error()
+    assert lib.jpp_stage_create(None, None) == -1
+    assert lib.jpp_norm_fwd(None, None) == -1
+    assert lib.jpp_grad_accum_f32(None, None, None, 0, 0) == -1
+
+
+def test_struct_layouts_match_header_sizes():
+    # 7 pointers + 9 int64 + 5 int (+ padding) ; guards against field drift
+    assert ctypes.sizeof(rt.GemmArgs) == 7 * 8 + 9 * 8 + 5 * 4 + 4
+    assert ctypes.sizeof(rt.AttnArgs) == 10 * 8 + 8 * 8 + 6 * 4
+    assert ctypes.sizeof(rt.NormArgs) == 12 * 8 + 2 * 8 + 8
+    assert ctypes.sizeof(rt.StageDesc) == 19 * 4

@@ -1,0 +1,241 @@
+"""HIP kernels against the CPU oracle, called through the C ABI.
+
+Tolerances: outputs stored as bf16 are compared with rtol 2e-2 relative to the
+tensor's largest magnitude (the bar the north star sets for bf16), fp32
+accumulators with rtol 1e-4 where the arithmetic is fp32 end to end."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+
+from jaxpp_amd import runtime as rt
+from oracle import layers as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    rt.require_gpu()
+
+
+def dev_bf16(a):
+    return rt.DeviceBuffer.from_f32_as_bf16(a)
+
+
+def rnd(rng, *shape, scale=1.0):
+    return L.bf16_round((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+def close(got, want, rtol=2e-2, what=""):
+    scale = float(np.abs(want).max()) + 1e-30
+    err = float(np.abs(got - want).max())
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+
+
+GEMM_CASES = [  # (trans_a, trans_b, epilogue)
+    (0, 1, rt.EPI_BF16), (0, 1, rt.EPI_GELU), (0, 1, rt.EPI_F32),
+    (0, 0, rt.EPI_BF16), (0, 0, rt.EPI_DGELU),
+    (1, 1, rt.EPI_ACC_F32), (1, 1, rt.EPI_BF16), (1, 1, rt.EPI_F32),
+]
+
+
+@pytest.mark.parametrize("ta,tb,epi", GEMM_CASES)
+@pytest.mark.parametrize("tile,m,n,k", [(1, 128, 384, 192), (2, 512, 128, 64), (3, 256, 512, 320),
+                                        (0, 768, 256, 128)])
+def test_gemm(ta, tb, epi, tile, m, n, k):
+    print(f"gemm ta={ta} tb={tb} epi={epi} tile={tile} {m}x{n}x{k}", flush=True)
+    rng = np.random.default_rng(m + n + k + 7 * epi)
+    A = rnd(rng, m, k)
+    B = rnd(rng, n, k)
+    want = A @ B.T
+    a_h = A.T.copy() if ta else A
+    b_h = B.T.copy() if tb else B
+    da, db = dev_bf16(a_h), dev_bf16(b_h)
+    lda, ldb = a_h.shape[1], b_h.shape[1]
+    kw = {}
+    keep = []
+    if epi in (rt.EPI_BF16, rt.EPI_GELU):
+        bias = rnd(rng, n)
+        keep.append(dev_bf16(bias))
+        kw["bias"] = keep[-1].ptr
+        want = want + bias
+    if epi == rt.EPI_BF16:
+        resid = rnd(rng, m, n)
+        keep.append(dev_bf16(resid))
+        kw.update(resid=keep[-1].ptr, ldresid=n)
+        want = want + resid
+    if epi == rt.EPI_DGELU:
+        aux = rnd(rng, m, n)
+        keep.append(dev_bf16(aux))
+        kw.update(aux=keep[-1].ptr, ldaux=n)
+        want = want * L.gelu_grad(aux.astype(np.float64)).astype(np.float32)
+    f32_out = epi in (rt.EPI_ACC_F32, rt.EPI_F32)
+    if epi == rt.EPI_ACC_F32:
+        prev = rng.standard_normal((m, n)).astype(np.float32)
+        dc = rt.DeviceBuffer.from_numpy(prev)
+        want = want + prev
+    else:
+        dc = rt.DeviceBuffer(m * n * (4 if f32_out else 2))
+    if epi == rt.EPI_GELU:
+        dc2 = rt.DeviceBuffer(m * n * 2)
+        kw.update(c2=dc2.ptr, ldc2=n)
+    rt.gemm(da.ptr, db.ptr, dc.ptr, m, n, k, lda, ldb, n, ta, tb, epi, tile=tile, **kw)
+    rt.sync()
+    if f32_out:
+        got = dc.download(np.float32, (m, n))
+        close(got, want, 1e-4 * math.sqrt(k), "gemm f32")
+    else:
+        close(dc.download_bf16((m, n)), want, 1e-2, "gemm bf16")
+    if epi == rt.EPI_GELU:
+        close(dc2.download_bf16((m, n)), L.gelu(want.astype(np.float64)).astype(np.float32), 1e-2,
+              "gemm gelu")
+
+
+def test_gemm_rejects_bad_shapes():
+    d = rt.DeviceBuffer(1 << 16)
+    with pytest.raises(rt.JppError, match="multiples of 128"):
+        rt.gemm(d.ptr, d.ptr, d.ptr, 100, 128, 64, 64, 64, 128, 0, 0)
+    with pytest.raises(rt.JppError, match="unsupported combination"):
+        rt.gemm(d.ptr, d.ptr, d.ptr, 128, 128, 64, 128, 64, 128, 1, 0)
+    with pytest.raises(rt.JppError, match="null operand"):
+        rt.gemm(None, d.ptr, d.ptr, 128, 128, 64, 64, 64, 128, 0, 0)
+
+
+@pytest.mark.parametrize("d,causal,hq,hkv,batch,seq", [
+    (64, 0, 4, 4, 2, 256), (64, 1, 2, 2, 1, 384), (128, 1, 8, 2, 1, 512),
+    (128, 0, 2, 1, 2, 128), (128, 1, 4, 4, 1, 256),
+])
+def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
+    print(f"attention d={d} causal={causal} hq={hq} hkv={hkv} b={batch} s={seq}", flush=True)
+    rng = np.random.default_rng(d + seq + hq)
+    T, width = batch * seq, (hq + 2 * hkv) * d
+    qkv = rnd(rng, T, width)
+    do = rnd(rng, T, hq * d)
+    q = qkv[:, :hq * d].reshape(batch, seq, hq, d)
+    k = qkv[:, hq * d:(hq + hkv) * d].reshape(batch, seq, hkv, d)
+    v = qkv[:, (hq + hkv) * d:].reshape(batch, seq, hkv, d)
+    o_w, lse_w = L.attention_fwd(q, k, v, bool(causal))
+    dq_w, dk_w, dv_w = L.attention_bwd(q, k, v, L.bf16_round(o_w),
+                                       do.reshape(batch, seq, hq, d), lse_w, bool(causal))
+    dqkv_w = np.concatenate([dq_w.reshape(T, -1), dk_w.reshape(T, -1), dv_w.reshape(T, -1)], -1)
+
+    dqkv_d = rt.DeviceBuffer(T * width * 2)
+    dqkv_d.zero()
+    b_qkv, b_o, b_do = dev_bf16(qkv), rt.DeviceBuffer(T * hq * d * 2), dev_bf16(do)
+    b_lse = rt.DeviceBuffer(batch * hq * seq * 4)
+    b_delta = rt.DeviceBuffer(batch * hq * seq * 4)
+    a = rt.AttnArgs(b_qkv.ptr, b_qkv.ptr + hq * d * 2, b_qkv.ptr + (hq + hkv) * d * 2, b_o.ptr,
+                    b_lse.ptr, b_do.ptr, dqkv_d.ptr, dqkv_d.ptr + hq * d * 2,
+                    dqkv_d.ptr + (hq + hkv) * d * 2, b_delta.ptr,
+                    width, width, width, hq * d, hq * d, width, width, width,
+                    batch, seq, hq, hkv, d, causal)
+    rt.check(rt.load().jpp_attn_fwd(None, C.byref(a)))
+    rt.sync()
+    close(b_o.download_bf16((T, hq * d)), o_w.reshape(T, -1), 2e-2, "attn out")
+    np.testing.assert_allclose(b_lse.download(np.float32, (batch, hq, seq)), lse_w, rtol=0,
+                               atol=2e-2)
+    rt.check(rt.load().jpp_attn_bwd(None, C.byref(a)))
+    rt.sync()
+    got = dqkv_d.download_bf16((T, width))
+    close(got[:, :hq * d], dqkv_w[:, :hq * d], 2e-2, "dq")
+    close(got[:, hq * d:(hq + hkv) * d], dqkv_w[:, hq * d:(hq + hkv) * d], 2e-2, "dk")
+    close(got[:, (hq + hkv) * d:], dqkv_w[:, (hq + hkv) * d:], 2e-2, "dv")
+
+
+@pytest.mark.parametrize("ln,rows,cols", [(True, 300, 256), (True, 1024, 1024), (False, 512, 4096),
+                                          (False, 130, 8192), (False, 64, 128)])
+def test_norm_fwd_bwd(ln, rows, cols):
+    print(f"norm ln={ln} {rows}x{cols}", flush=True)
+    rng = np.random.default_rng(rows + cols)
+    x, dy, resid = rnd(rng, rows, cols, scale=2.0), rnd(rng, rows, cols), rnd(rng, rows, cols)
+    g = L.bf16_round(1 + 0.1 * rng.standard_normal(cols).astype(np.float32))
+    b = L.bf16_round(0.1 * rng.standard_normal(cols).astype(np.float32))
+    eps = 1e-5
+    if ln:
+        y_w, mean_w, rstd_w = L.layernorm_fwd(x, g, b, eps)
+        dx_w, dg_w, db_w = L.layernorm_bwd(dy, x, mean_w, rstd_w, g)
+    else:
+        y_w, rstd_w = L.rmsnorm_fwd(x, g, eps)
+        dx_w, dg_w = L.rmsnorm_bwd(dy, x, rstd_w, g)
+    dx_w = dx_w + resid
+    bx, bg, bb, bdy, br = dev_bf16(x), dev_bf16(g), dev_bf16(b), dev_bf16(dy), dev_bf16(resid)
+    by, bdx = rt.DeviceBuffer(rows * cols * 2), rt.DeviceBuffer(rows * cols * 2)
+    bmean, brstd = rt.DeviceBuffer(rows * 4), rt.DeviceBuffer(rows * 4)
+    prev_g = rng.standard_normal(cols).astype(np.float32)
+    prev_b = rng.standard_normal(cols).astype(np.float32)
+    bdg, bdb = rt.DeviceBuffer.from_numpy(prev_g), rt.DeviceBuffer.from_numpy(prev_b)
+    part = rt.DeviceBuffer(2 * rt.NORM_PARTIALS * cols * 4)
+    a = rt.NormArgs(bx.ptr, bg.ptr, bb.ptr if ln else None, by.ptr, bmean.ptr if ln else None,
+                    brstd.ptr, bdy.ptr, br.ptr, bdx.ptr, bdg.ptr, bdb.ptr if ln else None,
+                    part.ptr, rows, cols, eps)
+    rt.check(rt.load().jpp_norm_fwd(None, C.byref(a)))
+    rt.check(rt.load().jpp_norm_bwd(None, C.byref(a)))
+    rt.sync()
+    close(by.download_bf16((rows, cols)), y_w, 1e-2, "norm y")
+    np.testing.assert_allclose(brstd.download(np.float32, (rows,)), rstd_w, rtol=1e-4)
+    if ln:
+        np.testing.assert_allclose(bmean.download(np.float32, (rows,)), mean_w, rtol=1e-3, atol=1e-5)
+    close(bdx.download_bf16((rows, cols)), dx_w, 1e-2, "norm dx")
+    close(bdg.download(np.float32, (cols,)), prev_g + dg_w, 1e-3, "dgamma")
+    if ln:
+        close(bdb.download(np.float32, (cols,)), prev_b + db_w, 1e-3, "dbeta")
+
+
+def test_swiglu_rope_accum_colsum_cast():
+    rng = np.random.default_rng(5)
+    lib = rt.load()
+    rows, f = 96, 1024
+    gu, ds = rnd(rng, rows, 2 * f, scale=2.0), rnd(rng, rows, f)
+    bgu, bds = dev_bf16(gu), dev_bf16(ds)
+    bs, bdgu = rt.DeviceBuffer(rows * f * 2), rt.DeviceBuffer(rows * 2 * f * 2)
+    rt.check(lib.jpp_swiglu_fwd(None, bgu.ptr, bs.ptr, rows, f))
+    rt.check(lib.jpp_swiglu_bwd(None, bgu.ptr, bds.ptr, bdgu.ptr, rows, f))
+    rt.sync()
+    close(bs.download_bf16((rows, f)), L.swiglu(gu, f), 1e-2, "swiglu")
+    close(bdgu.download_bf16((rows, 2 * f)), L.swiglu_bwd(gu, ds, f), 1e-2, "swiglu bwd")
+
+    batch, seq, heads, d, extra = 2, 64, 6, 128, 2
+    ld = (heads + extra) * d
+    x = rnd(rng, batch * seq, ld)
+    cos, sin = L.rope_tables(seq, d, 5e5, np.float32)
+    bc, bsn = rt.DeviceBuffer.from_numpy(cos), rt.DeviceBuffer.from_numpy(sin)
+    for inverse in (0, 1):
+        bx = dev_bf16(x)
+        rt.check(lib.jpp_rope(None, bx.ptr, ld, bc.ptr, bsn.ptr, batch, seq, heads, d, inverse))
+        rt.sync()
+        want = x.copy()
+        rot = L.rope_apply(x[:, :heads * d].reshape(batch, seq, heads, d), cos, sin, bool(inverse))
+        want[:, :heads * d] = rot.reshape(batch * seq, -1)
+        got = bx.download_bf16((batch * seq, ld))
+        close(got, want, 1e-2, "rope")
+        np.testing.assert_array_equal(got[:, heads * d:], x[:, heads * d:])
+
+    for n, f32 in [(8 * 1000 + 3, 0), (4096, 1), (5, 0)]:
+        acc = rng.standard_normal(n).astype(np.float32)
+        g = rng.standard_normal(n).astype(np.float32)
+        if not f32:
+            g = L.bf16_round(g)
+        bacc = rt.DeviceBuffer.from_numpy(acc)
+        bg = rt.DeviceBuffer.from_numpy(g if f32 else rt.to_bf16_bits(g))
+        rt.check(lib.jpp_grad_accum_f32(None, bacc.ptr, bg.ptr, n, f32))
+        rt.sync()
+        np.testing.assert_array_equal(bacc.download(np.float32, (n,)), acc + g)
+
+    rows, cols = 1000, 3072
+    xx = rnd(rng, rows, cols)
+    acc = rng.standard_normal(cols).astype(np.float32)
+    bacc, bx = rt.DeviceBuffer.from_numpy(acc), dev_bf16(xx)
+    part = rt.DeviceBuffer(rt.NORM_PARTIALS * cols * 4)
+    rt.check(lib.jpp_colsum_accum(None, bx.ptr, cols, rows, cols, bacc.ptr, part.ptr))
+    rt.sync()
+    close(bacc.download(np.float32, (cols,)), acc + xx.sum(0), 1e-4, "colsum")
+
+    src = rng.standard_normal(1001).astype(np.float32)
+    bsrc, bdst = rt.DeviceBuffer.from_numpy(src), rt.DeviceBuffer(1001 * 2)
+    rt.check(lib.jpp_cast_f32_to_bf16(None, bsrc.ptr, bdst.ptr, 1001))
+    rt.sync()
+    np.testing.assert_array_equal(bdst.download(np.uint16, (1001,)), L.f32_to_bf16_bits(src))
+    np.testing.assert_array_equal(rt.to_bf16_bits(src), L.f32_to_bf16_bits(src))

@@ -1,0 +1,159 @@
+"""The stage executor (through the C ABI) against the oracle's rank executor:
+same parameters, same synthetic boundary tensors, same task-table row.
+
+Bar: bf16 results within 2e-2 of the tensor's largest magnitude; the order of
+tasks must not change the accumulated gradients at all (bit-identical between
+two schedules of the same work)."""
+import numpy as np
+import pytest
+
+from jaxpp_amd import runtime as rt
+from jaxpp_amd import schedules as S
+from jaxpp_amd.model import LayerSpec, boundary_tensor, init_layer_params
+from jaxpp_amd.plan import make_rank_plan
+from jaxpp_amd.types import TaskType
+from oracle import layers as L
+from oracle import stage as O
+
+pytestmark = pytest.mark.gpu
+
+BERT = LayerSpec("bert", 128, 2, 256, 128, 1, eps=1e-12)
+BERT_TANH = LayerSpec("bert", 256, 4, 512, 128, 2, eps=1e-6, gelu_tanh=True)
+LLAMA = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
+                  rope_theta=5e5, eps=1e-5)
+LLAMA_D64 = LayerSpec("llama", 256, 4, 256, 256, 1, n_kv_heads=2, head_dim=64, causal=True,
+                      rope_theta=1e4, eps=1e-5)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    rt.require_gpu()
+
+
+def close(got, want, rtol, what):
+    scale = float(np.abs(want).max()) + 1e-30
+    err = float(np.abs(got - want).max())
+    assert np.isfinite(got).all(), f"{what}: non-finite"
+    assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+
+
+def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0):
+    shape = (spec.tokens, spec.hidden)
+    ex = rt.StageExecutor(spec, plan.n_chunks, layers_per_chunk, plan.max_live,
+                          plan.split_backward, fused)
+    for c, stage in enumerate(plan.stages):
+        for li in range(layers_per_chunk):
+            ex.set_params(c, li, params[stage][li])
+    ys, dxs = {}, {}
+    out = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+    for pt in plan.tasks:
+        t = pt.task
+        key = (t.stage_id, t.mubatch_idx)
+        print(f"  task {t} as {pt.exec_kind.name}", flush=True)
+        if pt.exec_kind is TaskType.BWD_W:
+            ex.run_task(pt.exec_kind, pt.chunk, t.mubatch_idx)
+            continue
+        kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
+        inp = rt.DeviceBuffer.from_f32_as_bf16(boundary_tensor(kind, *key, shape, seed))
+        ex.run_task(pt.exec_kind, pt.chunk, t.mubatch_idx, inp.ptr, out.ptr)
+        rt.sync()
+        (ys if kind == "x" else dxs)[key] = out.download_bf16(shape)
+    assert ex.live_slots() == 0
+    grads = {stage: [ex.get_grads(c, li) for li in range(layers_per_chunk)]
+             for c, stage in enumerate(plan.stages)}
+    ex.close()
+    return ys, dxs, grads
+
+
+def run_on_oracle(spec, plan, params, row, seed=0):
+    cfg = L.LayerCfg(**spec.as_dict())
+    shape = (spec.tokens, spec.hidden)
+    ro = O.RankOracle(cfg, {s: params[s] for s in plan.stages}, L.Numerics.bf16())
+    ys, dxs = ro.run_row(row,
+                         lambda s, m: L.bf16_round(boundary_tensor("x", s, m, shape, seed)),
+                         lambda s, m: L.bf16_round(boundary_tensor("dy", s, m, shape, seed)))
+    return ys, dxs, ro.acc
+
+
+def make_params(spec, stages, layers_per_chunk):
+    return {s: [{k: L.bf16_round(v) for k, v in
+                 init_layer_params(spec, 3, s * layers_per_chunk + li, perturb=True).items()}
+                for li in range(layers_per_chunk)] for s in stages}
+
+
+CASES = [
+    ("bert-1f1b", BERT, S.Std1F1B(2), 4, 0, 2),
+    ("bert-tanh-zb", BERT_TANH, S.ZeroBubble(2), 3, 1, 1),
+    ("llama-interleaved", LLAMA, S.Interleaved1F1B(4, 2), 4, 0, 2),
+    ("llama-zb-first-stage", LLAMA, S.ZeroBubble(2), 2, 0, 1),
+    ("llama-d64-zb", LLAMA_D64, S.ZeroBubble(3), 3, 1, 2),
+    ("llama-dualpipev", LLAMA, S.DualPipeV(4, 2), 4, 1, 1),
+]
+
+
+@pytest.mark.parametrize("name,spec,sched,n,rank,lpc", CASES, ids=[c[0] for c in CASES])
+def test_stage_matches_oracle(name, spec, sched, n, rank, lpc):
+    print(f"stage case {name}", flush=True)
+    plan = make_rank_plan(sched, n, rank)
+    params = make_params(spec, plan.stages, lpc)
+    row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
+    ys_w, dxs_w, acc_w = run_on_oracle(spec, plan, params, row)
+    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params)
+    assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
+    for k in ys_w:
+        close(ys[k], ys_w[k], 2e-2, f"y{k}")
+    for k in dxs_w:
+        close(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
+    for s in plan.stages:
+        for li in range(lpc):
+            for pname, want in acc_w[s][li].items():
+                close(grads[s][li][pname], want, 2e-2, f"grad {s}/{li}/{pname}")
+
+
+def test_task_order_does_not_change_gradients():
+    """GPipe order vs 1F1B order of the same work: accumulators bit-identical."""
+    spec, n = LLAMA, 4
+    params = make_params(spec, [0], 1)
+    res = []
+    for sched in (S.GPipe(2), S.Std1F1B(2), S.ZeroBubble(2)):
+        plan = make_rank_plan(sched, n, 0)
+        res.append(run_on_gpu(spec, plan, 1, params))
+    for other in res[1:]:
+        for k, v in res[0][2][0][0].items():
+            np.testing.assert_array_equal(other[2][0][0][k], v, err_msg=k)
+        for k, v in res[0][1].items():
+            np.testing.assert_array_equal(other[1][k], v)
+
+
+def test_unfused_accumulate_path_is_close():
+    spec, n = BERT, 2
+    params = make_params(spec, [0], 1)
+    plan = make_rank_plan(S.Std1F1B(1), n, 0)
+    a = run_on_gpu(spec, plan, 1, params, fused=True)
+    b = run_on_gpu(spec, plan, 1, params, fused=False)
+    for k, v in a[2][0][0].items():
+        close(b[2][0][0][k], v, 1e-2, k)
+
+
+def test_lifetime_errors():
+    spec = BERT
+    ex = rt.StageExecutor(spec, 1, 1, 1, False, True)
+    buf = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+    buf.zero()
+    with pytest.raises(rt.JppError, match="no forward residuals"):
+        ex.run_task(TaskType.BWD, 0, 0, buf.ptr, buf.ptr)
+    ex.run_task(TaskType.FWD, 0, 0, buf.ptr, buf.ptr)
+    with pytest.raises(rt.JppError, match="already live"):
+        ex.run_task(TaskType.FWD, 0, 0, buf.ptr, buf.ptr)
+    with pytest.raises(rt.JppError, match="residual slots are live"):
+        ex.run_task(TaskType.FWD, 0, 1, buf.ptr, buf.ptr)
+    with pytest.raises(rt.JppError, match="without split_backward"):
+        ex.run_task(TaskType.BWD_I, 0, 0, buf.ptr, buf.ptr)
+    with pytest.raises(rt.JppError, match="chunk 3 out of range"):
+        ex.run_task(TaskType.FWD, 3, 0, buf.ptr, buf.ptr)
+    ex.run_task(TaskType.BWD, 0, 0, buf.ptr, buf.ptr)
+    rt.sync()
+    assert ex.live_slots() == 0
+    ex.close()
+    with pytest.raises(rt.JppError, match="head_dim must be 64 or 128"):
+        rt.StageExecutor(LayerSpec("bert", 128, 4, 256, 128, 1), 1, 1, 1)
