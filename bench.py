@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Stage throughput on one MI355X: one pipeline rank's microbatch loop
+(forward, backward, fp32 gradient accumulation, residual stash/restore) in the
+order the schedule's task table dictates, with synthetic boundary tensors.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3]
+
+A step is one full pass over the rank's row of the task table (all
+microbatches).  Prints one JSON line (see README / DESIGN.md for the fields).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from jaxpp_amd import runtime as rt            # noqa: E402
+from jaxpp_amd import schedules as S           # noqa: E402
+from jaxpp_amd.model import workloads          # noqa: E402
+from jaxpp_amd.plan import make_rank_plan      # noqa: E402
+from jaxpp_amd.types import TaskType           # noqa: E402
+
+MFMA_BF16_PEAK = 2.5e15     # dense bf16 FLOP/s, MI355X
+HBM_PEAK = 8.0e12           # B/s
+
+
+def synthetic_pool(n_elems: int, std: float, seed: int) -> np.ndarray:
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return rt.to_bf16_bits(rng.standard_normal(n_elems, dtype=np.float32) * np.float32(std))
+
+
+class Workbench:
+    """Device state of one workload: executor, parameters, boundary tensors."""
+
+    def __init__(self, wl, fused=True):
+        self.wl = wl
+        spec = wl.layer
+        sched = getattr(S, wl.schedule)(**wl.schedule_kwargs)
+        self.plan = make_rank_plan(sched, wl.n_mubatches, wl.rank)
+        self.ex = rt.StageExecutor(spec, self.plan.n_chunks, wl.layers_per_stage,
+                                   self.plan.max_live, self.plan.split_backward, fused)
+        lib = rt.load()
+        # parameters: slices of one N(0, 0.02^2) pool at per-tensor offsets;
+        # norm gains one, biases zero
+        pool_n = 1 << 26
+        wpool = rt.DeviceBuffer.from_numpy(synthetic_pool(pool_n, 0.02, 0))
+        ones = rt.DeviceBuffer.from_numpy(rt.to_bf16_bits(np.ones(16384, np.float32)))
+        import ctypes as C
+        k = 0
+        for c in range(self.plan.n_chunks):
+            for li in range(wl.layers_per_stage):
+                for name, rows, cols in self.ex.params:
+                    dst = self.ex._ptr(lib.jpp_stage_param_ptr, c, li, name)
+                    n = rows * cols
+                    if rows > 1:
+                        done = 0
+                        while done < n:
+                            k += 1
+                            off = (k * 7919 * 4096) % (pool_n // 2)
+                            take = min(n - done, pool_n - off)
+                            rt.check(lib.jpp_memcpy_d2d_async(dst + 2 * done, wpool.ptr + 2 * off,
+                                                              2 * take, None))
+                            done += take
+                    elif name.endswith("_g"):
+                        rt.check(lib.jpp_memcpy_d2d_async(dst, ones.ptr, 2 * n, None))
+        rt.sync()
+        # boundary tensors ~N(0,1): one per (chunk, microbatch) and direction
+        act = spec.tokens * spec.hidden
+        bpool_n = act + (1 << 22)
+        bpool = rt.DeviceBuffer.from_numpy(synthetic_pool(bpool_n, 1.0, 1))
+        self.x_in, self.dy_in = {}, {}
+        j = 0
+        for c in range(self.plan.n_chunks):
+            for m in range(wl.n_mubatches):
+                for store in (self.x_in, self.dy_in):
+                    j += 1
+                    buf = rt.DeviceBuffer(act * 2)
+                    off = (j * 104729 * 8) % (1 << 22)
+                    rt.check(lib.jpp_memcpy_d2d_async(buf.ptr, bpool.ptr + 2 * off, act * 2, None))
+                    store[c, m] = buf
+        self.out = rt.DeviceBuffer(act * 2)
+        rt.sync()
+        self._keep = (wpool, ones, bpool)
+
+    def step(self):
+        ex = self.ex
+        ex.zero_grads()                       # `Add.state`: accumulators start from zero
+        for pt in self.plan.tasks:
+            m = pt.task.mubatch_idx
+            if pt.exec_kind is TaskType.FWD:
+                ex.run_task(pt.exec_kind, pt.chunk, m, self.x_in[pt.chunk, m].ptr, self.out.ptr)
+            elif pt.exec_kind is TaskType.BWD_W:
+                ex.run_task(pt.exec_kind, pt.chunk, m)
+            else:
+                ex.run_task(pt.exec_kind, pt.chunk, m, self.dy_in[pt.chunk, m].ptr, self.out.ptr)
+
+    def step_flops(self) -> float:
+        wl = self.wl
+        return 3.0 * wl.layer.fwd_flops() * wl.layers_per_stage * self.plan.n_chunks * wl.n_mubatches
+
+
+def dominant_gemm_class(wl) -> str:
+    # weight-gradient GEMM with the fp32 accumulate epilogue: a third of the
+    # FLOPs and the longest kernel per call
+    big = wl.layer.hidden >= 4096
+    return "gemm_tn_accf32_256x256" if big else "gemm_tn_accf32_128x128"
+
+
+def cpu_baseline(wl, budget_layers: int = 1):
+    """The numpy oracle on the host cores: one microbatch through
+    `budget_layers` layer(s), forward + backward-input + backward-weight +
+    accumulate, scaled to the whole row (layers x chunks x microbatches)."""
+    from oracle import layers as L
+    from oracle import stage as O
+    from jaxpp_amd.model import boundary_tensor, init_layer_params
+    spec = wl.layer
+    cfg = L.LayerCfg(**spec.as_dict())
+    nm = L.Numerics.f32()
+    params = [init_layer_params(spec, 0, li) for li in range(budget_layers)]
+    shape = (spec.tokens, spec.hidden)
+    x = boundary_tensor("x", 0, 0, shape)
+    dy = boundary_tensor("dy", 0, 0, shape)
+    ro = O.RankOracle(cfg, {0: params}, nm)
+    t0 = time.perf_counter()
+    ro.fwd(0, 0, x)
+    ro.bwd(0, 0, dy)
+    dt = time.perf_counter() - t0
+    n_chunks = len([s for s in range(wl.schedule_kwargs["num_stages"])
+                    if getattr(S, wl.schedule)(**wl.schedule_kwargs).get_mpmd_idx(s) == wl.rank])
+    scale = wl.layers_per_stage * n_chunks * wl.n_mubatches / budget_layers
+    try:
+        import threadpoolctl
+        threads = max((p.get("num_threads", 1) for p in threadpoolctl.threadpool_info()),
+                      default=1)
+    except Exception:
+        threads = os.cpu_count() or 1
+    return {"value": wl.tokens_per_step / (dt * scale), "unit": "tokens/s", "cores": int(threads),
+            "kind": "port",
+            "sample": (f"numpy fp32 oracle, 1 microbatch x {budget_layers} layer "
+                       f"fwd+bwd_i+bwd_w+accumulate = {dt:.2f} s, extrapolated x{scale:g}")}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--unfused-accumulate", action="store_true",
+                    help="bf16 weight gradient + separate fp32 accumulate pass")
+    ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build executes one pipeline rank on one GPU; --gpus > 1 is not "
+              "supported (the other ranks' boundary tensors are synthetic).", file=sys.stderr)
+        sys.exit(2)
+    rt.require_gpu()
+    wl = workloads()[args.workload]
+    wb = Workbench(wl, fused=not args.unfused_accumulate)
+    cls = args.probe or dominant_gemm_class(wl)
+
+    for _ in range(args.warmup):
+        wb.step()
+    rt.sync()
+    start, stop = rt.Event(), rt.Event()
+    with rt.probe(cls) as pr:
+        start.record()
+        for _ in range(args.steps):
+            wb.step()
+        stop.record()
+        stop.sync()
+    rt.sync()
+    ms = start.elapsed_ms(stop) / args.steps
+    tokens = wl.tokens_per_step
+    flops = wb.step_flops()
+    spec = wl.layer
+    rec = {
+        "metric": "stage_tokens_per_sec_fwd_bwd",
+        "value": tokens / (ms * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": (f"{wl.name}: {spec.family} stage, rank {wl.rank} of {wl.schedule}"
+                         f"{wl.schedule_kwargs}, {self_desc(wl, wb)}"),
+            "tokens_per_step": tokens, "n_mubatches": wl.n_mubatches,
+            "layers": wl.layers_per_stage * wb.plan.n_chunks,
+            "peak_live_microbatches": wb.plan.max_live,
+            "fused_wgrad_accumulate": not args.unfused_accumulate,
+            "device_bytes": wb.ex.nbytes,
+        },
+        "algorithmic_flops_per_step": flops,
+        "mfma_peak_frac": flops / (ms * 1e-3) / MFMA_BF16_PEAK,
+    }
+    if pr.launches:
+        avg_ms = pr.total_ms / pr.launches
+        hbm = pr.flops == 0
+        ach = (pr.bytes if hbm else pr.flops) / (pr.total_ms * 1e-3)
+        rec["roofline"] = {
+            "kernel": cls, "bound": "hbm" if hbm else "mfma",
+            "achieved": ach / (1e9 if hbm else 1e12),
+            "peak": (HBM_PEAK / 1e9) if hbm else (MFMA_BF16_PEAK / 1e12),
+            "unit": "GB/s" if hbm else "TFLOP/s",
+            "frac": ach / (HBM_PEAK if hbm else MFMA_BF16_PEAK),
+            "traffic": None,
+            "launches": pr.launches, "avg_launch_ms": avg_ms,
+            "algorithmic_per_launch": (pr.bytes if hbm else pr.flops) / pr.launches,
+        }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(rec))
+
+
+def self_desc(wl, wb) -> str:
+    s = wl.layer
+    return (f"{wl.layers_per_stage} layers x {wb.plan.n_chunks} chunk(s), hidden {s.hidden}, "
+            f"heads {s.n_heads}/{s.kvh}, ffn {s.ffn}, seq {s.seq}, microbatch {s.batch}, "
+            f"{wl.n_mubatches} microbatches")
+
+
+if __name__ == "__main__":
+    main()

@@ -65,6 +65,19 @@ int jpp_event_sync(void* event);
 int jpp_event_elapsed_ms(void* start, void* stop, float* ms);
 int jpp_mem_info(size_t* free_bytes, size_t* total_bytes);
 
+/* ---- launch probe: per-kernel timings, the counterpart of the reference's
+ * collect_task_times_ms (src/jaxpp/jax_primitives.py:742-773) at kernel
+ * granularity.  Between begin and end every launch of the named kernel class
+ * is bracketed by HIP events on the stream it is launched on; end waits for
+ * them and returns the number of launches, their summed duration and the
+ * algorithmic FLOPs / HBM bytes the launchers declared.  Class names:
+ *   gemm_<nn|nt|tn>_<bf16|gelu|dgelu|accf32|f32>_<BM>x<BN>   (nn: y = x W,
+ *       nt: dx = dy W^T, tn: dW = x^T dy)
+ *   attn_fwd, attn_bwd_dq, attn_bwd_dkv, norm_fwd, norm_bwd, swiglu_fwd,
+ *   swiglu_bwd, rope, grad_accum, colsum */
+int jpp_probe_begin(const char* kernel_class);
+int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, double* total_bytes);
+
 /* ---- GEMM: stands in for the `dot_general`s of a stage task ----------------
  * C[M,N] = epilogue( sum_k Aop[m,k] * Bop[n,k] ), bf16 operands, fp32 MFMA
  * accumulation.

@@ -5,8 +5,37 @@
 
 #include "common.h"
 
+#include <string>
+#include <utility>
+#include <vector>
+
 namespace {
 thread_local char g_err[1024] = "";
+
+struct Probe {
+  bool active = false;
+  std::string cls;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> events;
+  hipEvent_t open_ev = nullptr;
+  double flops = 0, bytes = 0;
+} g_probe;
+}  // namespace
+
+bool jpp_probe_wants(const char* kernel_class) {
+  return g_probe.active && g_probe.cls == kernel_class;
+}
+void jpp_probe_open(hipStream_t stream) {
+  hipEventCreate(&g_probe.open_ev);
+  hipEventRecord(g_probe.open_ev, stream);
+}
+void jpp_probe_close(hipStream_t stream, double flops, double bytes) {
+  hipEvent_t stop;
+  hipEventCreate(&stop);
+  hipEventRecord(stop, stream);
+  g_probe.events.emplace_back(g_probe.open_ev, stop);
+  g_probe.open_ev = nullptr;
+  g_probe.flops += flops;
+  g_probe.bytes += bytes;
 }
 
 int jpp_set_error(int code, const char* fmt, ...) {
@@ -100,6 +129,37 @@ int jpp_event_sync(void* event) {
 int jpp_event_elapsed_ms(void* start, void* stop, float* ms) {
   JPP_REQUIRE(ms, "event_elapsed: null");
   JPP_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return JPP_OK;
+}
+int jpp_probe_begin(const char* kernel_class) {
+  JPP_REQUIRE(kernel_class && *kernel_class, "probe_begin: empty class name");
+  JPP_REQUIRE(!g_probe.active, "probe_begin: a probe is already active");
+  g_probe.active = true;
+  g_probe.cls = kernel_class;
+  g_probe.flops = g_probe.bytes = 0;
+  return JPP_OK;
+}
+int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, double* total_bytes) {
+  JPP_REQUIRE(g_probe.active, "probe_end: no active probe");
+  g_probe.active = false;
+  double ms = 0;
+  hipError_t err = hipSuccess;
+  for (auto& ev : g_probe.events) {
+    float t = 0;
+    hipError_t e = hipEventSynchronize(ev.second);
+    if (e == hipSuccess) e = hipEventElapsedTime(&t, ev.first, ev.second);
+    if (e != hipSuccess) err = e;
+    ms += t;
+    hipEventDestroy(ev.first);
+    hipEventDestroy(ev.second);
+  }
+  if (launches) *launches = (int64_t)g_probe.events.size();
+  if (total_ms) *total_ms = ms;
+  if (total_flops) *total_flops = g_probe.flops;
+  if (total_bytes) *total_bytes = g_probe.bytes;
+  g_probe.events.clear();
+  if (err != hipSuccess)
+    return jpp_set_error(JPP_ERR_HIP, "probe_end: %s", hipGetErrorString(err));
   return JPP_OK;
 }
 int jpp_mem_info(size_t* free_bytes, size_t* total_bytes) {

@@ -515,6 +515,9 @@ extern "C" int jpp_attn_fwd(void* stream, const jpp_attn_args* a) {
   AttnParams p = make_params(a);
   dim3 grid(a->seq / 128, a->n_heads, a->batch);
   hipStream_t st = (hipStream_t)stream;
+  const double fl = 4.0 * a->batch * a->seq * (double)a->seq * a->n_heads * a->head_dim *
+                    (a->causal ? 0.5 : 1.0);
+  ProbeScope probe(st, "attn_fwd", fl, 0);
 #define JPP_AF(D_, C_) hipLaunchKernelGGL((attn_fwd_kernel<D_, C_>), grid, dim3(256), 0, st, p)
   if (a->head_dim == 64) { if (a->causal) JPP_AF(64, true); else JPP_AF(64, false); }
   else { if (a->causal) JPP_AF(128, true); else JPP_AF(128, false); }
@@ -540,10 +543,16 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
   dim3 gdelta((unsigned)((items + 255) / 256));
   dim3 gq(a->seq / 128, a->n_heads, a->batch);
   dim3 gkv(a->seq / 128, a->n_kv_heads, a->batch);
+  const double fl = 8.0 * a->batch * a->seq * (double)a->seq * a->n_heads * a->head_dim *
+                    (a->causal ? 0.5 : 1.0);
 #define JPP_AB(D_, C_)                                                             \
   do {                                                                             \
     hipLaunchKernelGGL((attn_delta_kernel<D_>), gdelta, dim3(256), 0, st, p);      \
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, C_>), gq, dim3(256), 0, st, p);     \
+    {                                                                              \
+      ProbeScope probe(st, "attn_bwd_dq", fl * 0.4, 0);                            \
+      hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, C_>), gq, dim3(256), 0, st, p);   \
+    }                                                                              \
+    ProbeScope probe(st, "attn_bwd_dkv", fl * 0.6, 0);                             \
     JPP_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<D_, C_>,    \
                                       hipFuncAttributeMaxDynamicSharedMemorySize,  \
                                       4 * D_ * 128 + 512));                        \

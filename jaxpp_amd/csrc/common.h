@@ -36,6 +36,27 @@ int jpp_set_error(int code, const char* fmt, ...);
                            hipGetErrorString(e_), __FILE__, __LINE__);          \
   } while (0)
 
+// -- launch probe -------------------------------------------------------------
+// While a probe is active (jpp_probe_begin), every launch whose class name
+// matches is bracketed by HIP events on its own stream; jpp_probe_end sums the
+// durations and the algorithmic work the launcher declared.
+bool jpp_probe_wants(const char* kernel_class);
+void jpp_probe_open(hipStream_t stream);
+void jpp_probe_close(hipStream_t stream, double flops, double bytes);
+
+struct ProbeScope {
+  hipStream_t stream;
+  double flops, bytes;
+  bool on;
+  ProbeScope(hipStream_t s, const char* cls, double fl, double by)
+      : stream(s), flops(fl), bytes(by), on(jpp_probe_wants(cls)) {
+    if (on) jpp_probe_open(stream);
+  }
+  ~ProbeScope() {
+    if (on) jpp_probe_close(stream, flops, bytes);
+  }
+};
+
 // -- bf16 <-> f32 -------------------------------------------------------------
 __device__ __forceinline__ float bf16_to_f32(bf16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);

@@ -407,6 +407,7 @@ int jpp_norm_fwd(void* stream, const jpp_norm_args* a) {
               8 * 64 * kMaxChunksPerLane, (long)a->cols);
   JPP_REQUIRE((a->beta == nullptr) == (a->mean == nullptr),
               "norm_fwd: beta and mean are both given (LayerNorm) or both NULL (RMSNorm)");
+  ProbeScope probe((hipStream_t)stream, "norm_fwd", 0, 4.0 * a->rows * a->cols);
   return a->beta ? launch_norm_fwd<true>((hipStream_t)stream, a)
                  : launch_norm_fwd<false>((hipStream_t)stream, a);
 }
@@ -420,12 +421,14 @@ int jpp_norm_bwd(void* stream, const jpp_norm_args* a) {
               8 * 64 * kMaxChunksPerLane, (long)a->cols);
   const bool ln = a->mean != nullptr;
   JPP_REQUIRE(!ln || a->dbeta, "norm_bwd: LayerNorm needs dbeta");
+  ProbeScope probe((hipStream_t)stream, "norm_bwd", 0, (a->resid ? 8.0 : 6.0) * a->rows * a->cols);
   return ln ? launch_norm_bwd<true>((hipStream_t)stream, a)
             : launch_norm_bwd<false>((hipStream_t)stream, a);
 }
 
 int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f) {
   JPP_REQUIRE(gu && s && rows > 0 && f > 0 && f % 8 == 0, "swiglu_fwd: bad arguments");
+  ProbeScope probe((hipStream_t)stream, "swiglu_fwd", 0, 6.0 * rows * f);
   hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid_for(rows * (f / 8))), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)gu, (bf16_t*)s, (long)rows, (int)f);
   JPP_LAUNCH_CHECK();
@@ -435,6 +438,7 @@ int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t 
 int jpp_swiglu_bwd(void* stream, const void* gu, const void* ds, void* dgu, int64_t rows,
                    int64_t f) {
   JPP_REQUIRE(gu && ds && dgu && rows > 0 && f > 0 && f % 8 == 0, "swiglu_bwd: bad arguments");
+  ProbeScope probe((hipStream_t)stream, "swiglu_bwd", 0, 10.0 * rows * f);
   hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid_for(rows * (f / 8))), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)gu, (const bf16_t*)ds, (bf16_t*)dgu,
                      (long)rows, (int)f);
@@ -449,6 +453,7 @@ int jpp_rope(void* stream, void* x, int64_t ld, const float* cos_tab, const floa
                   ld >= (int64_t)n_rot_heads * head_dim,
               "rope: bad shape");
   const long rows = (long)batch * seq;
+  ProbeScope probe((hipStream_t)stream, "rope", 0, 4.0 * rows * n_rot_heads * head_dim);
   hipLaunchKernelGGL(rope_kernel, dim3(grid_for(rows * n_rot_heads * (head_dim / 16))), dim3(256),
                      0, (hipStream_t)stream, (bf16_t*)x, (long)ld, cos_tab, sin_tab, rows, seq,
                      n_rot_heads, head_dim, inverse);
@@ -461,6 +466,7 @@ int jpp_grad_accum_f32(void* stream, float* acc, const void* g, int64_t count, i
   JPP_REQUIRE((uintptr_t)acc % 16 == 0 && (uintptr_t)g % 16 == 0,
               "grad_accum: operands must be 16-byte aligned");
   if (count == 0) return JPP_OK;
+  ProbeScope probe((hipStream_t)stream, "grad_accum", 0, (g_is_f32 ? 12.0 : 10.0) * count);
   const long n8 = count / 8;
   hipStream_t st = (hipStream_t)stream;
   if (n8) {
@@ -487,6 +493,7 @@ int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int6
                   ld >= cols,
               "colsum: bad arguments");
   hipStream_t st = (hipStream_t)stream;
+  ProbeScope probe(st, "colsum", 0, 2.0 * rows * cols);
   const int nb = (int)(rows < JPP_NORM_PARTIALS ? rows : JPP_NORM_PARTIALS);
   const int panels = (int)((cols / 8 + 255) / 256);
   hipLaunchKernelGGL(colsum_partial_kernel, dim3(nb, panels), dim3(256), 0, st, (const bf16_t*)x,

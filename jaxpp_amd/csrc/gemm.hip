@@ -15,6 +15,7 @@
 // the "B" port, so a lane ends up holding 4 consecutive n for one m and the
 // epilogue writes 8-byte (bf16) or 16-byte (f32) runs.
 #include <math.h>
+#include <stdio.h>
 
 #include "common.h"
 
@@ -183,8 +184,23 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 }
 
 template <int BM, int BN, bool TA, bool TB, int EPI>
+const char* class_name() {
+  static char name[64] = "";
+  if (!name[0]) {
+    const char* lay = TA ? "tn" : (TB ? "nn" : "nt");
+    const char* epi = EPI == JPP_EPI_BF16 ? "bf16" : EPI == JPP_EPI_GELU ? "gelu"
+                    : EPI == JPP_EPI_DGELU ? "dgelu" : EPI == JPP_EPI_ACC_F32 ? "accf32" : "f32";
+    snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d", lay, epi, BM, BN);
+  }
+  return name;
+}
+
+template <int BM, int BN, bool TA, bool TB, int EPI>
 int launch(hipStream_t stream, GemmParams& p) {
   constexpr int SMEM = 2 * (BM + BN) * 128;
+  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI>(), 2.0 * p.m * p.n * p.k,
+                   2.0 * ((double)p.m * p.k + (double)p.n * p.k) +
+                       (double)p.m * p.n * (EPI == JPP_EPI_ACC_F32 ? 8 : EPI == JPP_EPI_F32 ? 4 : 2));
   auto kern = gemm_kernel<BM, BN, TA, TB, EPI>;
   static bool configured = false;  // per instantiation; attribute is sticky
   if (!configured) {

@@ -76,7 +76,7 @@ EXPORTS = [
     "jpp_free", "jpp_memcpy_h2d", "jpp_memcpy_d2h", "jpp_memcpy_d2d_async", "jpp_fill_u32",
     "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_device_sync",
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
-    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
+    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
     "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
@@ -117,6 +117,9 @@ def load():
     lib.jpp_event_sync.argtypes = [C.c_void_p]
     lib.jpp_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
     lib.jpp_mem_info.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    lib.jpp_probe_begin.argtypes = [C.c_char_p]
+    lib.jpp_probe_end.argtypes = [C.POINTER(C.c_int64), C.POINTER(C.c_double),
+                                  C.POINTER(C.c_double), C.POINTER(C.c_double)]
     lib.jpp_gemm_bf16.argtypes = [C.c_void_p, C.POINTER(GemmArgs)]
     lib.jpp_attn_fwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
@@ -266,6 +269,27 @@ class Event:
                 load().jpp_event_destroy(self.ptr)
         except Exception:
             pass
+
+
+class probe:
+    """Times every launch of one kernel class with HIP events on the launch
+    stream (reference: ``collect_task_times_ms``,
+    src/jaxpp/jax_primitives.py:742-773).  After the ``with`` block:
+    ``launches``, ``total_ms``, ``flops``, ``bytes``."""
+
+    def __init__(self, kernel_class: str):
+        self.kernel_class = kernel_class
+        self.launches, self.total_ms, self.flops, self.bytes = 0, 0.0, 0.0, 0.0
+
+    def __enter__(self):
+        check(load().jpp_probe_begin(self.kernel_class.encode()))
+        return self
+
+    def __exit__(self, *exc):
+        n, ms, fl, by = C.c_int64(), C.c_double(), C.c_double(), C.c_double()
+        check(load().jpp_probe_end(C.byref(n), C.byref(ms), C.byref(fl), C.byref(by)))
+        self.launches, self.total_ms, self.flops, self.bytes = n.value, ms.value, fl.value, by.value
+        return False
 
 
 # ---------------------------------------------------------------------------
