@@ -164,3 +164,81 @@ struct TileLoader {
     }
   }
 };
+
+// ---------------------------------------------------------------------------
+// Direct-to-LDS tiles (global_load_lds_dwordx4): no register staging.
+// A wave-level load moves 64 x 16 bytes from per-lane global addresses into
+// 1 KiB of LDS in lane order, so the LDS image of a tile is its memory image
+// with the 16-byte chunks permuted inside each KiB.
+//
+//   MC = false  memory [ROWS][64..], contraction index contiguous.  LDS image
+//               is the swizzled slab read by slab_frag().
+//   MC = true   memory [64][ROWS..], contraction index is the slow one.  LDS
+//               image keeps that orientation, chunk c of row k stored at
+//               c ^ ((k & 3) << 2); fragments come out through the LDS
+//               transpose read (ds_read_b64_tr_b16), which hands lane i of a
+//               16-lane group the column i of a 4 x 16 block.
+// ---------------------------------------------------------------------------
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+#define JPP_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define JPP_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+// One wave-level direct-to-LDS load.  Issued through inline assembly so that the
+// compiler does not serialise later LDS reads of *other* stages behind it; the
+// caller waits for completion itself (vmcnt) before the data is read.
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)p;
+}
+__device__ __forceinline__ void dma_load16(const bf16_t* g, uint32_t lds_addr) {
+  const uint32_t addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(addr), "v"(g)
+               : "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+template <int ROWS, bool MC>
+struct DmaTile {
+  static constexpr int BYTES = ROWS * 128;
+  static constexpr int INSTS = ROWS / 32;  // wave-level loads per wave (4 waves share a tile)
+
+  // `tile` is the LDS byte address (lds_address()) of the tile's first byte
+  static __device__ __forceinline__ void issue(const bf16_t* __restrict__ src, long ld,
+                                               uint32_t tile, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < INSTS; ++i) {
+      const int inst = wave * INSTS + i;
+      const bf16_t* g;
+      if constexpr (!MC) {
+        const int row = inst * 8 + (lane >> 3);
+        g = src + (long)row * ld + (((lane & 7) ^ slab_swz(row)) << 3);
+      } else {
+        constexpr int CPR = ROWS / 8, RPI = 64 / CPR;
+        const int k = inst * RPI + lane / CPR;
+        g = src + (long)k * ld + ((((lane % CPR) ^ ((k & 3) << 2))) << 3);
+      }
+      dma_load16(g, tile + inst * 1024);
+    }
+  }
+
+  // MFMA operand fragment: rows row0 .. row0+31 of the operand, K-step ks
+  static __device__ __forceinline__ bf16x8 frag(const uint8_t* tile, int row0, int ks, int lane) {
+    if constexpr (!MC) {
+      return slab_frag(tile, row0, ks, lane);
+    } else {
+      const int g = lane >> 4, s = lane & 15;
+      const int n = row0 + ((g & 1) << 4) + ((s & 3) << 2);
+      const int kq = s >> 2;  // == k & 3
+      const int k = ks * 16 + ((g >> 1) << 3) + kq;
+      const uint8_t* p = tile + k * (ROWS * 2) + ((((n >> 3) ^ (kq << 2))) << 4) + ((n & 7) << 1);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)JPP_LDS_PTR(p));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) s16x4*)JPP_LDS_PTR(p + 4 * ROWS * 2));
+      const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, v);
+    }
+  }
+};

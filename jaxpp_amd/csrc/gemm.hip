@@ -72,9 +72,11 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm,
 
 template <int BM, int BN, bool TA, bool TB, int EPI>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
-  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  using TileA = DmaTile<BM, TA>;
+  using TileB = DmaTile<BN, TB>;
+  constexpr int A_BYTES = TileA::BYTES, STAGE = TileA::BYTES + TileB::BYTES;
   constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 MFMA tiles per wave
-  extern __shared__ __align__(16) uint8_t smem[];
+  extern __shared__ __align__(1024) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -87,11 +89,6 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   const long a_step = TA ? 64 * p.lda : 64;
   const long b_step = TB ? 64 * p.ldb : 64;
 
-  using LA = TileLoader<BM, TA>;
-  using LB = TileLoader<BN, TB>;
-  typename LA::Regs ra;
-  typename LB::Regs rb;
-
   f32x16 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -101,35 +98,40 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int kt_n = p.k / 64;
-  LA::load(ra, a_src, p.lda, tid);
-  LB::load(rb, b_src, p.ldb, tid);
-  LA::store(ra, smem, tid);
-  LB::store(rb, smem + A_BYTES, tid);
+  const uint32_t lds0 = lds_address(smem);
+  TileA::issue(a_src, p.lda, lds0, wave, lane);
+  TileB::issue(b_src, p.ldb, lds0 + A_BYTES, wave, lane);
+  dma_wait_all();
   __syncthreads();
 
   for (int kt = 0; kt < kt_n; ++kt) {
     const uint8_t* sa = smem + (kt & 1) * STAGE;
     const uint8_t* sb = sa + A_BYTES;
-    // fetch the next K-step (the last iteration re-reads its own, unused)
-    const int kn = min(kt + 1, kt_n - 1);
-    LA::load(ra, a_src + (long)kn * a_step, p.lda, tid);
-    LB::load(rb, b_src + (long)kn * b_step, p.ldb, tid);
+    // The other stage was last read one iteration ago (barrier below): start
+    // filling it with the next K-step straight from HBM while this one is
+    // multiplied.  The last iteration re-reads its own step, unused.
+    {
+      const int kn = min(kt + 1, kt_n - 1);
+      const uint32_t da = lds0 + ((kt + 1) & 1) * STAGE;
+      TileA::issue(a_src + (long)kn * a_step, p.lda, da, wave, lane);
+      TileB::issue(b_src + (long)kn * b_step, p.ldb, da + A_BYTES, wave, lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       bf16x8 fw[TN], fx[TM];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fw[j] = slab_frag(sb, wn * (BN / 2) + j * 32, ks, lane);
+      for (int j = 0; j < TN; ++j) fw[j] = TileB::frag(sb, wn * (BN / 2) + j * 32, ks, lane);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fx[i] = slab_frag(sa, wm * (BM / 2) + i * 32, ks, lane);
+      for (int i = 0; i < TM; ++i) fx[i] = TileA::frag(sa, wm * (BM / 2) + i * 32, ks, lane);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fx[i], acc[i][j], 0, 0, 0);
     }
-    uint8_t* da = smem + ((kt + 1) & 1) * STAGE;
-    LA::store(ra, da, tid);
-    LB::store(rb, da + A_BYTES, tid);
+    __builtin_amdgcn_sched_barrier(0);
+    dma_wait_all();
     __syncthreads();
   }
 
