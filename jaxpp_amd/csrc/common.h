@@ -184,17 +184,26 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 #define JPP_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define JPP_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-// One wave-level direct-to-LDS load.  Issued through inline assembly so that the
-// compiler does not serialise later LDS reads of *other* stages behind it; the
-// caller waits for completion itself (vmcnt) before the data is read.
+// One wave-level direct-to-LDS load: 64 lanes x 16 bytes from `base + off`
+// (uniform 64-bit base, per-lane 32-bit byte offset) to LDS bytes
+// [lds_addr, lds_addr + 1024) in lane order.  Issued through inline assembly
+// so that the compiler does not serialise LDS reads of the *other* stage
+// behind it; the caller waits for completion itself (dma_wait_all) before the
+// data is read.
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)p;
 }
-__device__ __forceinline__ void dma_load16(const bf16_t* g, uint32_t lds_addr) {
-  const uint32_t addr = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+__device__ __forceinline__ const bf16_t* uniform_ptr(const bf16_t* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const bf16_t*)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ void dma_load16(const bf16_t* base, uint32_t off, uint32_t lds_addr) {
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(addr), "v"(g)
+               : "s"(lds_addr), "v"(off), "s"(base)
                : "memory");
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -203,24 +212,32 @@ template <int ROWS, bool MC>
 struct DmaTile {
   static constexpr int BYTES = ROWS * 128;
   static constexpr int INSTS = ROWS / 32;  // wave-level loads per wave (4 waves share a tile)
+  typedef uint32_t Offsets[INSTS];
 
-  // `tile` is the LDS byte address (lds_address()) of the tile's first byte
-  static __device__ __forceinline__ void issue(const bf16_t* __restrict__ src, long ld,
-                                               uint32_t tile, int wave, int lane) {
+  // per-lane byte offsets (from the tile's first element) of this wave's loads;
+  // loop invariant
+  static __device__ __forceinline__ void offsets(Offsets& off, long ld, int wave, int lane) {
 #pragma unroll
     for (int i = 0; i < INSTS; ++i) {
       const int inst = wave * INSTS + i;
-      const bf16_t* g;
       if constexpr (!MC) {
         const int row = inst * 8 + (lane >> 3);
-        g = src + (long)row * ld + (((lane & 7) ^ slab_swz(row)) << 3);
+        off[i] = (uint32_t)(((long)row * ld + (((lane & 7) ^ slab_swz(row)) << 3)) * 2);
       } else {
         constexpr int CPR = ROWS / 8, RPI = 64 / CPR;
         const int k = inst * RPI + lane / CPR;
-        g = src + (long)k * ld + ((((lane % CPR) ^ ((k & 3) << 2))) << 3);
+        off[i] = (uint32_t)(((long)k * ld + ((((lane % CPR) ^ ((k & 3) << 2))) << 3)) * 2);
       }
-      dma_load16(g, tile + inst * 1024);
     }
+  }
+
+  // loads FIRST .. FIRST+COUNT-1 of this wave's share; `tile` = LDS byte address
+  template <int FIRST, int COUNT>
+  static __device__ __forceinline__ void issue(const bf16_t* src, const Offsets& off,
+                                               uint32_t tile, int wave) {
+#pragma unroll
+    for (int i = FIRST; i < FIRST + COUNT; ++i)
+      dma_load16(src, off[i], tile + (wave * INSTS + i) * 1024);
   }
 
   // MFMA operand fragment: rows row0 .. row0+31 of the operand, K-step ks

@@ -99,38 +99,54 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
   const int kt_n = p.k / 64;
   const uint32_t lds0 = lds_address(smem);
-  TileA::issue(a_src, p.lda, lds0, wave, lane);
-  TileB::issue(b_src, p.ldb, lds0 + A_BYTES, wave, lane);
+  typename TileA::Offsets offa;
+  typename TileB::Offsets offb;
+  TileA::offsets(offa, p.lda, wave, lane);
+  TileB::offsets(offb, p.ldb, wave, lane);
+  constexpr int IA = TileA::INSTS, IB = TileB::INSTS;
+  TileA::template issue<0, IA>(uniform_ptr(a_src), offa, lds0, wave);
+  TileB::template issue<0, IB>(uniform_ptr(b_src), offb, lds0 + A_BYTES, wave);
   dma_wait_all();
   __syncthreads();
 
   for (int kt = 0; kt < kt_n; ++kt) {
     const uint8_t* sa = smem + (kt & 1) * STAGE;
     const uint8_t* sb = sa + A_BYTES;
-    // The other stage was last read one iteration ago (barrier below): start
-    // filling it with the next K-step straight from HBM while this one is
+    // The other stage was last read one iteration ago (barrier below): it is
+    // refilled with the next K-step straight from HBM while this one is
     // multiplied.  The last iteration re-reads its own step, unused.
-    {
-      const int kn = min(kt + 1, kt_n - 1);
-      const uint32_t da = lds0 + ((kt + 1) & 1) * STAGE;
-      TileA::issue(a_src + (long)kn * a_step, p.lda, da, wave, lane);
-      TileB::issue(b_src + (long)kn * b_step, p.ldb, da + A_BYTES, wave, lane);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    const int kn = min(kt + 1, kt_n - 1);
+    const uint32_t da = lds0 + ((kt + 1) & 1) * STAGE;
+    const bf16_t* ga = uniform_ptr(a_src + (long)kn * a_step);
+    const bf16_t* gb = uniform_ptr(b_src + (long)kn * b_step);
+
+    bf16x8 fw[2][TN], fx[2][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag(sb, wn * (BN / 2) + j * 32, 0, lane);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fx[0][i] = TileA::frag(sa, wm * (BM / 2) + i * 32, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      bf16x8 fw[TN], fx[TM];
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks < 3) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fw[j] = TileB::frag(sb, wn * (BN / 2) + j * 32, ks, lane);
+        for (int j = 0; j < TN; ++j)
+          fw[nxt][j] = TileB::frag(sb, wn * (BN / 2) + j * 32, ks + 1, lane);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fx[i] = TileA::frag(sa, wm * (BM / 2) + i * 32, ks, lane);
+        for (int i = 0; i < TM; ++i)
+          fx[nxt][i] = TileA::frag(sa, wm * (BM / 2) + i * 32, ks + 1, lane);
+      }
+      // the HBM -> LDS loads of the next K-step go out under the first two
+      // MFMA blocks, leaving them the rest of the iteration to land
+      if (ks == 0) TileA::template issue<0, IA>(ga, offa, da, wave);
+      if (ks == 1) TileB::template issue<0, IB>(gb, offb, da + A_BYTES, wave);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fx[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cur][j], fx[cur][i], acc[i][j],
+                                                              0, 0, 0);
     }
-    __builtin_amdgcn_sched_barrier(0);
     dma_wait_all();
     __syncthreads();
   }
