@@ -50,23 +50,36 @@ __device__ __forceinline__ bf16x8 global_frag(const bf16_t* base, long ld, int k
   return *(const bf16x8*)(base + (long)(lane & 31) * ld + ks * 16 + (lane >> 5) * 8);
 }
 
+// a [64][D] tile lives in LDS as D/64 slabs of [64][64]
 template <int D>
-__device__ __forceinline__ bf16x8 slabs_frag(const uint8_t* slabs, int rows_per_slab, int row0,
-                                             int ks, int lane) {
-  // a [rows][D] operand is held as D/64 slabs of [rows][64]
-  return slab_frag(slabs + (ks >> 2) * rows_per_slab * 128, row0, ks & 3, lane);
+__device__ __forceinline__ bf16x8 slabs_frag(const uint8_t* slabs, int row0, int ks, int lane) {
+  return slab_frag(slabs + (ks >> 2) * 8192, row0, ks & 3, lane);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// HBM -> LDS copy of a [64][D] tile (row stride ld) by the 4 waves of a
+// workgroup, as D/64 swizzled slabs; no registers involved.
+using Tile64 = DmaTile<64, false>;
+template <int D>
+__device__ __forceinline__ void dma_tile(const bf16_t* src, const Tile64::Offsets& off,
+                                         uint32_t lds, int wave) {
+#pragma unroll
+  for (int c = 0; c < D / 64; ++c)
+    Tile64::issue<0, Tile64::INSTS>(uniform_ptr(src + c * 64), off, lds + c * 8192, wave);
 }
 
 // ---------------------------------------------------------------------------
-// forward
+// forward: one workgroup per 128 queries of one head, 32 queries per wave;
+// K/V blocks of 64 keys double-buffered in LDS
 // ---------------------------------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   constexpr int KS = D / 16;  // MFMA steps over the head dimension
   constexpr int DT = D / 32;  // output tiles over the head dimension
-  constexpr int NSLAB = D / 64;
-  __shared__ __align__(16) uint8_t lds_k[NSLAB * 64 * 128];
-  __shared__ __align__(16) uint8_t lds_vt[D * 128];
+  constexpr int TILE = D * 128;  // bytes of a [64][D] tile
+  constexpr int STAGE = 2 * TILE;
+  extern __shared__ __align__(1024) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int qb = CAUSAL ? (gridDim.x - 1 - blockIdx.x) : blockIdx.x;  // heavy blocks first
@@ -88,85 +101,90 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
   for (int i = 0; i < DT; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;  // running max of the raw scores, running sum
   const float sc = p.scale * kLog2e;
 
-  using LK = TileLoader<64, false>;
-  using LV = TileLoader<D, true, true>;
-  typename LK::Regs rk[NSLAB];
-  typename LV::Regs rv;
   const bf16_t* kbase = p.k + row0 * p.ldk + hk * D;
   const bf16_t* vbase = p.v + row0 * p.ldv + hk * D;
   const int nblk = CAUSAL ? (qb * 128 + 128) / 64 : p.seq / 64;
+  Tile64::Offsets offk, offv;
+  Tile64::offsets(offk, p.ldk, wave, lane);
+  Tile64::offsets(offv, p.ldv, wave, lane);
+  const uint32_t lds0 = lds_address(smem);
 
-#pragma unroll
-  for (int c = 0; c < NSLAB; ++c) LK::load(rk[c], kbase + c * 64, p.ldk, tid);
-  LV::load(rv, vbase, p.ldv, tid);
+  dma_tile<D>(kbase, offk, lds0, wave);
+  dma_tile<D>(vbase, offv, lds0 + TILE, wave);
+  dma_wait_all();
+  __syncthreads();
 
   for (int blk = 0; blk < nblk; ++blk) {
     const int k0 = blk * 64;
-    if (blk) __syncthreads();
-#pragma unroll
-    for (int c = 0; c < NSLAB; ++c) LK::store(rk[c], lds_k + c * 64 * 128, tid);
-    LV::store(rv, lds_vt, tid);
-    __syncthreads();
+    const uint8_t* lds_k = smem + (blk & 1) * STAGE;
+    const uint8_t* lds_v = lds_k + TILE;
     {
-      const int kn = min(blk + 1, nblk - 1) * 64;
-#pragma unroll
-      for (int c = 0; c < NSLAB; ++c) LK::load(rk[c], kbase + (long)kn * p.ldk + c * 64, p.ldk, tid);
-      LV::load(rv, vbase + (long)kn * p.ldv, p.ldv, tid);
+      const long kn = (long)min(blk + 1, nblk - 1) * 64;
+      const uint32_t dst = lds0 + ((blk + 1) & 1) * STAGE;
+      dma_tile<D>(kbase + kn * p.ldk, offk, dst, wave);
+      dma_tile<D>(vbase + kn * p.ldv, offv, dst + TILE, wave);
     }
-    if (CAUSAL && k0 > q0 + 31) continue;  // whole block above this wave's diagonal
-
-    f32x16 s[2];
+    if (!(CAUSAL && k0 > q0 + 31)) {  // else: whole block above this wave's diagonal
+      f32x16 s[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < 2; ++t) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+        for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_k, 64, t * 32, ks, lane),
-                                                       qf[ks], s[t], 0, 0, 0);
-    }
-    float mx = -INFINITY;
+        for (int ks = 0; ks < KS; ++ks)
+          s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_k, t * 32, ks, lane),
+                                                         qf[ks], s[t], 0, 0, 0);
+      }
+      if (CAUSAL && k0 + 63 > q0) {  // block touches the diagonal
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float v = s[t][r] * sc;
-        if (CAUSAL) {
-          const int key = k0 + t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-          if (key > qi) v = -INFINITY;
+          for (int r = 0; r < 16; ++r) {
+            const int key = k0 + t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (key > qi) s[t][r] = -INFINITY;
+          }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run, mx);
+      const float neg = -m_new * sc;
+      float rs = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = fast_exp2(fmaf(s[t][r], sc, neg));
+          s[t][r] = e;
+          rs += e;
         }
-        s[t][r] = v;
-        mx = fmaxf(mx, v);
+      if (__any(m_new != m_run)) {  // rescale only when some row's maximum moved
+        const float alpha = fast_exp2((m_run - m_new) * sc);
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        m_run = m_new;
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = exp2f(m_run - m_new);
-    m_run = m_new;
-    float rs = 0.f;
+      l_run += rs;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int st = 0; st < 4; ++st) {
+        const bf16x8 pf = acc_to_frag(s[st >> 1], (st & 1) * 8);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = exp2f(s[t][r] - m_new);
-        s[t][r] = e;
-        rs += e;
+        for (int i = 0; i < DT; ++i)
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slab_frag_tr(lds_v, 64, i * 32, st, lane),
+                                                            pf, oacc[i], 0, 0, 0);
       }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int i = 0; i < DT; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-#pragma unroll
-    for (int st = 0; st < 4; ++st) {
-      const bf16x8 pf = acc_to_frag(s[st >> 1], (st & 1) * 8);
-#pragma unroll
-      for (int i = 0; i < DT; ++i)
-        oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slab_frag(lds_vt, i * 32, st, lane), pf,
-                                                          oacc[i], 0, 0, 0);
     }
+    dma_wait_all();
+    __syncthreads();
   }
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -181,7 +199,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
           make_uint2(pack_bf16x2(oacc[i][4 * g] * inv, oacc[i][4 * g + 1] * inv),
                      pack_bf16x2(oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv));
     }
-  if (lane < 32) p.lse[((long)b * p.n_heads + h) * p.seq + qi] = m_run * kLn2 + logf(l_tot);
+  if (lane < 32)
+    p.lse[((long)b * p.n_heads + h) * p.seq + qi] = m_run * p.scale + logf(l_tot);
 }
 
 // ---------------------------------------------------------------------------
@@ -219,11 +238,10 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
 // backward, dQ: one workgroup per 128 queries of one head
 // ---------------------------------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnParams p) {
-  constexpr int KS = D / 16, DT = D / 32, NSLAB = D / 64;
-  __shared__ __align__(16) uint8_t lds_k[NSLAB * 64 * 128];
-  __shared__ __align__(16) uint8_t lds_v[NSLAB * 64 * 128];
-  __shared__ __align__(16) uint8_t lds_kt[D * 128];
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
+  constexpr int KS = D / 16, DT = D / 32;
+  constexpr int TILE = D * 128, STAGE = 2 * TILE;
+  extern __shared__ __align__(1024) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int qb = CAUSAL ? (gridDim.x - 1 - blockIdx.x) : blockIdx.x;
@@ -254,74 +272,64 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dqacc[i][r] = 0.f;
 
-  using LK = TileLoader<64, false>;
-  using LT = TileLoader<D, true, true>;
-  typename LK::Regs rk[NSLAB], rv[NSLAB];
-  typename LT::Regs rkt;
   const bf16_t* kbase = p.k + row0 * p.ldk + hk * D;
   const bf16_t* vbase = p.v + row0 * p.ldv + hk * D;
   const int nblk = CAUSAL ? (qb * 128 + 128) / 64 : p.seq / 64;
+  Tile64::Offsets offk, offv;
+  Tile64::offsets(offk, p.ldk, wave, lane);
+  Tile64::offsets(offv, p.ldv, wave, lane);
+  const uint32_t lds0 = lds_address(smem);
 
-#pragma unroll
-  for (int c = 0; c < NSLAB; ++c) {
-    LK::load(rk[c], kbase + c * 64, p.ldk, tid);
-    LK::load(rv[c], vbase + c * 64, p.ldv, tid);
-  }
-  LT::load(rkt, kbase, p.ldk, tid);
+  dma_tile<D>(kbase, offk, lds0, wave);
+  dma_tile<D>(vbase, offv, lds0 + TILE, wave);
+  dma_wait_all();
+  __syncthreads();
 
   for (int blk = 0; blk < nblk; ++blk) {
     const int k0 = blk * 64;
-    if (blk) __syncthreads();
-#pragma unroll
-    for (int c = 0; c < NSLAB; ++c) {
-      LK::store(rk[c], lds_k + c * 64 * 128, tid);
-      LK::store(rv[c], lds_v + c * 64 * 128, tid);
-    }
-    LT::store(rkt, lds_kt, tid);
-    __syncthreads();
+    const uint8_t* lds_k = smem + (blk & 1) * STAGE;
+    const uint8_t* lds_v = lds_k + TILE;
     {
       const long kn = (long)min(blk + 1, nblk - 1) * 64;
-#pragma unroll
-      for (int c = 0; c < NSLAB; ++c) {
-        LK::load(rk[c], kbase + kn * p.ldk + c * 64, p.ldk, tid);
-        LK::load(rv[c], vbase + kn * p.ldv + c * 64, p.ldv, tid);
-      }
-      LT::load(rkt, kbase + kn * p.ldk, p.ldk, tid);
+      const uint32_t dst = lds0 + ((blk + 1) & 1) * STAGE;
+      dma_tile<D>(kbase + kn * p.ldk, offk, dst, wave);
+      dma_tile<D>(vbase + kn * p.ldv, offv, dst + TILE, wave);
     }
-    if (CAUSAL && k0 > q0 + 31) continue;
-
-    f32x16 s[2], dp[2];
+    if (!(CAUSAL && k0 > q0 + 31)) {
+      const bool diag = CAUSAL && k0 + 63 > q0;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < 2; ++t) {  // 32 keys at a time keeps the live scores small
+        f32x16 s, dp;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[t][r] = 0.f; dp[t][r] = 0.f; }
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_k, 64, t * 32, ks, lane),
-                                                       qf[ks], s[t], 0, 0, 0);
-        dp[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_v, 64, t * 32, ks, lane),
-                                                        dof[ks], dp[t], 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float pr = exp2f(s[t][r] * sc - lse2);
-        if (CAUSAL) {
-          const int key = k0 + t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-          if (key > qi) pr = 0.f;
+        for (int ks = 0; ks < KS; ++ks) {
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_k, t * 32, ks, lane),
+                                                      qf[ks], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_v, t * 32, ks, lane),
+                                                       dof[ks], dp, 0, 0, 0);
         }
-        s[t][r] = pr * (dp[t][r] - dlt) * p.scale;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float pr = fast_exp2(fmaf(s[r], sc, -lse2));
+          if (diag) {
+            const int key = k0 + t * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (key > qi) pr = 0.f;
+          }
+          s[r] = pr * (dp[r] - dlt) * p.scale;
+        }
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const bf16x8 dsf = acc_to_frag(s, h2 * 8);
+#pragma unroll
+          for (int i = 0; i < DT; ++i)
+            dqacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                slab_frag_tr(lds_k, 64, i * 32, 2 * t + h2, lane), dsf, dqacc[i], 0, 0, 0);
+        }
       }
-#pragma unroll
-    for (int st = 0; st < 4; ++st) {
-      const bf16x8 dsf = acc_to_frag(s[st >> 1], (st & 1) * 8);
-#pragma unroll
-      for (int i = 0; i < DT; ++i)
-        dqacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slab_frag(lds_kt, i * 32, st, lane), dsf,
-                                                           dqacc[i], 0, 0, 0);
     }
+    dma_wait_all();
+    __syncthreads();
   }
 
   bf16_t* drow = p.dq + (row0 + qi) * p.lddq + h * D;
@@ -340,15 +348,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnParams p) {
 // the query heads that share it and over 64-query blocks
 // ---------------------------------------------------------------------------
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnParams p) {
-  constexpr int KS = D / 16, DT = D / 32, NSLAB = D / 64;
-  extern __shared__ __align__(16) uint8_t dkv_smem[];  // 4 * D * 128 + 512 bytes
-  uint8_t* lds_q = dkv_smem;
-  uint8_t* lds_do = lds_q + D * 128;
-  uint8_t* lds_qt = lds_do + D * 128;
-  uint8_t* lds_dot = lds_qt + D * 128;
-  float* lds_lse = (float*)(lds_dot + D * 128);
-  float* lds_delta = lds_lse + 64;
+__global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(AttnParams p) {
+  constexpr int KS = D / 16, DT = D / 32;
+  constexpr int TILE = D * 128, STAGE = 2 * TILE + 512;
+  extern __shared__ __align__(1024) uint8_t smem[];  // 2 stages: Q tile, dO tile, lse[64], delta[64]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int kb = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
@@ -374,93 +377,108 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnParams p) {
     for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.f; dvacc[i][r] = 0.f; }
   const float sc = p.scale * kLog2e;
 
-  using LR = TileLoader<64, false>;
-  using LT = TileLoader<D, true, true>;
-  typename LR::Regs rq[NSLAB], rdo[NSLAB];
-  typename LT::Regs rqt, rdot;
-  float rstat = 0.f;
-
   const int qblk0 = CAUSAL ? (kb * 128) / 64 : 0;
   const int nqb = p.seq / 64 - qblk0;
   const int iters = grp * nqb;
+  Tile64::Offsets offq, offdo;
+  Tile64::offsets(offq, p.ldq, wave, lane);
+  Tile64::offsets(offdo, p.lddo, wave, lane);
+  const uint32_t lds0 = lds_address(smem);
 
-  auto fetch = [&](int it) {
+  // Q / dO tiles go HBM -> LDS directly; the 64 lse and 64 delta values of a
+  // block travel through one register per thread and are parked in LDS at the
+  // end of the previous iteration, so waiting for them never stalls the tiles.
+  float rstat = 0.f;
+  auto fetch = [&](int it, int stage) {
     const int hh = hk * grp + it / nqb;
     const long q0 = (long)(qblk0 + it % nqb) * 64;
-    const bf16_t* qsrc = p.q + (row0 + q0) * p.ldq + hh * D;
-    const bf16_t* dsrc = p.d_o + (row0 + q0) * p.lddo + hh * D;
-#pragma unroll
-    for (int c = 0; c < NSLAB; ++c) {
-      LR::load(rq[c], qsrc + c * 64, p.ldq, tid);
-      LR::load(rdo[c], dsrc + c * 64, p.lddo, tid);
-    }
-    LT::load(rqt, qsrc, p.ldq, tid);
-    LT::load(rdot, dsrc, p.lddo, tid);
     const long stat = ((long)b * p.n_heads + hh) * p.seq + q0;
     if (tid < 64) rstat = p.lse[stat + tid] * kLog2e;
     else if (tid < 128) rstat = p.delta[stat + tid - 64];
+    const uint32_t dst = lds0 + stage * STAGE;
+    dma_tile<D>(p.q + (row0 + q0) * p.ldq + hh * D, offq, dst, wave);
+    dma_tile<D>(p.d_o + (row0 + q0) * p.lddo + hh * D, offdo, dst + TILE, wave);
+  };
+  auto park = [&](int stage) {
+    float* st = (float*)(smem + stage * STAGE + 2 * TILE);
+    if (tid < 128) st[tid] = rstat;
   };
 
-  fetch(0);
+  fetch(0, 0);
+  park(0);
+  dma_wait_all();
+  __syncthreads();
+
   for (int it = 0; it < iters; ++it) {
     const int q0 = (qblk0 + it % nqb) * 64;
-    if (it) __syncthreads();
+    const uint8_t* lds_q = smem + (it & 1) * STAGE;
+    const uint8_t* lds_do = lds_q + TILE;
+    const float* lds_lse = (const float*)(lds_do + TILE);
+    const float* lds_delta = lds_lse + 64;
+    fetch(min(it + 1, iters - 1), (it + 1) & 1);
+    if (!(CAUSAL && q0 + 63 < k0)) {  // else: every query of the block precedes this wave's keys
+      const bool diag = CAUSAL && q0 < k0 + 31;
+      // TB score tiles (32 queries each) are in flight together: both when the
+      // wave owns the whole register file (independent chains to interleave),
+      // one when two workgroups share a CU.
+      constexpr int TB = D > 64 ? 2 : 1;
 #pragma unroll
-    for (int c = 0; c < NSLAB; ++c) {
-      LR::store(rq[c], lds_q + c * 64 * 128, tid);
-      LR::store(rdo[c], lds_do + c * 64 * 128, tid);
-    }
-    LT::store(rqt, lds_qt, tid);
-    LT::store(rdot, lds_dot, tid);
-    if (tid < 64) lds_lse[tid] = rstat;
-    else if (tid < 128) lds_delta[tid - 64] = rstat;
-    __syncthreads();
-    fetch(min(it + 1, iters - 1));
-    if (CAUSAL && q0 + 63 < k0) continue;  // every query of the block precedes this wave's keys
-
-    f32x16 s[2], dp[2];
+      for (int t0 = 0; t0 < 2; t0 += TB) {
+        f32x16 s[TB], dp[TB];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+        for (int u = 0; u < TB; ++u) {
+          const int t = t0 + u;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[t][r] = 0.f; dp[t][r] = 0.f; }
+          for (int r = 0; r < 16; ++r) { s[u][r] = 0.f; dp[u][r] = 0.f; }
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_q, 64, t * 32, ks, lane),
-                                                       kf[ks], s[t], 0, 0, 0);
-        dp[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_do, 64, t * 32, ks, lane),
-                                                        vf[ks], dp[t], 0, 0, 0);
-      }
-    }
+          for (int ks = 0; ks < KS; ++ks) {
+            s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_q, t * 32, ks, lane),
+                                                           kf[ks], s[u], 0, 0, 0);
+            dp[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_do, t * 32, ks, lane),
+                                                            vf[ks], dp[u], 0, 0, 0);
+          }
+        }
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+        for (int u = 0; u < TB; ++u) {
+          const int t = t0 + u;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int ql = t * 32 + g * 8 + (lane >> 5) * 4;
-        const float4 l4 = *(const float4*)(lds_lse + ql);
-        const float4 d4 = *(const float4*)(lds_delta + ql);
-        const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
-        const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
+          for (int g = 0; g < 4; ++g) {
+            const int ql = t * 32 + g * 8 + (lane >> 5) * 4;
+            const float4 l4 = *(const float4*)(lds_lse + ql);
+            const float4 d4 = *(const float4*)(lds_delta + ql);
+            const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
+            const float dl[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * g + e;
-          float pr = exp2f(s[t][r] * sc - ls[e]);
-          if (CAUSAL && ki > q0 + ql + e) pr = 0.f;
-          s[t][r] = pr;
-          dp[t][r] = pr * (dp[t][r] - dl[e]) * p.scale;
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * g + e;
+              float pr = fast_exp2(fmaf(s[u][r], sc, -ls[e]));
+              if (diag && ki > q0 + ql + e) pr = 0.f;
+              s[u][r] = pr;
+              dp[u][r] = pr * (dp[u][r] - dl[e]) * p.scale;
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < TB; ++u) {
+          const int t = t0 + u;
+#pragma unroll
+          for (int h2 = 0; h2 < 2; ++h2) {
+            const bf16x8 pf = acc_to_frag(s[u], h2 * 8);
+            const bf16x8 dsf = acc_to_frag(dp[u], h2 * 8);
+#pragma unroll
+            for (int i = 0; i < DT; ++i) {
+              dvacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  slab_frag_tr(lds_do, 64, i * 32, 2 * t + h2, lane), pf, dvacc[i], 0, 0, 0);
+              dkacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  slab_frag_tr(lds_q, 64, i * 32, 2 * t + h2, lane), dsf, dkacc[i], 0, 0, 0);
+            }
+          }
         }
       }
-#pragma unroll
-    for (int st = 0; st < 4; ++st) {
-      const bf16x8 pf = acc_to_frag(s[st >> 1], (st & 1) * 8);
-      const bf16x8 dsf = acc_to_frag(dp[st >> 1], (st & 1) * 8);
-#pragma unroll
-      for (int i = 0; i < DT; ++i) {
-        dvacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slab_frag(lds_dot, i * 32, st, lane), pf,
-                                                           dvacc[i], 0, 0, 0);
-        dkacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slab_frag(lds_qt, i * 32, st, lane), dsf,
-                                                           dkacc[i], 0, 0, 0);
-      }
     }
+    park((it + 1) & 1);
+    dma_wait_all();
+    __syncthreads();
   }
 
   bf16_t* dkrow = p.dk + (row0 + ki) * p.lddk + hk * D;
@@ -475,6 +493,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnParams p) {
       *(uint2*)(dvrow + d) = make_uint2(pack_bf16x2(dvacc[i][4 * g], dvacc[i][4 * g + 1]),
                                         pack_bf16x2(dvacc[i][4 * g + 2], dvacc[i][4 * g + 3]));
     }
+}
+
+template <class K>
+int set_smem(K kern, int bytes) {
+  JPP_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    bytes));
+  return JPP_OK;
 }
 
 int check_common(const jpp_attn_args* a, const char* who) {
@@ -518,7 +543,11 @@ extern "C" int jpp_attn_fwd(void* stream, const jpp_attn_args* a) {
   const double fl = 4.0 * a->batch * a->seq * (double)a->seq * a->n_heads * a->head_dim *
                     (a->causal ? 0.5 : 1.0);
   ProbeScope probe(st, "attn_fwd", fl, 0);
-#define JPP_AF(D_, C_) hipLaunchKernelGGL((attn_fwd_kernel<D_, C_>), grid, dim3(256), 0, st, p)
+#define JPP_AF(D_, C_)                                                                  \
+  do {                                                                                  \
+    if (int rc = set_smem(attn_fwd_kernel<D_, C_>, 4 * D_ * 128)) return rc;            \
+    hipLaunchKernelGGL((attn_fwd_kernel<D_, C_>), grid, dim3(256), 4 * D_ * 128, st, p); \
+  } while (0)
   if (a->head_dim == 64) { if (a->causal) JPP_AF(64, true); else JPP_AF(64, false); }
   else { if (a->causal) JPP_AF(128, true); else JPP_AF(128, false); }
 #undef JPP_AF
@@ -545,19 +574,17 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
   dim3 gkv(a->seq / 128, a->n_kv_heads, a->batch);
   const double fl = 8.0 * a->batch * a->seq * (double)a->seq * a->n_heads * a->head_dim *
                     (a->causal ? 0.5 : 1.0);
-#define JPP_AB(D_, C_)                                                             \
-  do {                                                                             \
-    hipLaunchKernelGGL((attn_delta_kernel<D_>), gdelta, dim3(256), 0, st, p);      \
-    {                                                                              \
-      ProbeScope probe(st, "attn_bwd_dq", fl * 0.4, 0);                            \
-      hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, C_>), gq, dim3(256), 0, st, p);   \
-    }                                                                              \
-    ProbeScope probe(st, "attn_bwd_dkv", fl * 0.6, 0);                             \
-    JPP_CHECK_HIP(hipFuncSetAttribute((const void*)attn_bwd_dkv_kernel<D_, C_>,    \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                                      4 * D_ * 128 + 512));                        \
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D_, C_>), gkv, dim3(256),              \
-                       4 * D_ * 128 + 512, st, p);                                 \
+#define JPP_AB(D_, C_)                                                              \
+  do {                                                                              \
+    hipLaunchKernelGGL((attn_delta_kernel<D_>), gdelta, dim3(256), 0, st, p);       \
+    if (int rc = set_smem(attn_bwd_dq_kernel<D_, C_>, 4 * D_ * 128)) return rc;     \
+    if (int rc = set_smem(attn_bwd_dkv_kernel<D_, C_>, 4 * D_ * 128 + 1024)) return rc; \
+    {                                                                               \
+      ProbeScope probe(st, "attn_bwd_dq", fl * 0.4, 0);                             \
+      hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, C_>), gq, dim3(256), 4 * D_ * 128, st, p); \
+    }                                                                               \
+    ProbeScope probe(st, "attn_bwd_dkv", fl * 0.6, 0);                              \
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<D_, C_>), gkv, dim3(256), 4 * D_ * 128 + 1024, st, p); \
   } while (0)
   if (a->head_dim == 64) { if (a->causal) JPP_AB(64, true); else JPP_AB(64, false); }
   else { if (a->causal) JPP_AB(128, true); else JPP_AB(128, false); }

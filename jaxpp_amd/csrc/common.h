@@ -259,3 +259,24 @@ struct DmaTile {
     }
   }
 };
+
+// Fragment of a [rows][64 * nslab] tile held as KC slabs, taken the other way
+// round: operand rows are the tile's columns col0 .. col0+31, the contraction
+// index is the tile's row.  Step `st` covers tile rows 16 st .. 16 st + 15 in
+// the order (4 hh + e, 8 + 4 hh + e), e = 0..3, hh = lane / 32: the order in
+// which 8 consecutive accumulator registers of a 32x32 MFMA tile enumerate
+// their row index, so such registers can be the other operand unchanged.
+__device__ __forceinline__ bf16x8 slab_frag_tr(const uint8_t* slabs, int rows_per_slab, int col0,
+                                               int st, int lane) {
+  const int g = lane >> 4, s = lane & 15;
+  const int n = col0 + ((g & 1) << 4) + ((s & 3) << 2);
+  const int k = st * 16 + ((g >> 1) << 2) + (s >> 2);
+  const uint8_t* slab = slabs + (n >> 6) * rows_per_slab * 128 + ((n & 7) << 1);
+  const int c = (n & 63) >> 3;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s16x4*)JPP_LDS_PTR(slab + slab_off(k, c)));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s16x4*)JPP_LDS_PTR(slab + slab_off(k + 8, c)));
+  const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
