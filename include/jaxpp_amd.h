@@ -168,6 +168,12 @@ int jpp_grad_accum_f32(void* stream, float* acc, const void* g, int64_t count, i
 /* acc[j] += sum_t x[t,j] (bias gradients); partial: f32 [JPP_NORM_PARTIALS*cols]. */
 int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int64_t cols,
                      float* acc, float* partial);
+/* Loss of the last stage as in the reference's examples (README.md:76-78):
+ * loss[0] = scale * mean((out - target)^2) over `count` bf16 elements, and its
+ * cotangent dout = scale * 2 (out - target) / count (bf16).  partial: f32
+ * [JPP_NORM_PARTIALS] scratch; the reduction order is fixed. */
+int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t count, float scale,
+                 float* loss, void* dout, float* partial);
 int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count);
 int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count);
 

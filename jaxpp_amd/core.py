@@ -1,0 +1,413 @@
+"""Driver: ``mpmd_jit_with_loop`` and what it runs.
+
+Reference anchors
+  * ``mpmd_jit_with_loop`` / ``TraceableFunction`` - src/jaxpp/core.py:3892-3923,
+    :3151-3259: a decorator taking the MPMD mesh; the object it returns has
+    ``compile(*args)`` and ``__call__``.
+  * clustering the loop body at the stage markers - core.py:958-1180 - here
+    ``cluster_ops``; marker count must equal ``schedule.num_stages``.
+  * unrolling over microbatches and list-scheduling the unrolled tasks against
+    the per-rank tables - core.py:1896-2098 - here ``order_tasks``, with the
+    reference's two failure messages.
+  * ``task_impl`` dispatch of each task - src/jaxpp/jax_primitives.py:776-859 -
+    here one ``StageExecutor.run_task`` per task, all MPMD groups on one GPU.
+"""
+from __future__ import annotations
+
+import contextlib
+import ctypes as C
+import time
+from collections import defaultdict
+from dataclasses import dataclass
+from typing import Any, Callable, Iterable, Sequence
+
+import numpy as np
+
+from jaxpp_amd import tracing
+from jaxpp_amd.mesh import MpmdMesh
+from jaxpp_amd.plan import make_rank_plan
+from jaxpp_amd.schedules import (BaseSchedule, FusedTask, Task, mk_task_name,
+                                 preprocess_schedule_tasks)
+from jaxpp_amd.types import TaskType
+
+# ---------------------------------------------------------------------------
+# per-task timings (reference: collect_task_times_ms, jax_primitives.py:742-773)
+# ---------------------------------------------------------------------------
+_statistics = None
+
+
+@contextlib.contextmanager
+def collect_task_times_ms(enabled: bool = True):
+    """``with collect_task_times_ms() as stats`` -> ``{task_name: [ms, ...]}``;
+    while active every task is bracketed by device synchronisation, as in the
+    reference.  ``enabled=False`` yields ``None``."""
+    global _statistics
+    if not enabled:
+        yield
+        return
+    old, _statistics = _statistics, defaultdict(list)
+    try:
+        yield _statistics
+    finally:
+        _statistics = old
+
+
+# ---------------------------------------------------------------------------
+# autodiff marker for the traced body
+# ---------------------------------------------------------------------------
+def value_and_grad(fun: Callable, has_aux: bool = False) -> Callable:
+    """Like ``jax.value_and_grad`` for a loss traced through
+    ``jaxpp_amd.nn``: differentiates with respect to the first argument (the
+    parameter pytree).  The gradients are symbolic; ``treduce`` materialises
+    their sum over microbatches."""
+
+    def wrapped(params, *args):
+        if tracing.current() is None:
+            raise RuntimeError("value_and_grad(...) evaluates inside jaxpp_amd.treduce")
+        out = fun(params, *args)
+        grads = tracing.tree_map(lambda a: tracing.GradOf(id(a), tuple(np.shape(a))), params)
+        return out, grads
+
+    return wrapped
+
+
+# ---------------------------------------------------------------------------
+# loop body -> stages
+# ---------------------------------------------------------------------------
+@dataclass
+class StagedBody:
+    stage_layers: list          # per stage: [(spec, params dict), ...]
+    loss_scale: float | None    # scale of the mse loss of the last stage, if any
+    leaf_owner: dict            # id(param array) -> (stage, layer index, name)
+
+
+def cluster_ops(tr: tracing.Trace, target_num_stages: int) -> StagedBody:
+    stages, cur, has_mse = [], [], False
+    for op in tr.ops:
+        if op[0] == "layer":
+            if has_mse:
+                raise AssertionError("layers after the loss are not part of any stage")
+            cur.append((op[1], op[2]))
+        elif op[0] == "yield":
+            stages.append(cur)
+            cur = []
+        elif op[0] == "mse":
+            has_mse = True
+    if cur and stages:            # trailing layers join the last stage, like trailing eqns
+        stages[-1] = stages[-1] + cur
+    found = len(stages)
+    if found != target_num_stages:
+        raise AssertionError(f"Unexpected number of pipeline markers: found {found} "
+                             f"expected {target_num_stages}.\n")
+    owner = {}
+    for s, layers in enumerate(stages):
+        if not layers:
+            raise AssertionError(f"Empty stage {(s, TaskType.FWD)}")
+        for li, (_, params) in enumerate(layers):
+            for name, arr in params.items():
+                owner[id(arr)] = (s, li, name)
+    return StagedBody(stages, 1.0 if has_mse else None, owner)
+
+
+# ---------------------------------------------------------------------------
+# unrolled task graph + list scheduling
+# ---------------------------------------------------------------------------
+def task_dependencies(t: Task, num_stages: int, split: set) -> list:
+    """Tasks whose results ``t`` consumes.  ``split`` holds the stages whose
+    backward runs as BWD_I + BWD_W."""
+    s, m, k = t.stage_id, t.mubatch_idx, t.fwd_or_bwd
+    back = lambda st: TaskType.BWD_I if st in split else TaskType.BWD
+    deps = []
+    if k is TaskType.FWD:
+        if s > 0:
+            deps.append(Task.make(s - 1, m, TaskType.FWD))
+    elif k is TaskType.BWD_W:
+        deps.append(Task.make(s, m, TaskType.BWD_I))
+    else:
+        deps.append(Task.make(s, m, TaskType.FWD))
+        if s + 1 < num_stages:
+            deps.append(Task.make(s + 1, m, back(s + 1)))
+    if m > 0 and k is not TaskType.FWD:       # accumulators are loop carries
+        deps.append(Task.make(s, m - 1, k))
+    return deps
+
+
+@dataclass(frozen=True)
+class TimedEntry:
+    start_time: int
+    end_time: int
+    rank: int
+    entry: Any                   # Task | FusedTask
+
+
+def order_tasks(rows: list, num_stages: int) -> list:
+    """Global order of the per-rank rows: repeatedly advance the rank whose
+    next entry is ready and can start earliest (ties: lowest rank), then sort
+    by (start, end).  Restates ``reorder_nodes_with_schedule``
+    (src/jaxpp/core.py:1966-2098) including its two errors."""
+    split = {t.stage_id for row in rows for e in row
+             for t in (e if isinstance(e, FusedTask) else (e,))
+             if t.fwd_or_bwd is TaskType.BWD_W}
+    # a first-stage BWD_I that swallowed its BWD_W stands for the whole backward
+    all_tasks = [t for row in rows for e in row for t in (e if isinstance(e, FusedTask) else (e,))]
+    present = set(all_tasks)
+    done_at: dict = {}
+    pos = [0] * len(rows)
+    clock = [0] * len(rows)
+    out = []
+    remaining = len(all_tasks)
+    while remaining:
+        best = None
+        for r, row in enumerate(rows):
+            if pos[r] >= len(row):
+                continue
+            entry = row[pos[r]]
+            members = tuple(entry) if isinstance(entry, FusedTask) else (entry,)
+            ready, inside, ok = clock[r], set(), True
+            for t in members:
+                for d in task_dependencies(t, num_stages, split):
+                    if d not in present or d in inside:
+                        continue
+                    if d not in done_at:
+                        ok = False
+                        break
+                    ready = max(ready, done_at[d])
+                if not ok:
+                    break
+                inside.add(t)
+            if ok and (best is None or ready < best[0]):
+                best = (ready, r, entry, members)
+        if best is None:
+            where = {r: (pos[r], rows[r][pos[r]]) for r in range(len(rows)) if pos[r] < len(rows[r])}
+            raise AssertionError("Schedule does not honor data dependencies.\n"
+                                 f"Current position in schedule for ranks {where}.")
+        start, r, entry, members = best
+        end = start
+        for t in members:
+            end += t.latency
+            done_at[t] = end
+        out.append(TimedEntry(start, end, r, entry))
+        pos[r] += 1
+        clock[r] = end
+        remaining -= len(members)
+    for r, row in enumerate(rows):
+        if pos[r] != len(row):
+            raise AssertionError("Loop tasks have ended but schedule contains other tasks. "
+                                 f"{row[pos[r]:]}")
+    return sorted(out, key=lambda e: (e.start_time, e.end_time))
+
+
+def validate_schedule(schedule: BaseSchedule, n_mubatches: int,
+                      unpack_fused_tasks: bool = False) -> list:
+    """Preprocess the table and check it against the task graph; returns the
+    global order."""
+    rows = preprocess_schedule_tasks(schedule.tasks(n_mubatches), 0, unpack_fused_tasks)
+    seen = set()
+    for row in rows:
+        for e in row:
+            for t in (e if isinstance(e, FusedTask) else (e,)):
+                seen.add((t.stage_id, t.mubatch_idx, t.fwd_or_bwd))
+    for s in range(schedule.num_stages):
+        for m in range(n_mubatches):
+            if (s, m, TaskType.FWD) not in seen:
+                raise AssertionError("Loop tasks have ended but schedule contains other tasks. "
+                                     f"missing fwd_{s}__{m}")
+    return order_tasks(rows, schedule.num_stages)
+
+
+# ---------------------------------------------------------------------------
+# the decorator
+# ---------------------------------------------------------------------------
+_active_function = None
+
+
+class TraceableFunction:
+    def __init__(self, fun: Callable, mpmd_mesh: MpmdMesh, options: dict):
+        self.fun, self.mpmd_mesh, self.options = fun, mpmd_mesh, options
+        self._executors = {}        # key -> {rank: StageExecutor}
+        self.last_order = None      # TimedEntry list of the last loop
+        self.__wrapped__ = fun
+
+    def compile(self, *args, **kwargs):
+        """Runs the function once so that executors exist and kernels are
+        loaded; returns ``self`` (the compiled callable)."""
+        self(*args, **kwargs)
+        return self
+
+    def __call__(self, *args, **kwargs):
+        global _active_function
+        if _active_function is not None:
+            raise RuntimeError("nested mpmd_jit_with_loop calls are not supported")
+        _active_function = self
+        try:
+            with self.mpmd_mesh:
+                return self.fun(*args, **kwargs)
+        finally:
+            _active_function = None
+
+    def close(self):
+        for group in self._executors.values():
+            for ex in group.values():
+                ex.close()
+        self._executors.clear()
+
+
+def mpmd_jit_with_loop(fun: Callable | None = None, mpmd_mesh: MpmdMesh | None = None, *,
+                       in_shardings=None, out_shardings=None, in_specs=None, out_specs=None,
+                       static_argnums: int | Sequence[int] | None = None,
+                       static_argnames: str | Iterable[str] | None = None,
+                       donate_argnums: int | Sequence[int] | None = None,
+                       donate_argnames: str | Iterable[str] | None = None,
+                       compiler_options: dict | None = None) -> TraceableFunction:
+    """Signature of the reference's decorator (core.py:3892-3905).  Sharding,
+    static and donation arguments are accepted and validated the same way;
+    with one device per MPMD group there is nothing for them to change."""
+    if in_specs is not None and in_shardings is not None:
+        raise ValueError("Can't pass both in_shardings and in_specs")
+    if out_specs is not None and out_shardings is not None:
+        raise ValueError("Can't pass both out_shardings and out_specs")
+    if mpmd_mesh is None:
+        raise TypeError("mpmd_jit_with_loop() missing required argument: 'mpmd_mesh'")
+    opts = dict(in_shardings=in_shardings or in_specs, out_shardings=out_shardings or out_specs,
+                static_argnums=static_argnums, static_argnames=static_argnames,
+                donate_argnums=donate_argnums, donate_argnames=donate_argnames,
+                compiler_options=compiler_options)
+    if fun is None:
+        return lambda f: TraceableFunction(f, mpmd_mesh, opts)
+    return TraceableFunction(fun, mpmd_mesh, opts)
+
+
+# ---------------------------------------------------------------------------
+# running the loop
+# ---------------------------------------------------------------------------
+def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSchedule):
+    from jaxpp_amd import runtime as rt
+    fn = _active_function
+    if fn is None:
+        raise RuntimeError("treduce executes under mpmd_jit_with_loop (it needs the MPMD mesh)")
+    mesh = fn.mpmd_mesh
+    body = cluster_ops(tr, schedule.num_stages)
+    S = schedule.num_stages
+    rows = preprocess_schedule_tasks(schedule.tasks(n), 0, False)
+    if len(rows) != mesh.mpmd_dim:
+        raise AssertionError(f"schedule places tasks on {len(rows)} MPMD groups, the mesh has "
+                             f"{mesh.mpmd_dim}")
+    order = order_tasks(rows, S)
+    fn.last_order = order
+    plans = [make_rank_plan(schedule, n, r) for r in range(len(rows))]
+
+    spec = body.stage_layers[0][0][0]
+    lib = rt.load()
+    key = (spec, tuple(len(l) for l in body.stage_layers), type(schedule).__name__, S, n)
+    if key not in fn._executors:
+        fn.close()
+        group = {}
+        for r, plan in enumerate(plans):
+            counts = {len(body.stage_layers[s]) for s in plan.stages}
+            specs = {sp for s in plan.stages for sp, _ in body.stage_layers[s]}
+            if len(counts) != 1 or specs != {spec}:
+                raise NotImplementedError("the stages of one rank must hold the same layers")
+            group[r] = rt.StageExecutor(spec, plan.n_chunks, counts.pop(), plan.max_live,
+                                        plan.split_backward, True)
+        fn._executors[key] = group
+    execs = fn._executors[key]
+    chunk_of = {s: (r, plans[r].stages.index(s)) for r in range(len(plans)) for s in plans[r].stages}
+    for s, layers in enumerate(body.stage_layers):
+        r, c = chunk_of[s]
+        for li, (_, params) in enumerate(layers):
+            execs[r].set_params(c, li, params)
+    for ex in execs.values():
+        ex.zero_grads()
+
+    act_elems = spec.tokens * spec.hidden
+    if x.shape[1:] != (spec.tokens, spec.hidden):
+        x = x.reshape(n, spec.tokens, spec.hidden)
+    xs_dev = [rt.DeviceBuffer.from_f32_as_bf16(x[m]) for m in range(n)]
+    act, cot = {}, {}                   # (stage, mb) -> DeviceBuffer
+    free = []
+
+    def take():
+        return free.pop() if free else rt.DeviceBuffer(act_elems * 2)
+
+    loss_dev = rt.DeviceBuffer(4 * n)
+    partial = rt.DeviceBuffer(4 * rt.NORM_PARTIALS)
+    want_pred = any(isinstance(v, tracing.Traced) and v.shape != () for v in tracing.tree_leaves(outputs))
+    preds = {}
+    loss_scale = None
+    for v in tracing.tree_leaves(outputs):
+        if isinstance(v, tracing.Traced) and v.shape == () and v.producer[0] == "mse":
+            loss_scale = v.producer[1]
+
+    for te in order:
+        members = tuple(te.entry) if isinstance(te.entry, FusedTask) else (te.entry,)
+        for t in members:
+            s, m = t.stage_id, t.mubatch_idx
+            r, c = chunk_of[s]
+            kind = t.fwd_or_bwd
+            if kind is TaskType.BWD_I and s == 0 and t.latency > 1:
+                kind = TaskType.BWD
+            t0 = None
+            if _statistics is not None:
+                rt.sync()
+                t0 = time.perf_counter()
+            if kind is TaskType.FWD:
+                src = xs_dev[m] if s == 0 else act.pop((s, m))
+                dst = take()
+                execs[r].run_task(kind, c, m, src.ptr, dst.ptr)
+                if s > 0:
+                    free.append(src)
+                if s + 1 < S:
+                    act[s + 1, m] = dst
+                else:
+                    if body.loss_scale is None:
+                        raise AssertionError("the last stage has no loss to differentiate")
+                    d = take()
+                    rt.check(lib.jpp_mse_loss(None, dst.ptr, xs_dev[m].ptr, act_elems,
+                                              float(loss_scale), loss_dev.ptr + 4 * m, d.ptr,
+                                              partial.ptr))
+                    cot[s, m] = d
+                    if want_pred:
+                        preds[m] = dst.download_bf16((spec.tokens, spec.hidden))
+                    free.append(dst)
+            elif kind is TaskType.BWD_W:
+                execs[r].run_task(kind, c, m)
+            else:
+                src = cot.pop((s, m))
+                dst = take()
+                execs[r].run_task(kind, c, m, src.ptr, dst.ptr)
+                free.append(src)
+                if s > 0:
+                    cot[s - 1, m] = dst
+                else:
+                    free.append(dst)
+            if t0 is not None:
+                rt.sync()
+                _statistics[mk_task_name(s, t.fwd_or_bwd)].append((time.perf_counter() - t0) * 1e3)
+    rt.sync()
+    losses = loss_dev.download(np.float32, (n,))
+    grads = {s: [execs[chunk_of[s][0]].get_grads(chunk_of[s][1], li)
+                 for li in range(len(body.stage_layers[s]))] for s in range(S)}
+
+    def reduce_leaf(v, op):
+        if isinstance(v, tracing.GradOf):
+            if type(op).__name__ != "AddT":
+                raise NotImplementedError("gradients are reduced with Add")
+            s, li, name = body.leaf_owner[v.leaf_id]
+            return grads[s][li][name].reshape(v.shape)
+        if isinstance(v, tracing.Traced):
+            per_mb = ([np.float32(losses[m]) for m in range(n)] if v.shape == ()
+                      else [preds[m].reshape(v.shape) for m in range(n)])
+            state = op.state(n, per_mb[0])
+            for m in range(n):
+                state = op.update(state, per_mb[m], m)
+            return state
+        return v
+
+    def walk(v, op):
+        if isinstance(v, (tuple, list)):
+            return type(v)(walk(a, b) for a, b in zip(v, op))
+        if isinstance(v, dict):
+            return {k: walk(v[k], op[k]) for k in v}
+        return reduce_leaf(v, op)
+
+    return walk(outputs, ops)

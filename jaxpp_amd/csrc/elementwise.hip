@@ -346,6 +346,39 @@ __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* dst, uint32_t v
     dst[i] = v;
 }
 
+// loss of the last stage: mean((out - target)^2) * scale, and its cotangent
+__global__ __launch_bounds__(256) void mse_partial_kernel(const bf16_t* __restrict__ out,
+                                                          const bf16_t* __restrict__ target,
+                                                          long n8, float dscale,
+                                                          bf16_t* __restrict__ dout,
+                                                          float* __restrict__ partial) {
+  __shared__ float red[4];
+  float s = 0.f;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n8; i += (long)gridDim.x * 256) {
+    float a[8], b[8];
+    unpack8(((const uint4*)out)[i], a);
+    unpack8(((const uint4*)target)[i], b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float d = a[e] - b[e];
+      s += d * d;
+      a[e] = d * dscale;
+    }
+    ((uint4*)dout)[i] = pack8(a);
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) partial[blockIdx.x] = ((red[0] + red[1]) + red[2]) + red[3];
+}
+__global__ void mse_final_kernel(const float* partial, int n, float scale, float* loss) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    float s = 0.f;
+    for (int i = 0; i < n; ++i) s += partial[i];
+    loss[0] = s * scale;
+  }
+}
+
 int grid_for(long items, int per_block = 256, int cap = 256 * 32) {
   long g = (items + per_block - 1) / per_block;
   return (int)(g < 1 ? 1 : (g > cap ? cap : g));
@@ -500,6 +533,21 @@ int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int6
                      (long)ld, (long)rows, (int)cols, partial);
   hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 255) / 256)), dim3(256), 0, st,
                      partial, nb, (int)cols, acc);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t count, float scale,
+                 float* loss, void* dout, float* partial) {
+  JPP_REQUIRE(out && target && loss && dout && partial && count > 0 && count % 8 == 0,
+              "mse_loss: bad arguments (count must be a positive multiple of 8)");
+  hipStream_t st = (hipStream_t)stream;
+  const long n8 = count / 8;
+  const int nb = (int)(n8 < JPP_NORM_PARTIALS ? n8 : JPP_NORM_PARTIALS);
+  hipLaunchKernelGGL(mse_partial_kernel, dim3(nb), dim3(256), 0, st, (const bf16_t*)out,
+                     (const bf16_t*)target, n8, 2.0f * scale / (float)count, (bf16_t*)dout, partial);
+  hipLaunchKernelGGL(mse_final_kernel, dim3(1), dim3(64), 0, st, partial, nb,
+                     scale / (float)count, loss);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }

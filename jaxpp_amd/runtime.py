@@ -78,7 +78,7 @@ EXPORTS = [
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
     "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
-    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
+    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
     "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
     "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_bytes",
     "jpp_stage_run_task", "jpp_stage_live_slots",
@@ -133,6 +133,8 @@ def load():
     lib.jpp_grad_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
     lib.jpp_colsum_accum.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                      C.c_void_p, C.c_void_p]
+    lib.jpp_mse_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float,
+                                 C.c_void_p, C.c_void_p, C.c_void_p]
     lib.jpp_cast_f32_to_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
     lib.jpp_cast_bf16_to_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
     lib.jpp_stage_create.argtypes = [C.POINTER(StageDesc), C.POINTER(C.c_void_p)]
