@@ -109,7 +109,7 @@ typedef struct {
   int trans_a, trans_b;
   int epilogue;      /* jpp_epilogue */
   int gelu_tanh;     /* 0: erf form, 1: tanh approximation */
-  int tile;          /* 0: choose; 1: 128x128; 2: 256x128; 3: 256x256 (tuning/tests) */
+  int tile;          /* 0: choose; 1: 128x128; 2: 256x128; 3: 256x256; 4: 256x256 with 8 waves */
 } jpp_gemm_args;
 
 int jpp_gemm_bf16(void* stream, const jpp_gemm_args* args);

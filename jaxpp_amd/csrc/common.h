@@ -208,10 +208,11 @@ __device__ __forceinline__ void dma_load16(const bf16_t* base, uint32_t off, uin
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-template <int ROWS, bool MC>
+template <int ROWS, bool MC, int NW = 4>
 struct DmaTile {
   static constexpr int BYTES = ROWS * 128;
-  static constexpr int INSTS = ROWS / 32;  // wave-level loads per wave (4 waves share a tile)
+  static constexpr int INSTS = ROWS / (8 * NW);  // wave-level loads per wave (NW waves share a tile)
+  static_assert(INSTS >= 1, "tile too small for this many waves");
   typedef uint32_t Offsets[INSTS];
 
   // per-lane byte offsets (from the tile's first element) of this wave's loads;

@@ -98,16 +98,17 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const bf16_t* __restrict_
 // ---------------------------------------------------------------------------
 // norm backward: dx per row, and per-block partial sums of dgamma / dbeta
 // ---------------------------------------------------------------------------
+constexpr int kNormBwdWaves = 8;
 template <bool LN, int NCH>
-__global__ __launch_bounds__(256) void norm_bwd_kernel(
+__global__ __launch_bounds__(kNormBwdWaves * 64) void norm_bwd_kernel(
     const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x, const float* __restrict__ mean_in,
     const float* __restrict__ rstd_in, const bf16_t* __restrict__ gamma,
     const bf16_t* __restrict__ resid, bf16_t* __restrict__ dx, float* __restrict__ partial,
     long rows, int cols) {
-  __shared__ float red[4][64 * 8];
+  __shared__ float red[kNormBwdWaves][64 * 8];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nchunk = cols >> 3;
-  const long stride = (long)gridDim.x * 4;
+  const long stride = (long)gridDim.x * kNormBwdWaves;
   float pg[NCH][8], pb[LN ? NCH : 1][8];
 #pragma unroll
   for (int i = 0; i < NCH; ++i)
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(
       pg[i][e] = 0.f;
       if (LN) pb[i][e] = 0.f;
     }
-  for (long row = (long)blockIdx.x * 4 + wave; row < rows; row += stride) {
+  for (long row = (long)blockIdx.x * kNormBwdWaves + wave; row < rows; row += stride) {
     const float rstd = rstd_in[row];
     const float mean = LN ? mean_in[row] : 0.f;
     const uint4* xr = (const uint4*)(x + row * cols);
@@ -167,7 +168,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(
       }
     }
   }
-  // combine the 4 waves of the block in a fixed order, one chunk column at a time
+  // combine the waves of the block in a fixed order, one chunk column at a time
   float* pgam = partial + (long)blockIdx.x * cols;
   float* pbet = partial + ((long)gridDim.x + blockIdx.x) * cols;
 #pragma unroll
@@ -182,8 +183,9 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(
       if (wave == 0 && c < nchunk) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float t = ((red[0][lane * 8 + e] + red[1][lane * 8 + e]) + red[2][lane * 8 + e]) +
-                          red[3][lane * 8 + e];
+          float t = red[0][lane * 8 + e];
+#pragma unroll
+          for (int w = 1; w < kNormBwdWaves; ++w) t += red[w][lane * 8 + e];
           (pass ? pbet : pgam)[c * 8 + e] = t;
         }
       }
@@ -191,15 +193,25 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(
   }
 }
 
-// acc[j] += sum_b partial[b][j], b ascending
+// acc[j] += sum_b partial[b][j]: a block owns 32 columns; 8 thread groups sum
+// interleaved subsets of the partials, then one combines them in a fixed order
 __global__ __launch_bounds__(256) void partial_reduce_kernel(const float* __restrict__ partial,
                                                              int nblocks, int cols,
                                                              float* __restrict__ acc) {
-  const int j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= cols) return;
+  __shared__ float red[8][32];
+  const int c = threadIdx.x & 31, g = threadIdx.x >> 5;
+  const int j = blockIdx.x * 32 + c;
   float s = 0.f;
-  for (int b = 0; b < nblocks; ++b) s += partial[(long)b * cols + j];
-  acc[j] += s;
+  if (j < cols)
+    for (int b = g; b < nblocks; b += 8) s += partial[(long)b * cols + j];
+  red[g][c] = s;
+  __syncthreads();
+  if (g == 0 && j < cols) {
+    float t = red[0][c];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) t += red[w][c];
+    acc[j] += t;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -407,7 +419,7 @@ int launch_norm_bwd(hipStream_t st, const jpp_norm_args* a) {
   const int nch = (int)((a->cols / 8 + 63) / 64);
   const int blocks = JPP_NORM_PARTIALS;
 #define JPP_NB(N)                                                                             \
-  hipLaunchKernelGGL((norm_bwd_kernel<LN, N>), dim3(blocks), dim3(256), 0, st,                \
+  hipLaunchKernelGGL((norm_bwd_kernel<LN, N>), dim3(blocks), dim3(kNormBwdWaves * 64), 0, st, \
                      (const bf16_t*)a->dy, (const bf16_t*)a->x, a->mean, a->rstd,             \
                      (const bf16_t*)a->gamma, (const bf16_t*)a->resid, (bf16_t*)a->dx,        \
                      a->partial, (long)a->rows, (int)a->cols)
@@ -418,7 +430,7 @@ int launch_norm_bwd(hipStream_t st, const jpp_norm_args* a) {
   else JPP_NB(16);
 #undef JPP_NB
   JPP_LAUNCH_CHECK();
-  const int cb = (int)((a->cols + 255) / 256);
+  const int cb = (int)((a->cols + 31) / 32);
   hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb), dim3(256), 0, st, a->partial, blocks,
                      (int)a->cols, a->dgamma);
   if (LN)
@@ -531,7 +543,7 @@ int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int6
   const int panels = (int)((cols / 8 + 255) / 256);
   hipLaunchKernelGGL(colsum_partial_kernel, dim3(nb, panels), dim3(256), 0, st, (const bf16_t*)x,
                      (long)ld, (long)rows, (int)cols, partial);
-  hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 255) / 256)), dim3(256), 0, st,
+  hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 31) / 32)), dim3(256), 0, st,
                      partial, nb, (int)cols, acc);
   JPP_LAUNCH_CHECK();
   return JPP_OK;

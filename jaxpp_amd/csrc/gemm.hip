@@ -70,16 +70,17 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm,
   tn = (pid % width) / gsize;
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
-  using TileA = DmaTile<BM, TA>;
-  using TileB = DmaTile<BN, TB>;
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
+  using TileA = DmaTile<BM, TA, NW>;
+  using TileB = DmaTile<BN, TB, NW>;
   constexpr int A_BYTES = TileA::BYTES, STAGE = TileA::BYTES + TileB::BYTES;
-  constexpr int TM = BM / 64, TN = BN / 64;  // 32x32 MFMA tiles per wave
+  constexpr int WN = NW / 2;                        // waves: 2 along m, NW/2 along n
+  constexpr int TM = BM / 64, TN = BN / (32 * WN);  // 32x32 MFMA tiles per wave
   extern __shared__ __align__(1024) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   int tm, tn;
   tile_of_block(p.tiles_m, p.tiles_n, tm, tn);
   const long m0 = (long)tm * BM, n0 = (long)tn * BN;
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
     bf16x8 fw[2][TN], fx[2][TM];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag(sb, wn * (BN / 2) + j * 32, 0, lane);
+    for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag(sb, wn * (BN / WN) + j * 32, 0, lane);
 #pragma unroll
     for (int i = 0; i < TM; ++i) fx[0][i] = TileA::frag(sa, wm * (BM / 2) + i * 32, 0, lane);
 #pragma unroll
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
       if (ks < 3) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          fw[nxt][j] = TileB::frag(sb, wn * (BN / 2) + j * 32, ks + 1, lane);
+          fw[nxt][j] = TileB::frag(sb, wn * (BN / WN) + j * 32, ks + 1, lane);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
           fx[nxt][i] = TileA::frag(sa, wm * (BM / 2) + i * 32, ks + 1, lane);
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const long n = n0 + wn * (BN / 2) + j * 32 + g * 8 + (lane >> 5) * 4;
+        const long n = n0 + wn * (BN / WN) + j * 32 + g * 8 + (lane >> 5) * 4;
         float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
         float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
         if constexpr (EPI == JPP_EPI_ACC_F32) {
@@ -201,25 +202,25 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
   }
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI>
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW>
 const char* class_name() {
   static char name[64] = "";
   if (!name[0]) {
     const char* lay = TA ? "tn" : (TB ? "nn" : "nt");
     const char* epi = EPI == JPP_EPI_BF16 ? "bf16" : EPI == JPP_EPI_GELU ? "gelu"
                     : EPI == JPP_EPI_DGELU ? "dgelu" : EPI == JPP_EPI_ACC_F32 ? "accf32" : "f32";
-    snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d", lay, epi, BM, BN);
+    snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d%s", lay, epi, BM, BN, NW == 8 ? "w8" : "");
   }
   return name;
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI>
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4>
 int launch(hipStream_t stream, GemmParams& p) {
   constexpr int SMEM = 2 * (BM + BN) * 128;
-  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI>(), 2.0 * p.m * p.n * p.k,
+  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW>(), 2.0 * p.m * p.n * p.k,
                    2.0 * ((double)p.m * p.k + (double)p.n * p.k) +
                        (double)p.m * p.n * (EPI == JPP_EPI_ACC_F32 ? 8 : EPI == JPP_EPI_F32 ? 4 : 2));
-  auto kern = gemm_kernel<BM, BN, TA, TB, EPI>;
+  auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW>;
   static bool configured = false;  // per instantiation; attribute is sticky
   if (!configured) {
     JPP_CHECK_HIP(hipFuncSetAttribute((const void*)kern,
@@ -228,7 +229,7 @@ int launch(hipStream_t stream, GemmParams& p) {
   }
   p.tiles_m = p.m / BM;
   p.tiles_n = p.n / BN;
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), SMEM, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(NW * 64), SMEM, stream, p);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -238,18 +239,17 @@ int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
   switch (tile) {
     case 1: return launch<128, 128, TA, TB, EPI>(stream, p);
     case 2: return launch<256, 128, TA, TB, EPI>(stream, p);
+    case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
     default: return launch<256, 256, TA, TB, EPI>(stream, p);
   }
 }
 
-// Largest tile that still gives every CU work: 256 CUs, one 256x256 or two
-// 128x128 workgroups resident per CU.
+// 256 CUs.  The 256x256 tile run by 8 waves (two per SIMD, so one wave's LDS
+// reads hide under the other's MFMAs) is the fastest whenever it gives most CUs
+// a tile; smaller problems take 128x128 tiles, two workgroups per CU.
 int choose_tile(long m, long n) {
   const long t256 = (m % 256 == 0 && n % 256 == 0) ? (m / 256) * (n / 256) : 0;
-  const long t2 = (m % 256 == 0) ? (m / 256) * (n / 128) : 0;
-  if (t256 >= 256) return 3;
-  if (t2 >= 256) return 2;
-  return 1;
+  return t256 >= 192 ? 4 : 1;
 }
 
 }  // namespace
@@ -289,8 +289,8 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
   if (tile >= 2 && a->m % 256) tile = 1;
-  if (tile == 3 && a->n % 256) tile = 2;
-  JPP_REQUIRE(tile >= 1 && tile <= 3, "gemm: unknown tile %d", tile);
+  if (tile >= 3 && a->n % 256) tile = 2;
+  JPP_REQUIRE(tile >= 1 && tile <= 4, "gemm: unknown tile %d", tile);
 
   const int ta = a->trans_a != 0, tb = a->trans_b != 0, e = a->epilogue;
 #define JPP_GEMM_CASE(TA_, TB_, E_) \
