@@ -106,6 +106,11 @@ class Workbench:
         return 3.0 * wl.layer.fwd_flops() * wl.layers_per_stage * self.plan.n_chunks * wl.n_mubatches
 
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size)
+MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.150e9}
+
+
 def dominant_gemm_class(wl) -> str:
     # weight-gradient GEMM with the fp32 accumulate epilogue: a third of the
     # FLOPs and the longest kernel per call
@@ -212,7 +217,7 @@ def main():
             "peak": (HBM_PEAK / 1e9) if hbm else (MFMA_BF16_PEAK / 1e12),
             "unit": "GB/s" if hbm else "TFLOP/s",
             "frac": ach / (HBM_PEAK if hbm else MFMA_BF16_PEAK),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get((wl.name, cls)),
             "launches": pr.launches, "avg_launch_ms": avg_ms,
             "algorithmic_per_launch": (pr.bytes if hbm else pr.flops) / pr.launches,
         }
