@@ -110,7 +110,21 @@ typedef struct {
   int epilogue;      /* jpp_epilogue */
   int gelu_tanh;     /* 0: erf form, 1: tanh approximation */
   int tile;          /* 0: choose; 1: 128x128; 2: 256x128; 3: 256x256; 4: 256x256 with 8 waves */
+  /* grouped GEMM over experts (0 = plain).  seg: device int32 [n_seg + 1], row
+   * offsets of the expert groups in the token-permuted buffers, multiples of 256.
+   *   JPP_GROUP_M: rows of A and C are grouped; group e multiplies b + e * stride_b.
+   *                m is the capacity of the permuted buffer; tiles past seg[n_seg] exit.
+   *   JPP_GROUP_K: (weight gradients) C_e = c + e * stride_c gets the product over the
+   *                rows seg[e] .. seg[e+1] of A and B; k is ignored. */
+  const int32_t* seg;
+  int n_seg;
+  int group_mode;
+  int64_t stride_b, stride_c;
+  int64_t group_rows; /* non-padding rows over all groups, for the probe's FLOP and byte
+                       * accounting only (0: the padded extent is counted) */
 } jpp_gemm_args;
+
+enum { JPP_GROUP_NONE = 0, JPP_GROUP_M = 1, JPP_GROUP_K = 2 };
 
 int jpp_gemm_bf16(void* stream, const jpp_gemm_args* args);
 
@@ -176,6 +190,41 @@ int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t coun
                  float* loss, void* dout, float* partial);
 int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count);
 int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count);
+
+/* ---- top-2 mixture of experts: routing around the grouped GEMMs --------------
+ * Tokens are assigned to rows of "permuted" buffers, grouped by expert in token
+ * order, each group padded to a multiple of 256 rows (padding rows are zero);
+ * jpp_moe_capacity() rows always suffice.  seg[e] is the first row of expert e. */
+typedef struct {
+  const void* x;     /* bf16 [tokens, hidden]: router input (jpp_moe_route only) */
+  const void* wr;    /* bf16 [hidden, n_experts] */
+  int32_t* ids;      /* [tokens, 2] selected experts, by descending logit (ties: lower id) */
+  float* gates;      /* [tokens, 2] softmax over the two selected logits */
+  int32_t* row_of;   /* [tokens, 2] row of each assignment */
+  int32_t* tok_of;   /* [capacity] token of each row, -1 for padding */
+  float* gate_of;    /* [capacity] gate of each row */
+  int32_t* seg;      /* [n_experts + 1] */
+  void* work;        /* int32 [2 * ceil(tokens / 256) * n_experts] scratch */
+  int64_t tokens, hidden;
+  int n_experts, top_k; /* 8, 2 */
+} jpp_moe_args;
+
+int64_t jpp_moe_capacity(int64_t tokens, int n_experts, int top_k);
+int jpp_moe_route(void* stream, const jpp_moe_args* args);
+/* xp[row] = x[tok_of[row]] */
+int jpp_moe_gather(void* stream, const jpp_moe_args* args, const void* x, void* xp);
+/* y[t] = resid[t] + sum_k gates[t,k] * eo[row_of[t,k]] */
+int jpp_moe_combine_fwd(void* stream, const jpp_moe_args* args, const void* eo, const void* resid,
+                        void* y);
+/* dlogits f32 [tokens, n_experts]; deo[row] = gate_of[row] * dy[tok_of[row]] */
+int jpp_moe_bwd_prepare(void* stream, const jpp_moe_args* args, const void* dy, const void* eo,
+                        float* dlogits, void* deo);
+/* dx[t] = dxp[row_of[t,0]] + dxp[row_of[t,1]] + dlogits[t] Wr^T */
+int jpp_moe_combine_bwd(void* stream, const jpp_moe_args* args, const void* dxp,
+                        const float* dlogits, void* dx);
+/* acc[hidden, n_experts] += x^T dlogits; partial: f32 [64 * hidden * n_experts] */
+int jpp_moe_router_wgrad(void* stream, const jpp_moe_args* args, const void* x,
+                         const float* dlogits, float* acc, float* partial);
 
 /* ---- stage executor: stands in for `task_impl` on one pipeline rank ----------
  * A stage object holds this rank's chunks (the stages the schedule places on

@@ -33,6 +33,11 @@ struct GemmParams {
   long lda, ldb, ldc, ldc2, ldresid, ldaux;
   int gelu_tanh;
   int tiles_m, tiles_n;
+  // grouped (mixture-of-experts) problems: seg[0..n_seg] are row offsets, multiples of 256
+  const int* seg;
+  int n_seg, group_mode;
+  int64_t group_rows;
+  long stride_b, stride_c;
 };
 
 __device__ __forceinline__ float gelu_f(float u, int tanh_form) {
@@ -57,9 +62,8 @@ __device__ __forceinline__ float gelu_grad_f(float u, int tanh_form) {
 // XCDs (8 of them, each with its own L2); give every XCD a contiguous range of
 // tiles, and inside a range walk GROUP tile-rows at a time so the B panels in
 // flight stay L2 resident.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int nwg = tiles_m * tiles_n;
-  int pid = blockIdx.x;
   if ((nwg & 7) == 0) pid = (pid & 7) * (nwg >> 3) + (pid >> 3);
   constexpr int GROUP = 8;
   const int width = GROUP * tiles_n;
@@ -82,11 +86,31 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
   int tm, tn;
-  tile_of_block(p.tiles_m, p.tiles_n, tm, tn);
+  const int tiles = p.tiles_m * p.tiles_n;
+  tile_of_block(p.group_mode == JPP_GROUP_K ? (int)blockIdx.x % tiles : (int)blockIdx.x, p.tiles_m,
+                p.tiles_n, tm, tn);
   const long m0 = (long)tm * BM, n0 = (long)tn * BN;
 
   const bf16_t* a_src = TA ? p.a + m0 : p.a + m0 * p.lda;
   const bf16_t* b_src = TB ? p.b + n0 : p.b + n0 * p.ldb;
+  int kt_n = p.k / 64;
+  if (p.group_mode == JPP_GROUP_M) {
+    // rows of A and C are grouped by expert; each group multiplies its own B
+    if (m0 >= p.seg[p.n_seg]) return;
+    int e = 0;
+    while (p.seg[e + 1] <= m0) ++e;
+    b_src += (long)e * p.stride_b;
+  } else if (p.group_mode == JPP_GROUP_K) {
+    // one output per expert; the contraction runs over the expert's rows
+    const int e = blockIdx.x / tiles;
+    const long r0 = p.seg[e];
+    kt_n = (p.seg[e + 1] - p.seg[e]) / 64;
+    a_src += r0 * p.lda;
+    b_src += r0 * p.ldb;
+    p.c = EPI == JPP_EPI_BF16 ? (void*)((bf16_t*)p.c + (long)e * p.stride_c)
+                              : (void*)((float*)p.c + (long)e * p.stride_c);
+    if (kt_n == 0 && EPI == JPP_EPI_ACC_F32) return;
+  }
   const long a_step = TA ? 64 * p.lda : 64;
   const long b_step = TB ? 64 * p.ldb : 64;
 
@@ -98,15 +122,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int kt_n = p.k / 64;
   const uint32_t lds0 = lds_address(smem);
   typename TileA::Offsets offa;
   typename TileB::Offsets offb;
   TileA::offsets(offa, p.lda, wave, lane);
   TileB::offsets(offb, p.ldb, wave, lane);
   constexpr int IA = TileA::INSTS, IB = TileB::INSTS;
-  TileA::template issue<0, IA>(uniform_ptr(a_src), offa, lds0, wave);
-  TileB::template issue<0, IB>(uniform_ptr(b_src), offb, lds0 + A_BYTES, wave);
+  if (kt_n > 0) {
+    TileA::template issue<0, IA>(uniform_ptr(a_src), offa, lds0, wave);
+    TileB::template issue<0, IB>(uniform_ptr(b_src), offb, lds0 + A_BYTES, wave);
+  }
   dma_wait_all();
   __syncthreads();
 
@@ -217,9 +242,14 @@ const char* class_name() {
 template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4>
 int launch(hipStream_t stream, GemmParams& p) {
   constexpr int SMEM = 2 * (BM + BN) * 128;
-  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW>(), 2.0 * p.m * p.n * p.k,
-                   2.0 * ((double)p.m * p.k + (double)p.n * p.k) +
-                       (double)p.m * p.n * (EPI == JPP_EPI_ACC_F32 ? 8 : EPI == JPP_EPI_F32 ? 4 : 2));
+  // algorithmic extent: grouped launches count the non-padding rows when the caller gave them
+  const double cb = EPI == JPP_EPI_ACC_F32 ? 8 : EPI == JPP_EPI_F32 ? 4 : 2;
+  double am = p.m, ak = p.k, copies = 1;
+  if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
+  if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
+  const double b_bytes = 2.0 * p.n * ak * (p.group_mode == JPP_GROUP_M ? p.n_seg : 1);
+  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW>(), 2.0 * am * p.n * ak,
+                   2.0 * am * ak + b_bytes + copies * am * p.n * cb);
   auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW>;
   static bool configured = false;  // per instantiation; attribute is sticky
   if (!configured) {
@@ -229,7 +259,8 @@ int launch(hipStream_t stream, GemmParams& p) {
   }
   p.tiles_m = p.m / BM;
   p.tiles_n = p.n / BN;
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(NW * 64), SMEM, stream, p);
+  const int blocks = p.tiles_m * p.tiles_n * (p.group_mode == JPP_GROUP_K ? p.n_seg : 1);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(NW * 64), SMEM, stream, p);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -257,12 +288,14 @@ int choose_tile(long m, long n) {
 extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   hipStream_t stream = (hipStream_t)stream_;
   JPP_REQUIRE(a && a->a && a->b && a->c, "gemm: null operand");
-  JPP_REQUIRE(a->m > 0 && a->n > 0 && a->k > 0, "gemm: empty problem %ldx%ldx%ld", (long)a->m,
-              (long)a->n, (long)a->k);
-  JPP_REQUIRE(a->m % 128 == 0 && a->n % 128 == 0 && a->k % 64 == 0,
+  const bool group_k = a->group_mode == JPP_GROUP_K;
+  JPP_REQUIRE(a->m > 0 && a->n > 0 && (a->k > 0 || group_k), "gemm: empty problem %ldx%ldx%ld",
+              (long)a->m, (long)a->n, (long)a->k);
+  JPP_REQUIRE(a->m % 128 == 0 && a->n % 128 == 0 && (a->k % 64 == 0 || group_k),
               "gemm: M,N must be multiples of 128 and K of 64, got %ldx%ldx%ld", (long)a->m,
               (long)a->n, (long)a->k);
-  JPP_REQUIRE(a->lda >= (a->trans_a ? a->m : a->k) && a->ldb >= (a->trans_b ? a->n : a->k) &&
+  JPP_REQUIRE(a->lda >= (a->trans_a ? a->m : (group_k ? 0 : a->k)) &&
+                  a->ldb >= (a->trans_b ? a->n : (group_k ? 0 : a->k)) &&
                   a->ldc >= a->n,
               "gemm: leading dimension too small");
   JPP_REQUIRE(a->lda % 8 == 0 && a->ldb % 8 == 0 && a->ldc % 4 == 0,
@@ -282,12 +315,23 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   p.lda = a->lda; p.ldb = a->ldb; p.ldc = a->ldc;
   p.ldc2 = a->ldc2; p.ldresid = a->ldresid; p.ldaux = a->ldaux;
   p.gelu_tanh = a->gelu_tanh;
+  p.seg = a->seg; p.n_seg = a->n_seg; p.group_mode = a->group_mode;
+  p.group_rows = a->group_rows;
+  p.stride_b = a->stride_b; p.stride_c = a->stride_c;
+  if (a->group_mode != JPP_GROUP_NONE) {
+    JPP_REQUIRE(a->group_mode == JPP_GROUP_M || a->group_mode == JPP_GROUP_K,
+                "gemm: unknown group_mode %d", a->group_mode);
+    JPP_REQUIRE(a->seg && a->n_seg > 0 && a->n_seg <= 256, "gemm: grouped problem needs seg[n_seg+1]");
+    JPP_REQUIRE(a->m % 256 == 0 && a->n % 256 == 0, "gemm: grouped problems need M, N multiples of 256");
+    JPP_REQUIRE(!a->bias && !a->resid, "gemm: grouped problems take no bias / residual");
+  }
   if (a->epilogue == JPP_EPI_GELU)
     JPP_REQUIRE(a->c2 && a->ldc2 >= a->n && a->ldc2 % 4 == 0, "gemm: GELU epilogue needs c2");
   if (a->epilogue == JPP_EPI_DGELU)
     JPP_REQUIRE(a->aux && a->ldaux >= a->n && a->ldaux % 4 == 0, "gemm: dGELU epilogue needs aux");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
+  if (a->group_mode != JPP_GROUP_NONE) tile = (a->tile == 3) ? 3 : 4;  // 256-row segments
   if (tile >= 2 && a->m % 256) tile = 1;
   if (tile >= 3 && a->n % 256) tile = 2;
   JPP_REQUIRE(tile >= 1 && tile <= 4, "gemm: unknown tile %d", tile);

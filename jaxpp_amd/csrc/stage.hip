@@ -55,16 +55,19 @@ struct LayerStash {
   Buf a, mean1, rstd1, x1, u, g, c, mean2, rstd2;
   // llama
   Buf n1, h1, n2, gu, s;
+  // mixtral: routing tables and token-permuted expert buffers (gu, s reused, [cap, ..])
+  Buf ids, gates, row_of, tok_of, gate_of, seg, xp, eo;
   // cotangents kept for the weight-gradient task
   Buf dc, du, da, dqkv;   // bert (dqkv shared with llama)
   Buf dyin, dgu, dh1;     // llama
+  Buf deo, dlogits;       // mixtral
 };
 
 }  // namespace
 
 struct jpp_stage {
   jpp_stage_desc d;
-  int64_t T, h, f, qkvw, ctxw, hd;
+  int64_t T, h, f, qkvw, ctxw, hd, cap = 0;  // cap: rows of the token-permuted buffers
   std::vector<ParamInfo> pinfo;
   std::vector<size_t> poff;        // element offset of parameter i inside a layer block
   size_t layer_elems = 0;
@@ -80,7 +83,7 @@ struct jpp_stage {
   uint8_t* scratch = nullptr;
   size_t scratch_bytes = 0;
   LayerStash wshared;              // cotangent buffers when the backward is not split
-  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_delta, s_wg, s_cos, s_sin;
+  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_delta, s_wg, s_cos, s_sin, s_moework;
   size_t total_bytes = 0;
 
   bf16_t* P(int chunk, int layer, int i) {
@@ -97,6 +100,34 @@ namespace {
 
 enum BertP { B_Wqkv, B_bqkv, B_Wo, B_bo, B_ln1g, B_ln1b, B_W1, B_b1, B_W2, B_b2, B_ln2g, B_ln2b };
 enum LlamaP { L_rms1, L_Wqkv, L_Wo, L_rms2, L_Wgu, L_Wd };
+enum MixtralP { X_rms1, X_Wqkv, X_Wo, X_rms2, X_Wr, X_Wgu, X_Wd };
+
+int ggemm(hipStream_t st, int mode, const int* seg, int n_seg, const void* a, int64_t lda, int ta,
+          const void* b, int64_t ldb, int tb, int64_t stride_b, void* c, int64_t ldc,
+          int64_t stride_c, int64_t m, int64_t n, int64_t k, int epi, int64_t rows) {
+  jpp_gemm_args g;
+  memset(&g, 0, sizeof(g));
+  g.a = a; g.b = b; g.c = c; g.m = m; g.n = n; g.k = k;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.trans_a = ta; g.trans_b = tb; g.epilogue = epi;
+  g.seg = seg; g.n_seg = n_seg; g.group_mode = mode; g.stride_b = stride_b; g.stride_c = stride_c;
+  g.group_rows = rows;
+  return jpp_gemm_bf16(st, &g);
+}
+
+void moe_args(jpp_stage* s, jpp_moe_args& m, uint8_t* slot, const LayerStash& L, int chunk,
+              int li) {
+  memset(&m, 0, sizeof(m));
+  m.x = slot + L.n2.off;
+  m.wr = s->P(chunk, li, X_Wr);
+  m.ids = (int32_t*)(slot + L.ids.off);
+  m.gates = (float*)(slot + L.gates.off);
+  m.row_of = (int32_t*)(slot + L.row_of.off);
+  m.tok_of = (int32_t*)(slot + L.tok_of.off);
+  m.gate_of = (float*)(slot + L.gate_of.off);
+  m.seg = (int32_t*)(slot + L.seg.off);
+  m.work = s->S<>(s->s_moework);
+  m.tokens = s->T; m.hidden = s->h; m.n_experts = s->d.n_experts; m.top_k = s->d.top_k;
+}
 
 int gemm(hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int64_t ldb, int tb,
          void* c, int64_t ldc, int64_t m, int64_t n, int64_t k, int epi, const void* bias = nullptr,
@@ -198,6 +229,21 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
           JPP_EPI_BF16, nullptr, at(L.x), h));
   RC(norm_f(s, st, at(L.h1), s->P(chunk, li, L_rms2), nullptr, at(L.n2), nullptr,
             (float*)at(L.rstd2)));
+  if (s->d.family == JPP_FAMILY_MIXTRAL) {
+    jpp_moe_args ma;
+    moe_args(s, ma, slot, L, chunk, li);
+    const int E = s->d.n_experts;
+    const int* seg = ma.seg;
+    RC(jpp_moe_route(st, &ma));
+    RC(jpp_moe_gather(st, &ma, at(L.n2), at(L.xp)));
+    RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.xp), h, 0, s->P(chunk, li, X_Wgu), 2 * f, 1, h * 2 * f,
+             at(L.gu), 2 * f, 0, s->cap, 2 * f, h, JPP_EPI_BF16, s->T * s->d.top_k));
+    RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), s->cap, f));
+    RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.s), f, 0, s->P(chunk, li, X_Wd), h, 1, f * h, at(L.eo), h,
+             0, s->cap, h, f, JPP_EPI_BF16, s->T * s->d.top_k));
+    RC(jpp_moe_combine_fwd(st, &ma, at(L.eo), at(L.h1), y));
+    return JPP_OK;
+  }
   RC(gemm(st, at(L.n2), h, 0, s->P(chunk, li, L_Wgu), 2 * f, 1, at(L.gu), 2 * f, T, 2 * f, h,
           JPP_EPI_BF16));
   RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), T, f));
@@ -250,10 +296,24 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
   void* ds = s->S<>(s->s_t1);
   void* dn = s->S<>(s->s_t2);   // dn2, later dn1
   void* dctx = s->S<>(s->s_t3);
-  RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, ds, f, T, f, h, JPP_EPI_BF16));
-  RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), T, f));
-  RC(gemm(st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
-          JPP_EPI_BF16));
+  if (s->d.family == JPP_FAMILY_MIXTRAL) {
+    jpp_moe_args ma;
+    moe_args(s, ma, slot, L, chunk, li);
+    const int E = s->d.n_experts;
+    void* dxp = s->S<>(s->s_t4);
+    RC(jpp_moe_bwd_prepare(st, &ma, dy, at(L.eo), (float*)wt(W.dlogits), wt(W.deo)));
+    RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.deo), h, 0, s->P(chunk, li, X_Wd), h, 0, f * h, ds, f,
+             0, s->cap, f, h, JPP_EPI_BF16, s->T * s->d.top_k));
+    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), s->cap, f));
+    RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.dgu), 2 * f, 0, s->P(chunk, li, X_Wgu), 2 * f, 0,
+             h * 2 * f, dxp, h, 0, s->cap, h, 2 * f, JPP_EPI_BF16, s->T * s->d.top_k));
+    RC(jpp_moe_combine_bwd(st, &ma, dxp, (const float*)wt(W.dlogits), dn));
+  } else {
+    RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, ds, f, T, f, h, JPP_EPI_BF16));
+    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), T, f));
+    RC(gemm(st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
+            JPP_EPI_BF16));
+  }
   RC(norm_b(s, st, dn, at(L.h1), nullptr, (float*)at(L.rstd2), s->P(chunk, li, L_rms2), dy,
             wt(W.dh1), s->G(chunk, li, L_rms2), nullptr));
   RC(gemm(st, wt(W.dh1), h, 0, s->P(chunk, li, L_Wo), h, 0, dctx, s->ctxw, T, s->ctxw, h,
@@ -290,6 +350,20 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(wgrad(s, st, at(L.x), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
     return JPP_OK;
   }
+  if (s->d.family == JPP_FAMILY_MIXTRAL) {
+    jpp_moe_args ma;
+    moe_args(s, ma, slot, L, chunk, li);
+    const int E = s->d.n_experts;
+    RC(ggemm(st, JPP_GROUP_K, ma.seg, E, at(L.s), f, 1, wt(W.deo), h, 1, 0, s->G(chunk, li, X_Wd), h,
+             f * h, f, h, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+    RC(ggemm(st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, wt(W.dgu), 2 * f, 1, 0,
+             s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+    RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)wt(W.dlogits), s->G(chunk, li, X_Wr),
+                            s->S<float>(s->s_partial)));
+    RC(wgrad(s, st, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, X_Wo), s->ctxw, h));
+    RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw));
+    return JPP_OK;
+  }
   RC(wgrad(s, st, at(L.s), f, dy, h, s->G(chunk, li, L_Wd), f, h));
   RC(wgrad(s, st, at(L.n2), h, wt(W.dgu), 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f));
   RC(wgrad(s, st, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, L_Wo), s->ctxw, h));
@@ -317,8 +391,18 @@ void carve_layer(jpp_stage* s, Carver& c, LayerStash& L, bool with_w) {
     L.n1 = c.take(T * h * e);
     L.h1 = c.take(T * h * e);
     L.n2 = c.take(T * h * e);
-    L.gu = c.take(T * 2 * f * e);
-    L.s = c.take(T * f * e);
+    if (s->d.family == JPP_FAMILY_MIXTRAL) {
+      const size_t cap = s->cap;
+      L.ids = c.take(T * 2 * 4); L.gates = c.take(T * 2 * 4); L.row_of = c.take(T * 2 * 4);
+      L.tok_of = c.take(cap * 4); L.gate_of = c.take(cap * 4); L.seg = c.take(64 * 4);
+      L.xp = c.take(cap * h * e);
+      L.gu = c.take(cap * 2 * f * e);
+      L.s = c.take(cap * f * e);
+      L.eo = c.take(cap * h * e);
+    } else {
+      L.gu = c.take(T * 2 * f * e);
+      L.s = c.take(T * f * e);
+    }
   }
   if (with_w) {
     // carved by the caller through carve_w
@@ -332,6 +416,12 @@ void carve_w(jpp_stage* s, Carver& c, LayerStash& L) {
     L.dc = c.take(T * h * e);
     L.du = c.take(T * f * e);
     L.da = c.take(T * h * e);
+  } else if (s->d.family == JPP_FAMILY_MIXTRAL) {
+    L.dyin = c.take(T * h * e);
+    L.dgu = c.take(s->cap * 2 * f * e);
+    L.dh1 = c.take(T * h * e);
+    L.deo = c.take(s->cap * h * e);
+    L.dlogits = c.take(T * s->d.n_experts * 4);
   } else {
     L.dyin = c.take(T * h * e);
     L.dgu = c.take(T * 2 * f * e);
@@ -346,8 +436,16 @@ extern "C" {
 int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   JPP_REQUIRE(d && out, "stage_create: null");
   *out = nullptr;
-  JPP_REQUIRE(d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_LLAMA,
-              "stage_create: family %d is not built", d->family);
+  JPP_REQUIRE(d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_LLAMA ||
+                  d->family == JPP_FAMILY_MIXTRAL,
+              "stage_create: unknown family %d", d->family);
+  if (d->family == JPP_FAMILY_MIXTRAL) {
+    JPP_REQUIRE(d->n_experts == 8 && d->top_k == 2,
+                "stage_create: the mixture layer is built for 8 experts, top-2");
+    JPP_REQUIRE(d->hidden % 256 == 0 && d->ffn % 256 == 0,
+                "stage_create: the mixture layer needs hidden and ffn multiples of 256");
+    JPP_REQUIRE(d->fused_wgrad_accum, "stage_create: the mixture layer accumulates in the GEMM");
+  }
   JPP_REQUIRE(d->hidden > 0 && d->n_heads > 0 && d->ffn > 0 && d->seq > 0 && d->batch > 0,
               "stage_create: bad shape");
   JPP_REQUIRE(d->n_chunks > 0 && d->layers_per_chunk > 0 && d->max_live > 0,
@@ -373,7 +471,12 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   s->qkvw = (int64_t)(d->n_heads + 2 * kvh) * hd;
   s->ctxw = (int64_t)d->n_heads * hd;
   const int64_t h = s->h, f = s->f;
-  if (d->family == JPP_FAMILY_BERT)
+  if (d->family == JPP_FAMILY_MIXTRAL) s->cap = jpp_moe_capacity(T, d->n_experts, d->top_k);
+  if (d->family == JPP_FAMILY_MIXTRAL)
+    s->pinfo = {{"rms1_g", 1, h}, {"Wqkv", h, s->qkvw}, {"Wo", s->ctxw, h}, {"rms2_g", 1, h},
+                {"Wr", h, d->n_experts}, {"Wgu", d->n_experts * h, 2 * f},
+                {"Wd", d->n_experts * f, h}};
+  else if (d->family == JPP_FAMILY_BERT)
     s->pinfo = {{"Wqkv", h, 3 * h}, {"bqkv", 1, 3 * h}, {"Wo", h, h}, {"bo", 1, h},
                 {"ln1_g", 1, h}, {"ln1_b", 1, h}, {"W1", h, f}, {"b1", 1, f},
                 {"W2", f, h}, {"b2", 1, h}, {"ln2_g", 1, h}, {"ln2_b", 1, h}};
@@ -402,11 +505,16 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   const size_t e = 2;
   s->s_dx[0] = sc.take(T * h * e);
   s->s_dx[1] = sc.take(T * h * e);
-  s->s_t1 = sc.take(T * (d->family == JPP_FAMILY_BERT ? h : f) * e);
+  const size_t rows_t = d->family == JPP_FAMILY_MIXTRAL ? (size_t)s->cap : (size_t)T;
+  s->s_t1 = sc.take(rows_t * (d->family == JPP_FAMILY_BERT ? h : f) * e);
+  s->s_t4 = sc.take(d->family == JPP_FAMILY_MIXTRAL ? rows_t * h * e : 256);
+  s->s_moework = sc.take(d->family == JPP_FAMILY_MIXTRAL
+                             ? (size_t)2 * ((T + 255) / 256) * d->n_experts * 4 + 256 : 256);
   s->s_t2 = sc.take(T * h * e);
   s->s_t3 = sc.take(T * s->ctxw * e);
   const size_t widest = (size_t)std::max<int64_t>(std::max<int64_t>(s->qkvw, 2 * f), h);
-  s->s_partial = sc.take((size_t)2 * JPP_NORM_PARTIALS * widest * 4);
+  s->s_partial = sc.take(std::max((size_t)2 * JPP_NORM_PARTIALS * widest * 4,
+                                  (size_t)64 * h * 8 * 4));
   s->s_delta = sc.take((size_t)d->batch * d->n_heads * d->seq * 4);
   size_t max_w = 0;
   for (auto& p : s->pinfo) max_w = std::max(max_w, (size_t)(p.rows * p.cols));

@@ -34,7 +34,9 @@ class GemmArgs(C.Structure):
                 ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64),
                 ("ldc2", C.c_int64), ("ldresid", C.c_int64), ("ldaux", C.c_int64),
                 ("trans_a", C.c_int), ("trans_b", C.c_int), ("epilogue", C.c_int),
-                ("gelu_tanh", C.c_int), ("tile", C.c_int)]
+                ("gelu_tanh", C.c_int), ("tile", C.c_int),
+                ("seg", C.c_void_p), ("n_seg", C.c_int), ("group_mode", C.c_int),
+                ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("group_rows", C.c_int64)]
 
 
 class AttnArgs(C.Structure):
@@ -54,6 +56,13 @@ class NormArgs(C.Structure):
                 ("dy", C.c_void_p), ("resid", C.c_void_p), ("dx", C.c_void_p),
                 ("dgamma", C.c_void_p), ("dbeta", C.c_void_p), ("partial", C.c_void_p),
                 ("rows", C.c_int64), ("cols", C.c_int64), ("eps", C.c_float)]
+
+
+class MoeArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("wr", C.c_void_p), ("ids", C.c_void_p), ("gates", C.c_void_p),
+                ("row_of", C.c_void_p), ("tok_of", C.c_void_p), ("gate_of", C.c_void_p),
+                ("seg", C.c_void_p), ("work", C.c_void_p), ("tokens", C.c_int64),
+                ("hidden", C.c_int64), ("n_experts", C.c_int), ("top_k", C.c_int)]
 
 
 class StageDesc(C.Structure):
@@ -78,7 +87,9 @@ EXPORTS = [
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
     "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
-    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
+    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
+    "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
+    "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
     "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
     "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_bytes",
     "jpp_stage_run_task", "jpp_stage_live_slots",
@@ -135,6 +146,18 @@ def load():
                                      C.c_void_p, C.c_void_p]
     lib.jpp_mse_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float,
                                  C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.jpp_moe_capacity.restype = C.c_int64
+    lib.jpp_moe_capacity.argtypes = [C.c_int64, C.c_int, C.c_int]
+    lib.jpp_moe_route.argtypes = [C.c_void_p, C.POINTER(MoeArgs)]
+    lib.jpp_moe_gather.argtypes = [C.c_void_p, C.POINTER(MoeArgs), C.c_void_p, C.c_void_p]
+    lib.jpp_moe_combine_fwd.argtypes = [C.c_void_p, C.POINTER(MoeArgs), C.c_void_p, C.c_void_p,
+                                        C.c_void_p]
+    lib.jpp_moe_bwd_prepare.argtypes = [C.c_void_p, C.POINTER(MoeArgs), C.c_void_p, C.c_void_p,
+                                        C.c_void_p, C.c_void_p]
+    lib.jpp_moe_combine_bwd.argtypes = [C.c_void_p, C.POINTER(MoeArgs), C.c_void_p, C.c_void_p,
+                                        C.c_void_p]
+    lib.jpp_moe_router_wgrad.argtypes = [C.c_void_p, C.POINTER(MoeArgs), C.c_void_p, C.c_void_p,
+                                         C.c_void_p, C.c_void_p]
     lib.jpp_cast_f32_to_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
     lib.jpp_cast_bf16_to_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
     lib.jpp_stage_create.argtypes = [C.POINTER(StageDesc), C.POINTER(C.c_void_p)]
@@ -299,9 +322,10 @@ class probe:
 # ---------------------------------------------------------------------------
 def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, bias=None,
          resid=None, ldresid=0, aux=None, ldaux=0, c2=None, ldc2=0, gelu_tanh=0, tile=0,
-         stream=None):
+         stream=None, seg=None, n_seg=0, group_mode=0, stride_b=0, stride_c=0, group_rows=0):
     g = GemmArgs(a, b, c, c2, bias, resid, aux, m, n, k, lda, ldb, ldc, ldc2, ldresid, ldaux,
-                 int(trans_a), int(trans_b), epilogue, gelu_tanh, tile)
+                 int(trans_a), int(trans_b), epilogue, gelu_tanh, tile, seg, n_seg, group_mode,
+                 stride_b, stride_c, group_rows)
     check(load().jpp_gemm_bf16(stream, C.byref(g)))
 
 

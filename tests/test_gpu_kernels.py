@@ -239,3 +239,126 @@ def test_swiglu_rope_accum_colsum_cast():
     rt.sync()
     np.testing.assert_array_equal(bdst.download(np.uint16, (1001,)), L.f32_to_bf16_bits(src))
     np.testing.assert_array_equal(rt.to_bf16_bits(src), L.f32_to_bf16_bits(src))
+
+
+def moe_setup(rng, T, h):
+    lib = rt.load()
+    E = 8
+    x = rnd(rng, T, h)
+    wr = rnd(rng, h, E, scale=1.0 / math.sqrt(h))
+    cap = lib.jpp_moe_capacity(T, E, 2)
+    bufs = dict(x=dev_bf16(x), wr=dev_bf16(wr), ids=rt.DeviceBuffer(T * 8),
+                gates=rt.DeviceBuffer(T * 8), row_of=rt.DeviceBuffer(T * 8),
+                tok_of=rt.DeviceBuffer(cap * 4), gate_of=rt.DeviceBuffer(cap * 4),
+                seg=rt.DeviceBuffer(64 * 4), work=rt.DeviceBuffer(2 * ((T + 255) // 256) * E * 4 + 256))
+    a = rt.MoeArgs(bufs["x"].ptr, bufs["wr"].ptr, bufs["ids"].ptr, bufs["gates"].ptr,
+                   bufs["row_of"].ptr, bufs["tok_of"].ptr, bufs["gate_of"].ptr, bufs["seg"].ptr,
+                   bufs["work"].ptr, T, h, E, 2)
+    return lib, a, bufs, x, wr, cap
+
+
+def test_moe_routing_and_permutation():
+    rng = np.random.default_rng(11)
+    T, h, E = 1000, 256, 8
+    lib, a, b, x, wr, cap = moe_setup(rng, T, h)
+    rt.check(lib.jpp_moe_route(None, C.byref(a)))
+    rt.sync()
+    ids = b["ids"].download(np.int32, (T, 2))
+    gates = b["gates"].download(np.float32, (T, 2))
+    logits = (x.astype(np.float64) @ wr.astype(np.float64))
+    ids_w, gates_w = L.moe_route(logits, 2)
+    # a routing decision may differ only where two logits are within rounding of each other
+    diff = np.nonzero((ids != ids_w).any(1))[0]
+    for t in diff:
+        top3 = np.sort(logits[t])[::-1][:3]
+        assert min(top3[0] - top3[1], top3[1] - top3[2]) < 1e-4, (t, top3)
+    same = np.setdiff1d(np.arange(T), diff)
+    np.testing.assert_allclose(gates[same], gates_w[same], rtol=1e-4, atol=1e-6)
+    seg = b["seg"].download(np.int32, (E + 1,))
+    row_of = b["row_of"].download(np.int32, (T, 2))
+    tok_of = b["tok_of"].download(np.int32, (cap,))
+    gate_of = b["gate_of"].download(np.float32, (cap,))
+    assert seg[0] == 0 and (seg % 256 == 0).all() and seg[E] <= cap
+    for e in range(E):
+        toks = np.nonzero((ids == e).any(1))[0]            # token order inside the group
+        rows = np.arange(seg[e], seg[e] + len(toks))
+        np.testing.assert_array_equal(tok_of[rows], toks)
+        assert (tok_of[seg[e] + len(toks):seg[e + 1]] == -1).all()
+        slot = (ids[toks] == e).argmax(1)
+        np.testing.assert_array_equal(row_of[toks, slot], rows)
+        np.testing.assert_array_equal(gate_of[rows], gates[toks, slot])
+
+    # gather / combine forward / backward helpers
+    xp = rt.DeviceBuffer(cap * h * 2)
+    rt.check(lib.jpp_moe_gather(None, C.byref(a), b["x"].ptr, xp.ptr))
+    rt.sync()
+    xp_h = xp.download_bf16((cap, h))
+    valid = tok_of >= 0
+    np.testing.assert_array_equal(xp_h[:seg[E]][valid[:seg[E]]], x[tok_of[:seg[E]][valid[:seg[E]]]])
+    assert not xp_h[:seg[E]][~valid[:seg[E]]].any()
+    eo, resid, dy = rnd(rng, cap, h), rnd(rng, T, h), rnd(rng, T, h)
+    b_eo, b_res, b_dy = dev_bf16(eo), dev_bf16(resid), dev_bf16(dy)
+    y = rt.DeviceBuffer(T * h * 2)
+    rt.check(lib.jpp_moe_combine_fwd(None, C.byref(a), b_eo.ptr, b_res.ptr, y.ptr))
+    want = resid + gates[:, :1] * eo[row_of[:, 0]] + gates[:, 1:] * eo[row_of[:, 1]]
+    rt.sync()
+    close(y.download_bf16((T, h)), want, 1e-2, "moe combine")
+    dlog, deo = rt.DeviceBuffer(T * E * 4), rt.DeviceBuffer(cap * h * 2)
+    rt.check(lib.jpp_moe_bwd_prepare(None, C.byref(a), b_dy.ptr, b_eo.ptr, dlog.ptr, deo.ptr))
+    rt.sync()
+    dgate = np.stack([(dy * eo[row_of[:, k]]).sum(-1) for k in range(2)], -1)
+    dsel = gates * (dgate - (gates * dgate).sum(-1, keepdims=True))
+    dl_w = np.zeros((T, E), np.float32)
+    np.put_along_axis(dl_w, ids.astype(np.int64), dsel, -1)
+    close(dlog.download(np.float32, (T, E)), dl_w, 1e-4, "dlogits")
+    deo_w = np.zeros((cap, h), np.float32)
+    deo_w[row_of[:, 0]] = gates[:, :1] * dy
+    deo_w[row_of[:, 1]] = gates[:, 1:] * dy
+    close(deo.download_bf16((cap, h))[:seg[E]], deo_w[:seg[E]], 1e-2, "deo")
+    dx = rt.DeviceBuffer(T * h * 2)
+    rt.check(lib.jpp_moe_combine_bwd(None, C.byref(a), b_eo.ptr, dlog.ptr, dx.ptr))
+    rt.sync()
+    close(dx.download_bf16((T, h)), eo[row_of[:, 0]] + eo[row_of[:, 1]] + dl_w @ wr.T, 1e-2, "moe dx")
+    acc0 = rng.standard_normal((h, E)).astype(np.float32)
+    acc, part = rt.DeviceBuffer.from_numpy(acc0), rt.DeviceBuffer(64 * h * E * 4)
+    rt.check(lib.jpp_moe_router_wgrad(None, C.byref(a), b["x"].ptr, dlog.ptr, acc.ptr, part.ptr))
+    rt.sync()
+    close(acc.download(np.float32, (h, E)), acc0 + x.T @ dl_w, 1e-4, "dWr")
+
+
+def test_grouped_gemm():
+    rng = np.random.default_rng(12)
+    E, h, f = 8, 256, 512
+    counts = [300, 0, 256, 17, 700, 1, 255, 512]
+    seg = np.zeros(E + 1, np.int32)
+    for e, c in enumerate(counts):
+        seg[e + 1] = seg[e] + (c + 255) // 256 * 256
+    cap = int(seg[E]) + 512                      # capacity beyond the last group
+    xp = np.zeros((cap, h), np.float32)
+    for e, c in enumerate(counts):
+        xp[seg[e]:seg[e] + c] = rnd(rng, c, h)
+    w = rnd(rng, E, h, f, scale=0.1)
+    b_seg, b_xp, b_w = rt.DeviceBuffer.from_numpy(seg), dev_bf16(xp), dev_bf16(w)
+    out = rt.DeviceBuffer(cap * f * 2)
+    out.zero()
+    rt.gemm(b_xp.ptr, b_w.ptr, out.ptr, cap, f, h, h, f, f, 0, 1, rt.EPI_BF16, seg=b_seg.ptr, n_seg=E,
+            group_mode=1, stride_b=h * f)
+    rt.sync()
+    got = out.download_bf16((cap, f))
+    for e in range(E):
+        if counts[e]:
+            close(got[seg[e]:seg[e + 1]], xp[seg[e]:seg[e + 1]] @ w[e], 1e-2, f"group {e}")
+    assert not got[seg[E]:].any(), "tiles past the last group must not be written"
+    # weight gradients: per-expert contraction over the expert's rows, accumulated
+    dy = np.zeros((cap, f), np.float32)
+    dy[:seg[E]] = rnd(rng, int(seg[E]), f)
+    acc0 = rng.standard_normal((E, h, f)).astype(np.float32)
+    b_dy, b_acc = dev_bf16(dy), rt.DeviceBuffer.from_numpy(acc0)
+    rt.gemm(b_xp.ptr, b_dy.ptr, b_acc.ptr, h, f, 0, h, f, f, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
+            n_seg=E, group_mode=2, stride_c=h * f)
+    rt.sync()
+    got = b_acc.download(np.float32, (E, h, f))
+    for e in range(E):
+        want = acc0[e] + xp[seg[e]:seg[e + 1]].T @ dy[seg[e]:seg[e + 1]]
+        close(got[e], want, 1e-3, f"dW group {e}")
+    np.testing.assert_array_equal(got[1], acc0[1])       # empty group: untouched

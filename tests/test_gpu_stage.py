@@ -21,6 +21,8 @@ BERT = LayerSpec("bert", 128, 2, 256, 128, 1, eps=1e-12)
 BERT_TANH = LayerSpec("bert", 256, 4, 512, 128, 2, eps=1e-6, gelu_tanh=True)
 LLAMA = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
                   rope_theta=5e5, eps=1e-5)
+MIXTRAL = LayerSpec("mixtral", 256, 2, 256, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
+                    rope_theta=5e5, eps=1e-5, n_experts=8, top_k=2)
 LLAMA_D64 = LayerSpec("llama", 256, 4, 256, 256, 1, n_kv_heads=2, head_dim=64, causal=True,
                       rope_theta=1e4, eps=1e-5)
 
@@ -88,6 +90,8 @@ CASES = [
     ("llama-zb-first-stage", LLAMA, S.ZeroBubble(2), 2, 0, 1),
     ("llama-d64-zb", LLAMA_D64, S.ZeroBubble(3), 3, 1, 2),
     ("llama-dualpipev", LLAMA, S.DualPipeV(4, 2), 4, 1, 1),
+    ("mixtral-1f1b", MIXTRAL, S.Std1F1B(2), 3, 1, 2),
+    ("mixtral-dualpipev", MIXTRAL, S.DualPipeV(4, 2), 4, 0, 1),
 ]
 
 
@@ -104,10 +108,25 @@ def test_stage_matches_oracle(name, spec, sched, n, rank, lpc):
         close(ys[k], ys_w[k], 2e-2, f"y{k}")
     for k in dxs_w:
         close(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
+    bad = []
     for s in plan.stages:
         for li in range(lpc):
             for pname, want in acc_w[s][li].items():
-                close(grads[s][li][pname], want, 2e-2, f"grad {s}/{li}/{pname}")
+                got = grads[s][li][pname]
+                want = want.reshape(got.shape)
+                err = float(np.abs(got - want).max()) / (float(np.abs(want).max()) + 1e-30)
+                fro = float(np.linalg.norm(got - want) / (np.linalg.norm(want) + 1e-30))
+                # Top-2 expert selection is discontinuous: a token whose second and third
+                # router logits are within bf16 rounding of each other may go to another
+                # expert than in the oracle (1-2 of 256 tokens flip between the oracle's own
+                # bf16 and f32 numerics).  One token's outer product then lands in another
+                # expert's gradient, so router and expert weights are held to 2e-2 in the
+                # Frobenius norm and 1e-1 in the max norm; all else to 2e-2 in the max norm.
+                routed = spec.family == "mixtral" and pname in ("Wr", "Wgu", "Wd")
+                ok = (fro <= 2e-2 and err <= 1e-1) if routed else err <= 2e-2
+                if not (np.isfinite(got).all() and ok):
+                    bad.append(f"grad {s}/{li}/{pname}: max err {err:.4g}, frobenius {fro:.4g}")
+    assert not bad, "\n".join(bad)
 
 
 def test_task_order_does_not_change_gradients():
