@@ -207,6 +207,14 @@ __device__ __forceinline__ void dma_load16(const bf16_t* base, uint32_t off, uin
                : "memory");
 }
 __device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// waits until at most PENDING of this wave's most recent loads are outstanding
+template <int PENDING>
+__device__ __forceinline__ void dma_wait() {
+  static_assert(PENDING >= 0 && PENDING < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PENDING) : "memory");
+}
+// waits for this wave's LDS reads, so that what they read may be overwritten
+__device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 template <int ROWS, bool MC, int NW = 4>
 struct DmaTile {
@@ -239,6 +247,15 @@ struct DmaTile {
 #pragma unroll
     for (int i = FIRST; i < FIRST + COUNT; ++i)
       dma_load16(src, off[i], tile + (wave * INSTS + i) * 1024);
+  }
+
+  // loads part*COUNT .. part*COUNT+COUNT-1 (`part` constant after unrolling)
+  template <int COUNT>
+  static __device__ __forceinline__ void issue_part(int part, const bf16_t* src, const Offsets& off,
+                                                    uint32_t tile, int wave) {
+#pragma unroll
+    for (int i = 0; i < COUNT; ++i)
+      dma_load16(src, off[part * COUNT + i], tile + (wave * INSTS + part * COUNT + i) * 1024);
   }
 
   // MFMA operand fragment: rows row0 .. row0+31 of the operand, K-step ks

@@ -128,54 +128,72 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   TileA::offsets(offa, p.lda, wave, lane);
   TileB::offsets(offb, p.ldb, wave, lane);
   constexpr int IA = TileA::INSTS, IB = TileB::INSTS;
+  const int row_w = wn * (BN / WN), row_x = wm * (BM / 2);
+
+  // Software pipeline over K-steps of 64 with two LDS stages:
+  //   * the HBM -> LDS copy of K-step t+2 is issued inside K-step t, right after the
+  //     barrier that retires stage t&1's readers, so it has a whole K-step to land;
+  //   * that barrier sits in front of the last of the four MFMA blocks of a K-step and the
+  //     first fragments of K-step t+1 are read from LDS behind it, under those MFMAs.
+  bf16x8 fw[2][TN], fx[2][TM];
   if (kt_n > 0) {
     TileA::template issue<0, IA>(uniform_ptr(a_src), offa, lds0, wave);
     TileB::template issue<0, IB>(uniform_ptr(b_src), offb, lds0 + A_BYTES, wave);
+    const int k1 = min(1, kt_n - 1);
+    TileA::template issue<0, IA>(uniform_ptr(a_src + k1 * a_step), offa, lds0 + STAGE, wave);
+    TileB::template issue<0, IB>(uniform_ptr(b_src + k1 * b_step), offb, lds0 + STAGE + A_BYTES, wave);
+    dma_wait<IA + IB>();   // stage 0 has landed; stage 1 may still be in flight
   }
-  dma_wait_all();
   __syncthreads();
+#pragma unroll
+  for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag(smem + A_BYTES, row_w + j * 32, 0, lane);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) fx[0][i] = TileA::frag(smem, row_x + i * 32, 0, lane);
 
   for (int kt = 0; kt < kt_n; ++kt) {
     const uint8_t* sa = smem + (kt & 1) * STAGE;
     const uint8_t* sb = sa + A_BYTES;
-    // The other stage was last read one iteration ago (barrier below): it is
-    // refilled with the next K-step straight from HBM while this one is
-    // multiplied.  The last iteration re-reads its own step, unused.
-    const int kn = min(kt + 1, kt_n - 1);
-    const uint32_t da = lds0 + ((kt + 1) & 1) * STAGE;
+    const uint8_t* na = smem + ((kt + 1) & 1) * STAGE;
+    // past the end the last K-step is fetched again, unused
+    const int kn = min(kt + 2, kt_n - 1);
     const bf16_t* ga = uniform_ptr(a_src + (long)kn * a_step);
     const bf16_t* gb = uniform_ptr(b_src + (long)kn * b_step);
-
-    bf16x8 fw[2][TN], fx[2][TM];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag(sb, wn * (BN / WN) + j * 32, 0, lane);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fx[0][i] = TileA::frag(sa, wm * (BM / 2) + i * 32, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
       if (ks < 3) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          fw[nxt][j] = TileB::frag(sb, wn * (BN / WN) + j * 32, ks + 1, lane);
+        for (int j = 0; j < TN; ++j) fw[nxt][j] = TileB::frag(sb, row_w + j * 32, ks + 1, lane);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-          fx[nxt][i] = TileA::frag(sa, wm * (BM / 2) + i * 32, ks + 1, lane);
+        for (int i = 0; i < TM; ++i) fx[nxt][i] = TileA::frag(sa, row_x + i * 32, ks + 1, lane);
+      } else {
+        // every fragment of this stage is in registers: once all waves are here (and the
+        // other stage, requested one K-step ago, has landed) this stage can be refilled
+        dma_wait_all();
+        lds_wait_all();
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fw[nxt][j] = TileB::frag(na + A_BYTES, row_w + j * 32, 0, lane);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fx[nxt][i] = TileA::frag(na, row_x + i * 32, 0, lane);
       }
-      // the HBM -> LDS loads of the next K-step go out under the first two
-      // MFMA blocks, leaving them the rest of the iteration to land
-      if (ks == 0) TileA::template issue<0, IA>(ga, offa, da, wave);
-      if (ks == 1) TileB::template issue<0, IB>(gb, offb, da + A_BYTES, wave);
+      // the refill of the retired stage is spread over this block's MFMAs: a wave that
+      // issues its loads back to back waits on the memory pipeline with its MFMAs behind it
+      static_assert(IA % TM == 0 && IB % TM == 0, "loads per wave must split over the MFMA rows");
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i) {
+        if (ks == 3) {
+          TileA::template issue_part<IA / TM>(i, ga, offa, lds0 + (kt & 1) * STAGE, wave);
+          TileB::template issue_part<IB / TM>(i, gb, offb, lds0 + (kt & 1) * STAGE + A_BYTES, wave);
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cur][j], fx[cur][i], acc[i][j],
                                                               0, 0, 0);
+      }
     }
-    dma_wait_all();
-    __syncthreads();
   }
+  dma_wait_all();   // the refetches of the last two K-steps must not outlive the block's LDS
 
   // epilogue: lane holds m = base_m + (lane & 31), and for g = 0..3 the four
   // columns base_n + 8 g + 4 (lane >> 5) + {0,1,2,3}
