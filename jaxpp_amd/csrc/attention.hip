@@ -58,6 +58,17 @@ __device__ __forceinline__ bf16x8 slabs_frag(const uint8_t* slabs, int row0, int
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Makes the compiler wait here for the loads that produce these registers.  Without it the
+// wait lands at their first use inside the main loop as a vmcnt count, and there it also
+// waits for the HBM -> LDS copies of the next tile, which the wave has just issued (vmcnt
+// counts every vector memory operation of the wave, in order).
+template <int N>
+__device__ __forceinline__ void settle(bf16x8 (&f)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i]));
+}
+__device__ __forceinline__ void settle(float& x) { asm volatile("" : "+v"(x)); }
+
 // HBM -> LDS copy of a [64][D] tile (row stride ld) by the 4 waves of a
 // workgroup, as D/64 swizzled slabs; no registers involved.
 using Tile64 = DmaTile<64, false>;
@@ -67,6 +78,25 @@ __device__ __forceinline__ void dma_tile(const bf16_t* src, const Tile64::Offset
 #pragma unroll
   for (int c = 0; c < D / 64; ++c)
     Tile64::issue<0, Tile64::INSTS>(uniform_ptr(src + c * 64), off, lds + c * 8192, wave);
+}
+
+// Which (block, head, batch) a workgroup works on.  Workgroups are handed to the 8 XCDs
+// round robin in launch order, and each XCD has its own L2: the launch order is rearranged
+// so that one XCD sees only 1/8 of the (head, batch) pairs - adjacent heads, which share
+// their K/V under grouped-query attention - and its K/V working set stays in its L2.
+// Within an XCD blocks still go out in increasing x for all its heads (heavy first).
+struct Work { int x, h, b; };
+__device__ __forceinline__ Work xcd_work() {
+  const int gx = gridDim.x, gy = gridDim.y;
+  const int pairs = gy * gridDim.z;
+  int x = blockIdx.x, pair = blockIdx.y + gy * blockIdx.z;
+  if ((pairs & 7) == 0) {
+    const int l = x + gx * pair, per = pairs >> 3;
+    const int xcd = l & 7, j = l >> 3;
+    x = j / per;
+    pair = xcd * per + j % per;
+  }
+  return {x, pair % gy, pair / gy};
 }
 
 // ---------------------------------------------------------------------------
@@ -83,8 +113,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: scalar branches and addresses
-  const int qb = CAUSAL ? (gridDim.x - 1 - blockIdx.x) : blockIdx.x;  // heavy blocks first
-  const int h = blockIdx.y, b = blockIdx.z;
+  const Work w = xcd_work();
+  const int qb = CAUSAL ? (gridDim.x - 1 - w.x) : w.x;  // heavy blocks first
+  const int h = w.h, b = w.b;
   const int hk = h / (p.n_heads / p.n_kv_heads);
   const long row0 = (long)b * p.seq;
   const int q0 = qb * 128 + wave * 32;
@@ -96,6 +127,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = global_frag(qbase, p.ldq, ks, lane);
   }
+  settle(qf);
 
   f32x16 oacc[DT];
 #pragma unroll
@@ -129,16 +161,30 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
       dma_tile<D>(vbase + kn * p.ldv, offv, dst + TILE, wave);
     }
     if (!(CAUSAL && k0 > q0 + 31)) {  // else: whole block above this wave's diagonal
+      // Fragments are read from LDS in batches ahead of the MFMAs that consume them, so
+      // the MFMAs wait for the oldest read only (LDS returns in order), not for each one.
       f32x16 s[2];
+      {
+        bf16x8 kfr[2][KS];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+          for (int ks = 0; ks < KS; ++ks) kfr[t][ks] = slabs_frag<D>(lds_k, t * 32, ks, lane);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-          s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_k, t * 32, ks, lane),
-                                                         qf[ks], s[t], 0, 0, 0);
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks)
+            s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[t][ks], qf[ks], s[t], 0, 0, 0);
+        }
       }
+      // V^T fragments: requested now, they arrive under the softmax arithmetic
+      bf16x8 vfr[4][DT];
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+#pragma unroll
+        for (int i = 0; i < DT; ++i) vfr[st][i] = slab_frag_tr(lds_v, 64, i * 32, st, lane);
       if (CAUSAL && k0 + 63 > q0) {  // block touches the diagonal
         // the empty asm keeps this wave-uniform branch a branch (not selects on every block)
         asm volatile("" ::: "memory");
@@ -182,8 +228,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
         const bf16x8 pf = acc_to_frag(s[st >> 1], (st & 1) * 8);
 #pragma unroll
         for (int i = 0; i < DT; ++i)
-          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slab_frag_tr(lds_v, 64, i * 32, st, lane),
-                                                            pf, oacc[i], 0, 0, 0);
+          oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[st][i], pf, oacc[i], 0, 0, 0);
       }
     }
     dma_wait_all();
@@ -248,8 +293,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: scalar branches and addresses
-  const int qb = CAUSAL ? (gridDim.x - 1 - blockIdx.x) : blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z;
+  const Work w = xcd_work();
+  const int qb = CAUSAL ? (gridDim.x - 1 - w.x) : w.x;
+  const int h = w.h, b = w.b;
   const int hk = h / (p.n_heads / p.n_kv_heads);
   const long row0 = (long)b * p.seq;
   const int q0 = qb * 128 + wave * 32;
@@ -266,9 +312,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
     }
   }
   const long stat = ((long)b * p.n_heads + h) * p.seq + qi;
-  const float lse2 = p.lse[stat] * kLog2e;
-  const float dlt = p.delta[stat];
+  float lse2 = p.lse[stat] * kLog2e;
+  float dlt = p.delta[stat];
   const float sc = p.scale * kLog2e;
+  settle(qf);
+  settle(dof);
+  settle(lse2);
+  settle(dlt);
 
   f32x16 dqacc[DT];
 #pragma unroll
@@ -304,15 +354,26 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {  // 32 keys at a time keeps the live scores small
         f32x16 s, dp;
+        {
+          bf16x8 kfr[KS], vfr[KS];  // read ahead of the MFMAs that consume them
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+          for (int ks = 0; ks < KS; ++ks) {
+            kfr[ks] = slabs_frag<D>(lds_k, t * 32, ks, lane);
+            vfr[ks] = slabs_frag<D>(lds_v, t * 32, ks, lane);
+          }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_k, t * 32, ks, lane),
-                                                      qf[ks], s, 0, 0, 0);
-          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_v, t * 32, ks, lane),
-                                                       dof[ks], dp, 0, 0, 0);
+          for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[ks], qf[ks], s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[ks], dof[ks], dp, 0, 0, 0);
+          }
         }
+        bf16x8 ktr[2][DT];  // K^T fragments arrive under the elementwise arithmetic
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+          for (int i = 0; i < DT; ++i) ktr[h2][i] = slab_frag_tr(lds_k, 64, i * 32, 2 * t + h2, lane);
         if (diag) {  // wave-uniform; the empty asm keeps it a branch
           asm volatile("" ::: "memory");
 #pragma unroll
@@ -331,8 +392,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
           const bf16x8 dsf = acc_to_frag(s, h2 * 8);
 #pragma unroll
           for (int i = 0; i < DT; ++i)
-            dqacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                slab_frag_tr(lds_k, 64, i * 32, 2 * t + h2, lane), dsf, dqacc[i], 0, 0, 0);
+            dqacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr[h2][i], dsf, dqacc[i], 0, 0, 0);
         }
       }
     }
@@ -380,7 +440,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ksb = wave & 1, half = wave >> 1;
-  const int hk = blockIdx.y, b = blockIdx.z;
+  const Work w = xcd_work();
+  const int hk = w.h, b = w.b;
   const int grp = p.n_heads / p.n_kv_heads;
   const long row0 = (long)b * p.seq;
   const int nkb = p.seq / 64;
@@ -394,7 +455,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
   Tile64H::offsets(offdo, p.lddo, ksb, lane);
 
   for (int seg = 0; seg < (CAUSAL ? 2 : 1); ++seg) {
-    const int kb = CAUSAL ? (seg == 0 ? (int)blockIdx.x : nkb - 1 - (int)blockIdx.x) : (int)blockIdx.x;
+    const int kb = CAUSAL ? (seg == 0 ? w.x : nkb - 1 - w.x) : w.x;
     const int k0 = kb * 64 + ksb * 32;
     const int ki = k0 + (lane & 31);
 
@@ -408,6 +469,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
         vf[ks] = global_frag(vbase, p.ldv, ks, lane);
       }
     }
+    settle(kf);
+    settle(vf);
     f32x16 dkacc[DT], dvacc[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i)
@@ -416,7 +479,10 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
 
     const int qblk0 = CAUSAL ? kb : 0;
     const int nqb = nkb - qblk0;
-    const int total = grp * nqb;          // (head, query block) pairs to visit
+    // (query block, head) pairs to visit: from the last query block down, heads innermost.
+    // Every workgroup of a kv head starts at the same tiles and walks them at the same
+    // pace, so a tile is fetched into the XCD's L2 once and found there by the others.
+    const int total = grp * nqb;
     const int trips = (total + 1) / 2;    // per wave pair; the last one may be empty for pair 1
 
     // Q / dO tiles go HBM -> LDS directly; the 64 lse and 64 delta values of a
@@ -425,29 +491,46 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
     float rstat = 0.f;
     auto fetch = [&](int trip, int stage) {
       const int it = min(2 * trip + half, total - 1);
-      const int hh = hk * grp + it / nqb;
-      const long q0 = (long)(qblk0 + it % nqb) * 64;
+      const int hh = hk * grp + it % grp;
+      const long q0 = (long)(nkb - 1 - it / grp) * 64;
       const long stat = ((long)b * p.n_heads + hh) * p.seq + q0;
-      rstat = ht < 64 ? p.lse[stat + ht] * kLog2e : p.delta[stat + ht - 64];
+      // one unconditional load, consumed only in park(): nothing in between waits for it
+      rstat = *(ht < 64 ? p.lse + stat + ht : p.delta + stat + (ht - 64));
       const uint32_t dst = lds0 + stage * STAGE;
       dma_tile_pair<D>(p.q + (row0 + q0) * p.ldq + hh * D, offq, dst, ksb);
       dma_tile_pair<D>(p.d_o + (row0 + q0) * p.lddo + hh * D, offdo, dst + TILE, ksb);
     };
-    auto park = [&](int stage) { ((float*)(my + stage * STAGE + 2 * TILE))[ht] = rstat; };
+    auto park = [&](int stage) {
+      ((float*)(my + stage * STAGE + 2 * TILE))[ht] = ht < 64 ? rstat * kLog2e : rstat;
+    };
 
     // one 32-query tile against this wave's 32 keys
     auto tile = [&](bool diag, const uint8_t* lds_q, const uint8_t* lds_do, const float* lds_lse,
                     const float* lds_delta, int q0, int t) {
       f32x16 s, dp;
+      {
+        bf16x8 qfr[KS], dofr[KS];  // read ahead of the MFMAs that consume them
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+        for (int ks = 0; ks < KS; ++ks) {
+          qfr[ks] = slabs_frag<D>(lds_q, t * 32, ks, lane);
+          dofr[ks] = slabs_frag<D>(lds_do, t * 32, ks, lane);
+        }
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_q, t * 32, ks, lane), kf[ks],
-                                                    s, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(slabs_frag<D>(lds_do, t * 32, ks, lane),
-                                                     vf[ks], dp, 0, 0, 0);
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[ks], kf[ks], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dofr[ks], vf[ks], dp, 0, 0, 0);
+        }
       }
+      bf16x8 dotr[2][DT], qtr[2][DT];  // transposed fragments arrive under the arithmetic below
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+        for (int i = 0; i < DT; ++i) {
+          dotr[h2][i] = slab_frag_tr(lds_do, 64, i * 32, 2 * t + h2, lane);
+          qtr[h2][i] = slab_frag_tr(lds_q, 64, i * 32, 2 * t + h2, lane);
+        }
       if (CAUSAL && diag) {
         // only tiles on the diagonal pay for the mask: the empty asm keeps the compiler from
         // turning this (wave-uniform) branch into selects on every tile
@@ -479,10 +562,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
         const bf16x8 dsf = acc_to_frag(dp, h2 * 8);
 #pragma unroll
         for (int i = 0; i < DT; ++i) {
-          dvacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              slab_frag_tr(lds_do, 64, i * 32, 2 * t + h2, lane), pf, dvacc[i], 0, 0, 0);
-          dkacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              slab_frag_tr(lds_q, 64, i * 32, 2 * t + h2, lane), dsf, dkacc[i], 0, 0, 0);
+          dvacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dotr[h2][i], pf, dvacc[i], 0, 0, 0);
+          dkacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[h2][i], dsf, dkacc[i], 0, 0, 0);
         }
       }
     };
@@ -494,7 +575,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
 
     for (int trip = 0; trip < trips; ++trip) {
       const int it = 2 * trip + half;
-      const int q0 = (qblk0 + it % nqb) * 64;
+      const int q0 = (nkb - 1 - it / grp) * 64;
       const uint8_t* lds_q = my + (trip & 1) * STAGE;
       const uint8_t* lds_do = lds_q + TILE;
       const float* lds_lse = (const float*)(lds_do + TILE);
@@ -562,7 +643,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int kb = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  const Work w = xcd_work();
+  const int kb = w.x, hk = w.h, b = w.b;
   const int grp = p.n_heads / p.n_kv_heads;
   const long row0 = (long)b * p.seq;
   const int k0 = kb * 128 + wave * 32;
@@ -578,6 +660,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
       vf[ks] = global_frag(vbase, p.ldv, ks, lane);
     }
   }
+  settle(kf);
+  settle(vf);
   f32x16 dkacc[DT], dvacc[DT];
 #pragma unroll
   for (int i = 0; i < DT; ++i)
@@ -601,15 +685,16 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
     const int hh = hk * grp + it / nqb;
     const long q0 = (long)(qblk0 + it % nqb) * 64;
     const long stat = ((long)b * p.n_heads + hh) * p.seq + q0;
-    if (tid < 64) rstat = p.lse[stat + tid] * kLog2e;
-    else if (tid < 128) rstat = p.delta[stat + tid - 64];
+    // one unconditional load, consumed only in park(): nothing in between waits for it
+    const int st = tid & 127;
+    rstat = *(st < 64 ? p.lse + stat + st : p.delta + stat + (st - 64));
     const uint32_t dst = lds0 + stage * STAGE;
     dma_tile<D>(p.q + (row0 + q0) * p.ldq + hh * D, offq, dst, wave);
     dma_tile<D>(p.d_o + (row0 + q0) * p.lddo + hh * D, offdo, dst + TILE, wave);
   };
   auto park = [&](int stage) {
     float* st = (float*)(smem + stage * STAGE + 2 * TILE);
-    if (tid < 128) st[tid] = rstat;
+    if (tid < 128) st[tid] = tid < 64 ? rstat * kLog2e : rstat;
   };
 
   fetch(0, 0);
