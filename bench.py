@@ -39,13 +39,14 @@ def synthetic_pool(n_elems: int, std: float, seed: int) -> np.ndarray:
 class Workbench:
     """Device state of one workload: executor, parameters, boundary tensors."""
 
-    def __init__(self, wl, fused=True):
+    def __init__(self, wl, fused=True, two_streams=True):
         self.wl = wl
         spec = wl.layer
         sched = getattr(S, wl.schedule)(**wl.schedule_kwargs)
         self.plan = make_rank_plan(sched, wl.n_mubatches, wl.rank)
         self.ex = rt.StageExecutor(spec, self.plan.n_chunks, wl.layers_per_stage,
-                                   self.plan.max_live, self.plan.split_backward, fused)
+                                   self.plan.max_live, self.plan.split_backward, fused,
+                                   two_streams)
         lib = rt.load()
         # parameters: slices of one N(0, 0.02^2) pool at per-tensor offsets;
         # norm gains one, biases zero
@@ -100,6 +101,7 @@ class Workbench:
                 ex.run_task(pt.exec_kind, pt.chunk, m)
             else:
                 ex.run_task(pt.exec_kind, pt.chunk, m, self.dy_in[pt.chunk, m].ptr, self.out.ptr)
+        ex.join()                             # the step ends when the last weight gradient has landed
 
     def step_flops(self) -> float:
         wl = self.wl
@@ -161,6 +163,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused-accumulate", action="store_true",
                     help="bf16 weight gradient + separate fp32 accumulate pass")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="weight gradients on the caller's stream instead of a second one")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -169,7 +173,7 @@ def main():
         sys.exit(2)
     rt.require_gpu()
     wl = workloads()[args.workload]
-    wb = Workbench(wl, fused=not args.unfused_accumulate)
+    wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=not args.single_stream)
     cls = args.probe or dominant_gemm_class(wl)
 
     for _ in range(args.warmup):
@@ -202,6 +206,7 @@ def main():
             "layers": wl.layers_per_stage * wb.plan.n_chunks,
             "peak_live_microbatches": wb.plan.max_live,
             "fused_wgrad_accumulate": not args.unfused_accumulate,
+            "weight_gradient_stream": not args.single_stream,
             "device_bytes": wb.ex.nbytes,
         },
         "algorithmic_flops_per_step": flops,

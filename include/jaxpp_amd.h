@@ -248,6 +248,11 @@ typedef struct {
   int split_backward;    /* 1: BWD_I / BWD_W tasks will be issued separately */
   int fused_wgrad_accum; /* 1: accumulate in the weight-gradient GEMM epilogue;
                             0: bf16 gradient then jpp_grad_accum_f32 */
+  int two_streams;       /* 1: weight-gradient work (BWD_W tasks, and the weight-gradient half
+                            of BWD tasks) runs on a second HIP stream owned by the stage, forked
+                            from and ordered against the caller's stream with events; it may
+                            still be running when jpp_stage_run_task returns control of the
+                            caller's stream - see jpp_stage_join */
 } jpp_stage_desc;
 
 int jpp_stage_create(const jpp_stage_desc* desc, jpp_stage** out);
@@ -260,6 +265,10 @@ int jpp_stage_param_info(const jpp_stage* stage, int index, const char** name, i
 int jpp_stage_param_ptr(jpp_stage* stage, int chunk, int layer, int index, void** ptr);
 int jpp_stage_grad_ptr(jpp_stage* stage, int chunk, int layer, int index, float** ptr);
 int jpp_stage_zero_grads(jpp_stage* stage, void* stream);
+/* Makes `stream` wait for everything the stage has in flight on its own stream (weight
+ * gradients, with two_streams).  Call it before reading the accumulators on `stream`;
+ * jpp_stage_zero_grads does it by itself.  A no-op without two_streams. */
+int jpp_stage_join(jpp_stage* stage, void* stream);
 size_t jpp_stage_bytes(const jpp_stage* stage);
 /* One task.  `in` is the incoming boundary activation (FWD) or cotangent
  * (BWD, BWD_I), `out` receives the outgoing activation / cotangent; both are

@@ -82,9 +82,24 @@ struct jpp_stage {
   // scratch shared by all tasks (stream ordered)
   uint8_t* scratch = nullptr;
   size_t scratch_bytes = 0;
-  LayerStash wshared;              // cotangent buffers when the backward is not split
-  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_delta, s_wg, s_cos, s_sin, s_moework;
+  // Cotangent buffers when the backward is not split (else they live in the slot).  With a
+  // second stream there are three sets, used by layer index mod 3: the weight gradients of
+  // layer l+1 read set (l+1)%3 while layer l's input-gradient chain writes set l%3 and
+  // hands its result to layer l-1 in set (l-1)%3.
+  LayerStash wsets[3];
+  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_partial_side, s_delta, s_wg, s_cos, s_sin,
+      s_moework;
   size_t total_bytes = 0;
+  // second stream (two_streams): weight gradients trail the input-gradient chain
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork = nullptr;          // recorded on the caller's stream, awaited by `side`
+  hipEvent_t ev_set[3] = {};             // last weight-gradient reader of a cotangent set
+  bool set_pending[3] = {};
+  std::vector<hipEvent_t> ev_slot;       // last `side` reader of a slot
+  std::vector<char> slot_pending;
+  std::vector<hipEvent_t> ev_bwd_i;      // end of a slot's BWD_I task on the caller's stream
+  hipEvent_t ev_tail = nullptr;          // last work queued on `side`
+  bool tail_pending = false;
 
   bf16_t* P(int chunk, int layer, int i) {
     return params + ((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i];
@@ -339,6 +354,8 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
 // ---- one layer, weight-gradient half --------------------------------------------
 int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, uint8_t* wbase,
                 const LayerStash& W, const void* dy) {
+  // scratch for partial sums: the second stream has its own
+  float* partial = s->S<float>(st == s->side && s->side ? s->s_partial_side : s->s_partial);
   const LayerStash& L = s->lay[li];
   const int64_t h = s->h, f = s->f;
   auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
@@ -359,7 +376,7 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(ggemm(st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, wt(W.dgu), 2 * f, 1, 0,
              s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
     RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)wt(W.dlogits), s->G(chunk, li, X_Wr),
-                            s->S<float>(s->s_partial)));
+                            partial));
     RC(wgrad(s, st, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, X_Wo), s->ctxw, h));
     RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw));
     return JPP_OK;
@@ -501,7 +518,8 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
 
   // scratch
   Carver sc;
-  if (!d->split_backward) carve_w(s, sc, s->wshared);
+  if (!d->split_backward)
+    for (int i = 0; i < (d->two_streams ? 3 : 1); ++i) carve_w(s, sc, s->wsets[i]);
   const size_t e = 2;
   s->s_dx[0] = sc.take(T * h * e);
   s->s_dx[1] = sc.take(T * h * e);
@@ -515,6 +533,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   const size_t widest = (size_t)std::max<int64_t>(std::max<int64_t>(s->qkvw, 2 * f), h);
   s->s_partial = sc.take(std::max((size_t)2 * JPP_NORM_PARTIALS * widest * 4,
                                   (size_t)64 * h * 8 * 4));
+  s->s_partial_side = sc.take(d->two_streams ? (size_t)64 * h * 8 * 4 : 256);
   s->s_delta = sc.take((size_t)d->batch * d->n_heads * d->seq * 4);
   size_t max_w = 0;
   for (auto& p : s->pinfo) max_w = std::max(max_w, (size_t)(p.rows * p.cols));
@@ -560,7 +579,23 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
     hipMemcpy(s->S<>(s->s_cos), c.data(), c.size() * 4, hipMemcpyHostToDevice);
     hipMemcpy(s->S<>(s->s_sin), sn.data(), sn.size() * 4, hipMemcpyHostToDevice);
   }
-  hipError_t e5 = hipDeviceSynchronize();
+  hipError_t e5 = hipSuccess;
+  if (d->two_streams) {
+    // default priority; non-blocking so that it does not serialise against the null stream
+    e5 = hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking);
+    auto mk = [&](hipEvent_t* ev) {
+      if (e5 == hipSuccess) e5 = hipEventCreateWithFlags(ev, hipEventDisableTiming);
+    };
+    mk(&s->ev_fork);
+    mk(&s->ev_tail);
+    for (auto& ev : s->ev_set) mk(&ev);
+    s->ev_slot.assign(d->max_live, nullptr);
+    s->ev_bwd_i.assign(d->max_live, nullptr);
+    s->slot_pending.assign(d->max_live, 0);
+    for (auto& ev : s->ev_slot) mk(&ev);
+    for (auto& ev : s->ev_bwd_i) mk(&ev);
+  }
+  if (e5 == hipSuccess) e5 = hipDeviceSynchronize();
   if (e5 != hipSuccess) {
     jpp_stage_destroy(s);
     return jpp_set_error(JPP_ERR_HIP, "stage_create: %s", hipGetErrorString(e5));
@@ -572,6 +607,13 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
 int jpp_stage_destroy(jpp_stage* s) {
   if (!s) return JPP_OK;
   hipDeviceSynchronize();
+  auto drop = [](hipEvent_t ev) { if (ev) hipEventDestroy(ev); };
+  drop(s->ev_fork);
+  drop(s->ev_tail);
+  for (auto ev : s->ev_set) drop(ev);
+  for (auto ev : s->ev_slot) drop(ev);
+  for (auto ev : s->ev_bwd_i) drop(ev);
+  if (s->side) hipStreamDestroy(s->side);
   for (auto p : s->slots) hipFree(p);
   if (s->scratch) hipFree(s->scratch);
   if (s->grads) hipFree(s->grads);
@@ -611,8 +653,15 @@ int jpp_stage_grad_ptr(jpp_stage* s, int chunk, int layer, int i, float** ptr) {
   return JPP_OK;
 }
 
+int jpp_stage_join(jpp_stage* s, void* stream) {
+  JPP_REQUIRE(s, "stage: null");
+  if (s->tail_pending) JPP_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, s->ev_tail, 0));
+  return JPP_OK;
+}
+
 int jpp_stage_zero_grads(jpp_stage* s, void* stream) {
   JPP_REQUIRE(s, "stage: null");
+  RC(jpp_stage_join(s, stream));  // weight gradients still in flight accumulate into the old values
   const size_t n = (size_t)s->d.n_chunks * s->d.layers_per_chunk * s->layer_elems;
   return jpp_fill_u32(s->grads, 0u, n, stream);
 }
@@ -643,6 +692,11 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
     s->live[key] = slot_i;
     s->phase[key] = 1;
     uint8_t* slot = s->slots[slot_i];
+    if (s->side && s->slot_pending[slot_i]) {
+      // weight gradients of the slot's previous microbatch may still be reading it
+      JPP_CHECK_HIP(hipStreamWaitEvent(st, s->ev_slot[slot_i], 0));
+      s->slot_pending[slot_i] = 0;
+    }
     JPP_CHECK_HIP(hipMemcpyAsync(slot + s->lay[0].x.off, in, act, hipMemcpyDeviceToDevice, st));
     for (int li = 0; li < nl; ++li) {
       void* y = li + 1 < nl ? (void*)(slot + s->lay[li + 1].x.off) : out;
@@ -659,6 +713,23 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
   const int ph = s->phase[key];
   const bool split = s->d.split_backward != 0;
 
+  const bool two = s->side != nullptr;
+  const int slot_i = it->second;
+  // queue `side` behind what the caller's stream holds so far
+  auto fork = [&]() -> int {
+    JPP_CHECK_HIP(hipEventRecord(s->ev_fork, st));
+    JPP_CHECK_HIP(hipStreamWaitEvent(s->side, s->ev_fork, 0));
+    return JPP_OK;
+  };
+  // `side` has read the slot for the last time in this task
+  auto side_done_with_slot = [&]() -> int {
+    JPP_CHECK_HIP(hipEventRecord(s->ev_slot[slot_i], s->side));
+    s->slot_pending[slot_i] = 1;
+    JPP_CHECK_HIP(hipEventRecord(s->ev_tail, s->side));
+    s->tail_pending = true;
+    return JPP_OK;
+  };
+
   if (kind == JPP_BWD || kind == JPP_BWD_I) {
     JPP_REQUIRE(in && out, "run_task(BWD): needs in and out");
     if (ph != 1)
@@ -667,29 +738,59 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
     if (kind == JPP_BWD_I && !split)
       return jpp_set_error(JPP_ERR_STATE,
                            "run_task(BWD_I): stage was created without split_backward");
+    const bool bert = s->d.family == JPP_FAMILY_BERT;
+    // cotangent set of layer li when they live in scratch
+    auto set_of = [&](int li) { return two ? ((li % 3) + 3) % 3 : 0; };
+    auto wait_set = [&](int k) -> int {
+      if (two && s->set_pending[k]) {
+        JPP_CHECK_HIP(hipStreamWaitEvent(st, s->ev_set[k], 0));
+        s->set_pending[k] = false;
+      }
+      return JPP_OK;
+    };
     const void* dy = in;
     for (int li = nl - 1; li >= 0; --li) {
       uint8_t* wbase = split ? slot : s->scratch;
-      const LayerStash& W = split ? s->lay[li] : s->wshared;
+      const LayerStash& W = split ? s->lay[li] : s->wsets[set_of(li)];
+      if (!split) {
+        // this layer writes its own set and (its result) the set of the layer below
+        RC(wait_set(set_of(li)));
+        if (li > 0 && !bert) RC(wait_set(set_of(li - 1)));
+      }
       void* dx;
       if (li == 0) dx = out;
-      else if (split && s->d.family != JPP_FAMILY_BERT) dx = slot + s->lay[li - 1].dyin.off;
+      else if (split && !bert) dx = slot + s->lay[li - 1].dyin.off;
+      else if (two && !bert) dx = s->scratch + s->wsets[set_of(li - 1)].dyin.off;
       else dx = s->S<>(s->s_dx[li & 1]);
-      if (split && s->d.family != JPP_FAMILY_BERT && li == nl - 1) {
-        // the weight-gradient task reads the incoming cotangent again later
-        JPP_CHECK_HIP(hipMemcpyAsync(slot + s->lay[li].dyin.off, in, act,
-                                     hipMemcpyDeviceToDevice, st));
-        dy = slot + s->lay[li].dyin.off;
+      if (!bert && li == nl - 1 && (split || two)) {
+        // the weight gradients read the incoming cotangent later (a BWD_W task, or the
+        // second stream after this call has returned): keep a copy
+        uint8_t* keep = wbase + W.dyin.off;
+        JPP_CHECK_HIP(hipMemcpyAsync(keep, in, act, hipMemcpyDeviceToDevice, st));
+        dy = keep;
       }
       RC(layer_bwd_i(s, st, chunk, li, slot, wbase, W, dy, dx));
-      if (kind == JPP_BWD) RC(layer_bwd_w(s, st, chunk, li, slot, wbase, W, dy));
+      if (kind == JPP_BWD) {
+        if (two) {
+          RC(fork());
+          RC(layer_bwd_w(s, s->side, chunk, li, slot, wbase, W, dy));
+          if (!split) {
+            JPP_CHECK_HIP(hipEventRecord(s->ev_set[set_of(li)], s->side));
+            s->set_pending[set_of(li)] = true;
+          }
+        } else {
+          RC(layer_bwd_w(s, st, chunk, li, slot, wbase, W, dy));
+        }
+      }
       dy = dx;
     }
     if (kind == JPP_BWD) {
-      s->free_slots.push_back(it->second);
+      if (two) RC(side_done_with_slot());
+      s->free_slots.push_back(slot_i);
       s->live.erase(it);
       s->phase.erase(key);
     } else {
+      if (two) JPP_CHECK_HIP(hipEventRecord(s->ev_bwd_i[slot_i], st));
       s->phase[key] = 2;
     }
     return JPP_OK;
@@ -702,9 +803,16 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
     if (ph != 2)
       return jpp_set_error(JPP_ERR_STATE, "run_task(BWD_W): BWD_I of (chunk %d, mubatch %d) has not run",
                            chunk, mb);
+    hipStream_t ws = st;
+    if (two) {
+      // everything it needs was complete when the BWD_I task ended on the caller's stream
+      JPP_CHECK_HIP(hipStreamWaitEvent(s->side, s->ev_bwd_i[slot_i], 0));
+      ws = s->side;
+    }
     for (int li = nl - 1; li >= 0; --li)
-      RC(layer_bwd_w(s, st, chunk, li, slot, slot, s->lay[li], slot + s->lay[li].dyin.off));
-    s->free_slots.push_back(it->second);
+      RC(layer_bwd_w(s, ws, chunk, li, slot, slot, s->lay[li], slot + s->lay[li].dyin.off));
+    if (two) RC(side_done_with_slot());
+    s->free_slots.push_back(slot_i);
     s->live.erase(it);
     s->phase.erase(key);
     return JPP_OK;

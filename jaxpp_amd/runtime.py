@@ -72,7 +72,8 @@ class StageDesc(C.Structure):
                 ("rope_theta", C.c_float), ("eps", C.c_float), ("gelu_tanh", C.c_int),
                 ("n_experts", C.c_int), ("top_k", C.c_int), ("n_chunks", C.c_int),
                 ("layers_per_chunk", C.c_int), ("max_live", C.c_int),
-                ("split_backward", C.c_int), ("fused_wgrad_accum", C.c_int)]
+                ("split_backward", C.c_int), ("fused_wgrad_accum", C.c_int),
+                ("two_streams", C.c_int)]
 
 
 EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32 = range(5)
@@ -91,7 +92,8 @@ EXPORTS = [
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
     "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
     "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
-    "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_bytes",
+    "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_join",
+    "jpp_stage_bytes",
     "jpp_stage_run_task", "jpp_stage_live_slots",
 ]
 
@@ -170,6 +172,7 @@ def load():
     lib.jpp_stage_grad_ptr.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int,
                                        C.POINTER(C.c_void_p)]
     lib.jpp_stage_zero_grads.argtypes = [C.c_void_p, C.c_void_p]
+    lib.jpp_stage_join.argtypes = [C.c_void_p, C.c_void_p]
     lib.jpp_stage_run_task.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                        C.c_void_p, C.c_void_p]
     lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
@@ -334,14 +337,16 @@ class StageExecutor:
     residual slots, and the FWD / BWD / BWD_I / BWD_W tasks."""
 
     def __init__(self, spec, n_chunks: int, layers_per_chunk: int, max_live: int,
-                 split_backward: bool = False, fused_wgrad_accum: bool = True):
+                 split_backward: bool = False, fused_wgrad_accum: bool = True,
+                 two_streams: bool = True):
         require_gpu()
         self.spec = spec
         self.n_chunks, self.layers_per_chunk = n_chunks, layers_per_chunk
         d = StageDesc(FAMILY[spec.family], spec.hidden, spec.n_heads, spec.kvh, spec.d, spec.ffn,
                       spec.seq, spec.batch, int(spec.causal), spec.rope_theta, spec.eps,
                       int(spec.gelu_tanh), spec.n_experts, spec.top_k, n_chunks,
-                      layers_per_chunk, max_live, int(split_backward), int(fused_wgrad_accum))
+                      layers_per_chunk, max_live, int(split_backward), int(fused_wgrad_accum),
+                      int(two_streams))
         h = C.c_void_p()
         check(load().jpp_stage_create(C.byref(d), C.byref(h)))
         self.handle = h.value
@@ -371,6 +376,7 @@ class StageExecutor:
                        to_bf16_bits(a))
 
     def get_grads(self, chunk: int, layer: int) -> dict:
+        self.join()          # the copies below run on the null stream
         out = {}
         for name, rows, cols in self.params:
             shape = (cols,) if rows == 1 and not name.startswith("W") else (rows, cols)
@@ -380,6 +386,10 @@ class StageExecutor:
 
     def zero_grads(self, stream=None):
         check(load().jpp_stage_zero_grads(self.handle, stream))
+
+    def join(self, stream=None):
+        """Orders `stream` behind the weight-gradient work on the stage's own stream."""
+        check(load().jpp_stage_join(self.handle, stream))
 
     def run_task(self, kind: TaskType, chunk: int, mubatch: int, inp=None, out=None,
                  stream=None):

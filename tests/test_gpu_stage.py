@@ -39,10 +39,11 @@ def close(got, want, rtol, what):
     assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
 
 
-def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0):
+def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_streams=True,
+               sync_every_task=True):
     shape = (spec.tokens, spec.hidden)
     ex = rt.StageExecutor(spec, plan.n_chunks, layers_per_chunk, plan.max_live,
-                          plan.split_backward, fused)
+                          plan.split_backward, fused, two_streams)
     for c, stage in enumerate(plan.stages):
         for li in range(layers_per_chunk):
             ex.set_params(c, li, params[stage][li])
@@ -58,7 +59,8 @@ def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0):
         kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
         inp = rt.DeviceBuffer.from_f32_as_bf16(boundary_tensor(kind, *key, shape, seed))
         ex.run_task(pt.exec_kind, pt.chunk, t.mubatch_idx, inp.ptr, out.ptr)
-        rt.sync()
+        if sync_every_task:
+            rt.sync()
         (ys if kind == "x" else dxs)[key] = out.download_bf16(shape)
     assert ex.live_slots() == 0
     grads = {stage: [ex.get_grads(c, li) for li in range(layers_per_chunk)]
@@ -95,14 +97,18 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("two_streams", [True, False], ids=["two-streams", "one-stream"])
 @pytest.mark.parametrize("name,spec,sched,n,rank,lpc", CASES, ids=[c[0] for c in CASES])
-def test_stage_matches_oracle(name, spec, sched, n, rank, lpc):
-    print(f"stage case {name}", flush=True)
+def test_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
+    print(f"stage case {name} two_streams={two_streams}", flush=True)
     plan = make_rank_plan(sched, n, rank)
     params = make_params(spec, plan.stages, lpc)
     row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
     ys_w, dxs_w, acc_w = run_on_oracle(spec, plan, params, row)
-    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params)
+    # with the second stream the tasks are queued back to back (the download of a task's
+    # output waits on the null stream only), so weight gradients really trail behind
+    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params, two_streams=two_streams,
+                                sync_every_task=not two_streams)
     assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
     for k in ys_w:
         close(ys[k], ys_w[k], 2e-2, f"y{k}")
@@ -137,6 +143,8 @@ def test_task_order_does_not_change_gradients():
     for sched in (S.GPipe(2), S.Std1F1B(2), S.ZeroBubble(2)):
         plan = make_rank_plan(sched, n, 0)
         res.append(run_on_gpu(spec, plan, 1, params))
+    # ... and neither does moving the weight gradients to the second stream
+    res.append(run_on_gpu(spec, make_rank_plan(S.Std1F1B(2), n, 0), 1, params, two_streams=False))
     for other in res[1:]:
         for k, v in res[0][2][0][0].items():
             np.testing.assert_array_equal(other[2][0][0][k], v, err_msg=k)
