@@ -25,6 +25,7 @@ from jaxpp_amd import runtime as rt            # noqa: E402
 from jaxpp_amd import schedules as S           # noqa: E402
 from jaxpp_amd.model import workloads          # noqa: E402
 from jaxpp_amd.plan import make_rank_plan      # noqa: E402
+from jaxpp_amd.rank_loop import RankLoop       # noqa: E402
 from jaxpp_amd.types import TaskType           # noqa: E402
 
 MFMA_BF16_PEAK = 2.5e15     # dense bf16 FLOP/s, MI355X
@@ -86,21 +87,21 @@ class Workbench:
                     off = (j * 104729 * 8) % (1 << 22)
                     rt.check(lib.jpp_memcpy_d2d_async(buf.ptr, bpool.ptr + 2 * off, act * 2, None))
                     store[c, m] = buf
-        self.out = rt.DeviceBuffer(act * 2)
+        self.out = [rt.DeviceBuffer(act * 2), rt.DeviceBuffer(act * 2)]
+        self.loop = RankLoop(self.ex, self.plan, overlap_fused=two_streams)
         rt.sync()
         self._keep = (wpool, ones, bpool)
 
     def step(self):
         ex = self.ex
         ex.zero_grads()                       # `Add.state`: accumulators start from zero
-        for pt in self.plan.tasks:
+
+        def io(pt, lane):
             m = pt.task.mubatch_idx
-            if pt.exec_kind is TaskType.FWD:
-                ex.run_task(pt.exec_kind, pt.chunk, m, self.x_in[pt.chunk, m].ptr, self.out.ptr)
-            elif pt.exec_kind is TaskType.BWD_W:
-                ex.run_task(pt.exec_kind, pt.chunk, m)
-            else:
-                ex.run_task(pt.exec_kind, pt.chunk, m, self.dy_in[pt.chunk, m].ptr, self.out.ptr)
+            src = self.x_in if pt.exec_kind is TaskType.FWD else self.dy_in
+            return src[pt.chunk, m].ptr, self.out[lane].ptr
+
+        self.loop.run(io)
         ex.join()                             # the step ends when the last weight gradient has landed
 
     def step_flops(self) -> float:

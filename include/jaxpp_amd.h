@@ -61,6 +61,7 @@ int jpp_device_sync(void);
 int jpp_event_create(void** event);
 int jpp_event_destroy(void* event);
 int jpp_event_record(void* event, void* stream);
+int jpp_stream_wait_event(void* stream, void* event); /* later work on stream waits for event */
 int jpp_event_sync(void* event);
 int jpp_event_elapsed_ms(void* start, void* stop, float* ms);
 int jpp_mem_info(size_t* free_bytes, size_t* total_bytes);

@@ -122,6 +122,11 @@ int jpp_event_record(void* event, void* stream) {
   JPP_CHECK_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
   return JPP_OK;
 }
+int jpp_stream_wait_event(void* stream, void* event) {
+  JPP_REQUIRE(event, "stream_wait_event: null event");
+  JPP_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0));
+  return JPP_OK;
+}
 int jpp_event_sync(void* event) {
   JPP_CHECK_HIP(hipEventSynchronize((hipEvent_t)event));
   return JPP_OK;

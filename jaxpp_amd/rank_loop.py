@@ -1,0 +1,48 @@
+"""Runs one rank's row of the task table on a stage executor.
+
+The reference turns the members of a ``FusedTask`` into one task whose parts
+the compiler is free to overlap (src/jaxpp/core.py:2444-2513, ``fuse_groups``;
+src/jaxpp/schedules.py:48-54).  Here the forward member of a fused entry goes
+out on a second stream and the backward member on the first one; the streams
+meet again at the end of the entry, so everything after it sees both results.
+"""
+from __future__ import annotations
+
+from itertools import groupby
+
+from jaxpp_amd import runtime as rt
+from jaxpp_amd.types import TaskType
+
+
+class RankLoop:
+    def __init__(self, executor: "rt.StageExecutor", plan, overlap_fused: bool = True):
+        self.ex, self.plan = executor, plan
+        self.entries = [list(g) for _, g in groupby(plan.tasks, key=lambda pt: pt.group)]
+        self.overlap = overlap_fused and any(len(e) > 1 for e in self.entries)
+        if self.overlap:
+            self.aux = rt.Stream()
+            self.fork, self.join = rt.Event(), rt.Event()
+
+    def run(self, io):
+        """``io(pt, lane)`` -> (in_ptr, out_ptr) for a FWD / BWD / BWD_I task (lane 1: the task
+        runs beside another one and needs an output buffer of its own); BWD_W tasks take
+        none.  Everything is queued on the null stream, fused forwards on the second."""
+        ex = self.ex
+        for entry in self.entries:
+            beside = self.overlap and len(entry) > 1 and \
+                any(pt.exec_kind is TaskType.FWD for pt in entry) and \
+                any(pt.exec_kind is not TaskType.FWD for pt in entry)
+            if beside:
+                self.fork.record(None)
+                self.aux.wait(self.fork)
+            for pt in entry:
+                m = pt.task.mubatch_idx
+                if pt.exec_kind is TaskType.BWD_W:
+                    ex.run_task(pt.exec_kind, pt.chunk, m)
+                    continue
+                on_aux = beside and pt.exec_kind is TaskType.FWD
+                inp, out = io(pt, 1 if on_aux else 0)
+                ex.run_task(pt.exec_kind, pt.chunk, m, inp, out, self.aux.ptr if on_aux else None)
+            if beside:
+                self.join.record(self.aux.ptr)
+                rt.stream_wait(None, self.join)

@@ -84,7 +84,8 @@ FAMILY = {"bert": 0, "llama": 1, "mixtral": 2}
 EXPORTS = [
     "jpp_last_error", "jpp_version", "jpp_device_count", "jpp_set_device", "jpp_malloc",
     "jpp_free", "jpp_memcpy_h2d", "jpp_memcpy_d2h", "jpp_memcpy_d2d_async", "jpp_fill_u32",
-    "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_device_sync",
+    "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_stream_wait_event",
+    "jpp_device_sync",
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
     "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
@@ -122,6 +123,7 @@ def load():
     lib.jpp_memcpy_d2d_async.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
     lib.jpp_fill_u32.argtypes = [C.c_void_p, C.c_uint32, C.c_size_t, C.c_void_p]
     lib.jpp_stream_create.argtypes = [C.POINTER(C.c_void_p)]
+    lib.jpp_stream_wait_event.argtypes = [C.c_void_p, C.c_void_p]
     lib.jpp_stream_destroy.argtypes = [C.c_void_p]
     lib.jpp_stream_sync.argtypes = [C.c_void_p]
     lib.jpp_event_create.argtypes = [C.POINTER(C.c_void_p)]
@@ -272,6 +274,33 @@ def download_ptr(ptr: int, dtype, shape) -> np.ndarray:
 
 def sync():
     check(load().jpp_device_sync())
+
+
+class Stream:
+    """A HIP stream of default priority that does not synchronise with the null stream."""
+
+    def __init__(self):
+        p = C.c_void_p()
+        check(load().jpp_stream_create(C.byref(p)))
+        self.ptr = p.value
+
+    def wait(self, event: "Event"):
+        check(load().jpp_stream_wait_event(self.ptr, event.ptr))
+
+    def sync(self):
+        check(load().jpp_stream_sync(self.ptr))
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                load().jpp_stream_destroy(self.ptr)
+        except Exception:
+            pass
+
+
+def stream_wait(stream, event: "Event"):
+    """Work queued on `stream` (None: the null stream) after this call waits for `event`."""
+    check(load().jpp_stream_wait_event(stream, event.ptr))
 
 
 class Event:

@@ -11,6 +11,7 @@ from jaxpp_amd import runtime as rt
 from jaxpp_amd import schedules as S
 from jaxpp_amd.model import LayerSpec, boundary_tensor, init_layer_params
 from jaxpp_amd.plan import make_rank_plan
+from jaxpp_amd.rank_loop import RankLoop
 from jaxpp_amd.types import TaskType
 from oracle import layers as L
 from oracle import stage as O
@@ -39,30 +40,47 @@ def close(got, want, rtol, what):
     assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
 
 
-def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_streams=True,
-               sync_every_task=True):
+def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_streams=True):
+    """Runs the rank's row.  With two_streams the row is queued without host waits in between:
+    weight gradients trail on the stage's stream and the forward of a fused entry runs on a
+    second caller stream (RankLoop); otherwise one task at a time with a device sync."""
     shape = (spec.tokens, spec.hidden)
     ex = rt.StageExecutor(spec, plan.n_chunks, layers_per_chunk, plan.max_live,
                           plan.split_backward, fused, two_streams)
     for c, stage in enumerate(plan.stages):
         for li in range(layers_per_chunk):
             ex.set_params(c, li, params[stage][li])
-    ys, dxs = {}, {}
-    out = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+    ins, outs = {}, {}
     for pt in plan.tasks:
-        t = pt.task
-        key = (t.stage_id, t.mubatch_idx)
-        print(f"  task {t} as {pt.exec_kind.name}", flush=True)
         if pt.exec_kind is TaskType.BWD_W:
-            ex.run_task(pt.exec_kind, pt.chunk, t.mubatch_idx)
             continue
+        t = pt.task
         kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
-        inp = rt.DeviceBuffer.from_f32_as_bf16(boundary_tensor(kind, *key, shape, seed))
-        ex.run_task(pt.exec_kind, pt.chunk, t.mubatch_idx, inp.ptr, out.ptr)
-        if sync_every_task:
+        key = (kind, t.stage_id, t.mubatch_idx)
+        ins[key] = rt.DeviceBuffer.from_f32_as_bf16(
+            boundary_tensor(kind, t.stage_id, t.mubatch_idx, shape, seed))
+        outs[key] = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+
+    def io(pt, lane=0):
+        kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
+        key = (kind, pt.task.stage_id, pt.task.mubatch_idx)
+        return ins[key].ptr, outs[key].ptr
+
+    if two_streams:
+        RankLoop(ex, plan).run(io)
+    else:
+        for pt in plan.tasks:
+            print(f"  task {pt.task} as {pt.exec_kind.name}", flush=True)
+            if pt.exec_kind is TaskType.BWD_W:
+                ex.run_task(pt.exec_kind, pt.chunk, pt.task.mubatch_idx)
+            else:
+                ex.run_task(pt.exec_kind, pt.chunk, pt.task.mubatch_idx, *io(pt))
             rt.sync()
-        (ys if kind == "x" else dxs)[key] = out.download_bf16(shape)
+    ex.join()
+    rt.sync()
     assert ex.live_slots() == 0
+    ys = {k[1:]: b.download_bf16(shape) for k, b in outs.items() if k[0] == "x"}
+    dxs = {k[1:]: b.download_bf16(shape) for k, b in outs.items() if k[0] == "dy"}
     grads = {stage: [ex.get_grads(c, li) for li in range(layers_per_chunk)]
              for c, stage in enumerate(plan.stages)}
     ex.close()
@@ -105,10 +123,7 @@ def test_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
     params = make_params(spec, plan.stages, lpc)
     row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
     ys_w, dxs_w, acc_w = run_on_oracle(spec, plan, params, row)
-    # with the second stream the tasks are queued back to back (the download of a task's
-    # output waits on the null stream only), so weight gradients really trail behind
-    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params, two_streams=two_streams,
-                                sync_every_task=not two_streams)
+    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params, two_streams=two_streams)
     assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
     for k in ys_w:
         close(ys[k], ys_w[k], 2e-2, f"y{k}")
