@@ -3,13 +3,14 @@
 //
 //   C[m,n] = epilogue( sum_k Aop[m,k] * Bop[n,k] )
 //
-// A workgroup of 256 threads (4 waves, 2 x 2) owns a BM x BN output tile and
-// walks K in steps of 64.  Both operands live in LDS as swizzled [rows][64]
-// slabs with the contraction index contiguous, whatever their layout in HBM:
-// an operand whose contraction index is the slow one in memory (the weights
-// in a forward GEMM, both operands of a weight-gradient GEMM) is transposed in
-// registers on its way into LDS (TileLoader<.., TRANS=true>).  The next K-step
-// is fetched from HBM into registers while the current one is multiplied.
+// A workgroup of 4 or 8 waves owns a BM x BN output tile and walks K in steps
+// of 64.  Operand tiles travel HBM -> LDS without passing through registers
+// (global_load_lds_dwordx4), keeping the layout they have in HBM: an operand
+// whose contraction index is contiguous in memory lands as swizzled [rows][64]
+// slabs and is read back with 16-byte LDS reads; one whose contraction index
+// is the slow one (the weights in a forward GEMM, both operands of a
+// weight-gradient GEMM) lands as [64][rows] and is read back with the
+// transposing 8-byte LDS reads (ds_read_b64_tr_b16).
 //
 // The weight operand is fed to the MFMA "A" port and the activation operand to
 // the "B" port, so a lane ends up holding 4 consecutive n for one m and the
@@ -197,45 +198,77 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 
   // epilogue: lane holds m = base_m + (lane & 31), and for g = 0..3 the four
   // columns base_n + 8 g + 4 (lane >> 5) + {0,1,2,3}
+  const long m_lane = m0 + wm * (BM / 2) + (lane & 31);
+  const long n_lane = n0 + wn * (BN / WN) + (lane >> 5) * 4;
+  if constexpr (EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_F32) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const long m = m0 + wm * (BM / 2) + i * 32 + (lane & 31);
+    for (int i = 0; i < TM; ++i) {
+      const long m = m_lane + i * 32;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+      for (int j = 0; j < TN; ++j) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const long n = n0 + wn * (BN / WN) + j * 32 + g * 8 + (lane >> 5) * 4;
-        float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
-        float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
-        if constexpr (EPI == JPP_EPI_ACC_F32) {
+        for (int g = 0; g < 4; ++g) {
+          const long n = n_lane + j * 32 + g * 8;
           float4* dst = (float4*)((float*)p.c + m * p.ldc + n);
-          float4 o = *dst;
-          o.x += v0; o.y += v1; o.z += v2; o.w += v3;
+          float4 o = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                                 acc[i][j][4 * g + 3]);
+          if constexpr (EPI == JPP_EPI_ACC_F32) {
+            const float4 c = *dst;
+            o.x += c.x; o.y += c.y; o.z += c.z; o.w += c.w;
+          }
           *dst = o;
-        } else if constexpr (EPI == JPP_EPI_F32) {
-          *(float4*)((float*)p.c + m * p.ldc + n) = make_float4(v0, v1, v2, v3);
-        } else {
+        }
+      }
+    }
+  } else {
+    // Operands of the epilogue (bias, residual, GELU pre-activation) are fetched in one
+    // batch per row of MFMA tiles before anything is stored: a load issued between stores
+    // would have to wait for those stores as well (one counter orders both).
+    uint2 bb[TN][4];
+    if (p.bias) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) bb[j][g] = *(const uint2*)(p.bias + n_lane + j * 32 + g * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const long m = m_lane + i * 32;
+      uint2 xx[TN][4];  // residual, or the pre-activation of the GELU gradient
+      const bf16_t* extra = EPI == JPP_EPI_DGELU ? p.aux : (EPI == JPP_EPI_BF16 ? p.resid : nullptr);
+      const long ldx = EPI == JPP_EPI_DGELU ? p.ldaux : p.ldresid;
+      if (extra) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            xx[j][g] = *(const uint2*)(extra + m * ldx + n_lane + j * 32 + g * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const long n = n_lane + j * 32 + g * 8;
+          float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
+          float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
           if (p.bias) {
-            const uint2 bb = *(const uint2*)(p.bias + n);
-            v0 += bf16lo_to_f32(bb.x); v1 += bf16hi_to_f32(bb.x);
-            v2 += bf16lo_to_f32(bb.y); v3 += bf16hi_to_f32(bb.y);
+            v0 += bf16lo_to_f32(bb[j][g].x); v1 += bf16hi_to_f32(bb[j][g].x);
+            v2 += bf16lo_to_f32(bb[j][g].y); v3 += bf16hi_to_f32(bb[j][g].y);
           }
           if constexpr (EPI == JPP_EPI_BF16) {
-            if (p.resid) {
-              const uint2 rr = *(const uint2*)(p.resid + m * p.ldresid + n);
-              v0 += bf16lo_to_f32(rr.x); v1 += bf16hi_to_f32(rr.x);
-              v2 += bf16lo_to_f32(rr.y); v3 += bf16hi_to_f32(rr.y);
+            if (extra) {
+              v0 += bf16lo_to_f32(xx[j][g].x); v1 += bf16hi_to_f32(xx[j][g].x);
+              v2 += bf16lo_to_f32(xx[j][g].y); v3 += bf16hi_to_f32(xx[j][g].y);
             }
           } else if constexpr (EPI == JPP_EPI_GELU) {
             *(uint2*)((bf16_t*)p.c2 + m * p.ldc2 + n) =
                 make_uint2(pack_bf16x2(gelu_f(v0, p.gelu_tanh), gelu_f(v1, p.gelu_tanh)),
                            pack_bf16x2(gelu_f(v2, p.gelu_tanh), gelu_f(v3, p.gelu_tanh)));
           } else if constexpr (EPI == JPP_EPI_DGELU) {
-            const uint2 uu = *(const uint2*)(p.aux + m * p.ldaux + n);
-            v0 *= gelu_grad_f(bf16lo_to_f32(uu.x), p.gelu_tanh);
-            v1 *= gelu_grad_f(bf16hi_to_f32(uu.x), p.gelu_tanh);
-            v2 *= gelu_grad_f(bf16lo_to_f32(uu.y), p.gelu_tanh);
-            v3 *= gelu_grad_f(bf16hi_to_f32(uu.y), p.gelu_tanh);
+            v0 *= gelu_grad_f(bf16lo_to_f32(xx[j][g].x), p.gelu_tanh);
+            v1 *= gelu_grad_f(bf16hi_to_f32(xx[j][g].x), p.gelu_tanh);
+            v2 *= gelu_grad_f(bf16lo_to_f32(xx[j][g].y), p.gelu_tanh);
+            v3 *= gelu_grad_f(bf16hi_to_f32(xx[j][g].y), p.gelu_tanh);
           }
           *(uint2*)((bf16_t*)p.c + m * p.ldc + n) =
               make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
@@ -289,7 +322,7 @@ int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
     case 1: return launch<128, 128, TA, TB, EPI>(stream, p);
     case 2: return launch<256, 128, TA, TB, EPI>(stream, p);
     case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
-    default: return launch<256, 256, TA, TB, EPI>(stream, p);
+    default: return launch<128, 128, TA, TB, EPI>(stream, p);
   }
 }
 
@@ -349,10 +382,10 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     JPP_REQUIRE(a->aux && a->ldaux >= a->n && a->ldaux % 4 == 0, "gemm: dGELU epilogue needs aux");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
-  if (a->group_mode != JPP_GROUP_NONE) tile = (a->tile == 3) ? 3 : 4;  // 256-row segments
+  if (a->group_mode != JPP_GROUP_NONE) tile = 4;  // 256-row segments
+  JPP_REQUIRE(tile == 1 || tile == 2 || tile == 4, "gemm: unknown tile %d", tile);
   if (tile >= 2 && a->m % 256) tile = 1;
-  if (tile >= 3 && a->n % 256) tile = 2;
-  JPP_REQUIRE(tile >= 1 && tile <= 4, "gemm: unknown tile %d", tile);
+  if (tile == 4 && a->n % 256) tile = 2;
 
   const int ta = a->trans_a != 0, tb = a->trans_b != 0, e = a->epilogue;
 #define JPP_GEMM_CASE(TA_, TB_, E_) \
