@@ -115,14 +115,46 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   const long a_step = TA ? 64 * p.lda : 64;
   const long b_step = TB ? 64 * p.ldb : 64;
 
+  // lane holds m = m_lane + 32 i, and for g = 0..3 the four columns n_lane + 32 j + 8 g + {0..3}
+  const long m_lane = m0 + wm * (BM / 2) + (lane & 31);
+  const long n_lane = n0 + wn * (BN / WN) + (lane >> 5) * 4;
   f32x16 acc[TM][TN];
+  // C += A B (EPI_ACC_F32): the fp32 tile in memory is read in TM batches (one row of MFMA
+  // tiles each) during the first K-steps - requested at the end of K-step t, folded into the
+  // accumulators at the end of K-step t+1, where the wave waits for its operand copies
+  // anyway - and the epilogue only stores.  A read-modify-write epilogue would wait for HBM
+  // with the matrix cores idle.  Short K loops read the tile up front instead.
+  const bool stream_c = EPI == JPP_EPI_ACC_F32 && kt_n > TM;
+  float4 cbuf[TN][4];
+  auto load_c_row = [&](int i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        cbuf[j][g] = *(const float4*)((const float*)p.c + (m_lane + i * 32) * p.ldc + n_lane +
+                                      j * 32 + g * 8);
+  };
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
+  if constexpr (EPI == JPP_EPI_ACC_F32) {
+    if (!stream_c) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        load_c_row(i);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            acc[i][j][4 * g] = cbuf[j][g].x; acc[i][j][4 * g + 1] = cbuf[j][g].y;
+            acc[i][j][4 * g + 2] = cbuf[j][g].z; acc[i][j][4 * g + 3] = cbuf[j][g].w;
+          }
+      }
+    }
+  }
   const uint32_t lds0 = lds_address(smem);
   typename TileA::Offsets offa;
   typename TileB::Offsets offb;
@@ -144,6 +176,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     TileA::template issue<0, IA>(uniform_ptr(a_src + k1 * a_step), offa, lds0 + STAGE, wave);
     TileB::template issue<0, IB>(uniform_ptr(b_src + k1 * b_step), offb, lds0 + STAGE + A_BYTES, wave);
     dma_wait<IA + IB>();   // stage 0 has landed; stage 1 may still be in flight
+  }
+  if constexpr (EPI == JPP_EPI_ACC_F32) {
+    // the compiler waits for up-front reads of C here, not at their first use inside the K
+    // loop (where its wait would also cover the operand copies in flight)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(acc[i][j]));
   }
   __syncthreads();
 #pragma unroll
@@ -173,6 +213,24 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
         dma_wait_all();
         lds_wait_all();
         __syncthreads();
+        if constexpr (EPI == JPP_EPI_ACC_F32) {
+          if (stream_c && kt <= TM) {
+            // everything this wave had in flight has landed: fold in the row requested one
+            // K-step ago, request the next one
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+              if (kt == i + 1) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                  for (int g = 0; g < 4; ++g) {
+                    acc[i][j][4 * g] += cbuf[j][g].x; acc[i][j][4 * g + 1] += cbuf[j][g].y;
+                    acc[i][j][4 * g + 2] += cbuf[j][g].z; acc[i][j][4 * g + 3] += cbuf[j][g].w;
+                  }
+              }
+            if (kt < TM) load_c_row(kt);
+          }
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j) fw[nxt][j] = TileB::frag(na + A_BYTES, row_w + j * 32, 0, lane);
 #pragma unroll
@@ -196,30 +254,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   }
   dma_wait_all();   // the refetches of the last two K-steps must not outlive the block's LDS
 
-  // epilogue: lane holds m = base_m + (lane & 31), and for g = 0..3 the four
-  // columns base_n + 8 g + 4 (lane >> 5) + {0,1,2,3}
-  const long m_lane = m0 + wm * (BM / 2) + (lane & 31);
-  const long n_lane = n0 + wn * (BN / WN) + (lane >> 5) * 4;
   if constexpr (EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_F32) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const long m = m_lane + i * 32;
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const long n = n_lane + j * 32 + g * 8;
-          float4* dst = (float4*)((float*)p.c + m * p.ldc + n);
-          float4 o = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                                 acc[i][j][4 * g + 3]);
-          if constexpr (EPI == JPP_EPI_ACC_F32) {
-            const float4 c = *dst;
-            o.x += c.x; o.y += c.y; o.z += c.z; o.w += c.w;
-          }
-          *dst = o;
-        }
-      }
-    }
+        for (int g = 0; g < 4; ++g)
+          *(float4*)((float*)p.c + (m_lane + i * 32) * p.ldc + n_lane + j * 32 + g * 8) =
+              make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                          acc[i][j][4 * g + 3]);
   } else {
     // Operands of the epilogue (bias, residual, GELU pre-activation) are fetched in one
     // batch per row of MFMA tiles before anything is stored: a load issued between stores

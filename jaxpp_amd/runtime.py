@@ -367,7 +367,7 @@ class StageExecutor:
 
     def __init__(self, spec, n_chunks: int, layers_per_chunk: int, max_live: int,
                  split_backward: bool = False, fused_wgrad_accum: bool = True,
-                 two_streams: bool = True):
+                 two_streams: bool = False):
         require_gpu()
         self.spec = spec
         self.n_chunks, self.layers_per_chunk = n_chunks, layers_per_chunk
