@@ -162,6 +162,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--n-mubatches", type=int, default=None,
+                    help="override the workload's microbatch count (shorter runs under "
+                         "rocprofv3 --pmc, which serialises every dispatch; not the headline)")
     ap.add_argument("--unfused-accumulate", action="store_true",
                     help="bf16 weight gradient + separate fp32 accumulate pass")
     ap.add_argument("--two-streams", action="store_true",
@@ -176,6 +179,9 @@ def main():
         sys.exit(2)
     rt.require_gpu()
     wl = workloads()[args.workload]
+    if args.n_mubatches:
+        import dataclasses
+        wl = dataclasses.replace(wl, n_mubatches=args.n_mubatches)
     wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=args.two_streams)
     cls = args.probe or dominant_gemm_class(wl)
 
