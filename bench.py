@@ -111,7 +111,7 @@ class Workbench:
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size)
-MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.150e9}
+MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.133e9}
 
 
 def dominant_gemm_class(wl) -> str:
@@ -167,10 +167,12 @@ def main():
                          "rocprofv3 --pmc, which serialises every dispatch; not the headline)")
     ap.add_argument("--unfused-accumulate", action="store_true",
                     help="bf16 weight gradient + separate fp32 accumulate pass")
-    ap.add_argument("--two-streams", action="store_true",
+    ap.add_argument("--two-streams", choices=["auto", "on", "off"], default="auto",
                     help="weight gradients on the stage's second stream and the forward of a "
-                         "fused entry beside its backward (measured: +1%% at cfg3, -2%% at cfg5; "
-                         "per-kernel timings then include the other stream's kernels)")
+                         "fused entry beside its backward.  auto: on when the layers are too "
+                         "narrow for one kernel to fill the chip (hidden < 2048: +20%% at cfg2), off "
+                         "otherwise (+1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
+                         "include the other stream's kernels)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -182,7 +184,8 @@ def main():
     if args.n_mubatches:
         import dataclasses
         wl = dataclasses.replace(wl, n_mubatches=args.n_mubatches)
-    wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=args.two_streams)
+    two = wl.layer.hidden < 2048 if args.two_streams == "auto" else args.two_streams == "on"
+    wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two)
     cls = args.probe or dominant_gemm_class(wl)
 
     for _ in range(args.warmup):
@@ -215,7 +218,7 @@ def main():
             "layers": wl.layers_per_stage * wb.plan.n_chunks,
             "peak_live_microbatches": wb.plan.max_live,
             "fused_wgrad_accumulate": not args.unfused_accumulate,
-            "two_streams": args.two_streams,
+            "two_streams": two,
             "device_bytes": wb.ex.nbytes,
         },
         "algorithmic_flops_per_step": flops,
