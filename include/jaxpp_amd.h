@@ -94,17 +94,23 @@ typedef enum {
   JPP_EPI_GELU = 1,    /* u = acc + bias;  C = u,  C2 = gelu(u)   (both bf16)          */
   JPP_EPI_DGELU = 2,   /* C(bf16) = acc * gelu'(aux[m,n])                              */
   JPP_EPI_ACC_F32 = 3, /* C(f32) += acc      (the `add prev_acc g` of a backward task) */
-  JPP_EPI_F32 = 4      /* C(f32) = acc                                                 */
+  JPP_EPI_F32 = 4,     /* C(f32) = acc                                                 */
+  /* SwiGLU with gate and up projections interleaved in blocks of 32 columns: column 64q+w of
+   * the fused projection is gate feature 32q+w for w < 32 and up feature 32q+w-32 otherwise. */
+  JPP_EPI_SWIGLU = 5,  /* C(bf16) = acc (N = 2f, interleaved);
+                          C2[m, 32q+w] = silu(C[m, 64q+w]) * C[m, 64q+32+w]   (bf16, [M, f]) */
+  JPP_EPI_DSWIGLU = 6  /* acc = ds [M, N = f]; aux = the interleaved gate/up [M, 2f];
+                          C (bf16, [M, 2f], interleaved) = d(gate), d(up) of silu(gate)*up      */
 } jpp_epilogue;
 
 typedef struct {
   const void* a;
   const void* b;
   void* c;
-  void* c2;          /* second output (JPP_EPI_GELU) */
+  void* c2;          /* second output (JPP_EPI_GELU, JPP_EPI_SWIGLU) */
   const void* bias;  /* bf16 [N] or NULL */
   const void* resid; /* bf16 [M,N] or NULL */
-  const void* aux;   /* bf16 [M,N] (JPP_EPI_DGELU) */
+  const void* aux;   /* bf16 [M,N] (JPP_EPI_DGELU), [M,2N] (JPP_EPI_DSWIGLU) */
   int64_t m, n, k;
   int64_t lda, ldb, ldc, ldc2, ldresid, ldaux;
   int trans_a, trans_b;
@@ -168,10 +174,12 @@ int jpp_norm_fwd(void* stream, const jpp_norm_args* args);
 int jpp_norm_bwd(void* stream, const jpp_norm_args* args);
 
 /* ---- elementwise ------------------------------------------------------------ */
-/* s[t,j] = silu(gu[t,j]) * gu[t,f+j]; backward writes dgu [T,2f]. */
-int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f);
+/* s[t,j] = silu(gate[t,j]) * up[t,j]; backward writes dgu [T,2f] in gu's layout.
+ * interleaved = 0: gu = [gate | up] halves; 1: blocks of 32 columns as for JPP_EPI_SWIGLU. */
+int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f,
+                   int interleaved);
 int jpp_swiglu_bwd(void* stream, const void* gu, const void* ds, void* dgu, int64_t rows,
-                   int64_t f);
+                   int64_t f, int interleaved);
 /* Half-split rotary embedding applied in place to the first n_rot_heads heads
  * of each row (q and k heads are adjacent in a packed qkv row); cos/sin: f32
  * [seq, head_dim/2]; inverse != 0 rotates by the negative angle (backward). */

@@ -238,17 +238,26 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const bf16_t* __res
 // ---------------------------------------------------------------------------
 // SwiGLU
 // ---------------------------------------------------------------------------
+// gate and up of 8 features starting at feature 8c of row t: halves layout [gate | up], or
+// interleaved in blocks of 32 columns (column 64q+w: gate feature 32q+w for w < 32, else up)
+__device__ __forceinline__ long gate_col(int c, int f, int il) {
+  return il ? (long)(c >> 2) * 64 + (c & 3) * 8 : (long)c * 8;
+}
+__device__ __forceinline__ long up_col(int c, int f, int il) {
+  return il ? (long)(c >> 2) * 64 + 32 + (c & 3) * 8 : (long)f + (long)c * 8;
+}
+
 __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restrict__ gu,
                                                          bf16_t* __restrict__ s, long rows,
-                                                         int f) {
+                                                         int f, int il) {
   const int fc = f >> 3;
   const long total = rows * fc;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     const long t = i / fc;
     const int c = (int)(i - t * fc);
     float a[8], b[8];
-    unpack8(*(const uint4*)(gu + t * 2 * f + c * 8), a);
-    unpack8(*(const uint4*)(gu + t * 2 * f + f + c * 8), b);
+    unpack8(*(const uint4*)(gu + t * 2 * f + gate_col(c, f, il)), a);
+    unpack8(*(const uint4*)(gu + t * 2 * f + up_col(c, f, il)), b);
 #pragma unroll
     for (int e = 0; e < 8; ++e) a[e] = a[e] / (1.0f + __expf(-a[e])) * b[e];
     *(uint4*)(s + t * f + c * 8) = pack8(a);
@@ -258,15 +267,16 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restric
 __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restrict__ gu,
                                                          const bf16_t* __restrict__ ds,
                                                          bf16_t* __restrict__ dgu, long rows,
-                                                         int f) {
+                                                         int f, int il) {
   const int fc = f >> 3;
   const long total = rows * fc;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
     const long t = i / fc;
     const int c = (int)(i - t * fc);
+    const long gc = gate_col(c, f, il), uc = up_col(c, f, il);
     float a[8], b[8], d[8];
-    unpack8(*(const uint4*)(gu + t * 2 * f + c * 8), a);
-    unpack8(*(const uint4*)(gu + t * 2 * f + f + c * 8), b);
+    unpack8(*(const uint4*)(gu + t * 2 * f + gc), a);
+    unpack8(*(const uint4*)(gu + t * 2 * f + uc), b);
     unpack8(*(const uint4*)(ds + t * f + c * 8), d);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -276,8 +286,8 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restric
       a[e] = da;
       b[e] = db;
     }
-    *(uint4*)(dgu + t * 2 * f + c * 8) = pack8(a);
-    *(uint4*)(dgu + t * 2 * f + f + c * 8) = pack8(b);
+    *(uint4*)(dgu + t * 2 * f + gc) = pack8(a);
+    *(uint4*)(dgu + t * 2 * f + uc) = pack8(b);
   }
 }
 
@@ -471,22 +481,26 @@ int jpp_norm_bwd(void* stream, const jpp_norm_args* a) {
             : launch_norm_bwd<false>((hipStream_t)stream, a);
 }
 
-int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f) {
-  JPP_REQUIRE(gu && s && rows > 0 && f > 0 && f % 8 == 0, "swiglu_fwd: bad arguments");
+int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f,
+                   int interleaved) {
+  JPP_REQUIRE(gu && s && rows > 0 && f > 0 && f % (interleaved ? 32 : 8) == 0,
+              "swiglu_fwd: bad arguments");
   ProbeScope probe((hipStream_t)stream, "swiglu_fwd", 0, 6.0 * rows * f);
   hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid_for(rows * (f / 8))), dim3(256), 0,
-                     (hipStream_t)stream, (const bf16_t*)gu, (bf16_t*)s, (long)rows, (int)f);
+                     (hipStream_t)stream, (const bf16_t*)gu, (bf16_t*)s, (long)rows, (int)f,
+                     interleaved);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
 
 int jpp_swiglu_bwd(void* stream, const void* gu, const void* ds, void* dgu, int64_t rows,
-                   int64_t f) {
-  JPP_REQUIRE(gu && ds && dgu && rows > 0 && f > 0 && f % 8 == 0, "swiglu_bwd: bad arguments");
+                   int64_t f, int interleaved) {
+  JPP_REQUIRE(gu && ds && dgu && rows > 0 && f > 0 && f % (interleaved ? 32 : 8) == 0,
+              "swiglu_bwd: bad arguments");
   ProbeScope probe((hipStream_t)stream, "swiglu_bwd", 0, 10.0 * rows * f);
   hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid_for(rows * (f / 8))), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)gu, (const bf16_t*)ds, (bf16_t*)dgu,
-                     (long)rows, (int)f);
+                     (long)rows, (int)f, interleaved);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }

@@ -59,6 +59,17 @@ __device__ __forceinline__ float gelu_grad_f(float u, int tanh_form) {
          u * __expf(-0.5f * u * u) * 0.3989422804014327f;
 }
 
+// bf16 value of two packed elements, as floats (what a later kernel would read back)
+__device__ __forceinline__ float2 rounded(uint32_t packed) {
+  return make_float2(bf16lo_to_f32(packed), bf16hi_to_f32(packed));
+}
+__device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+__device__ __forceinline__ void swiglu_grad_f(float g, float u, float d, float& dg, float& du) {
+  const float sg = 1.0f / (1.0f + __expf(-g));
+  dg = d * u * sg * (1.0f + g * (1.0f - sg));
+  du = d * g * sg;
+}
+
 // Output tile of a workgroup.  Consecutive workgroup ids land on different
 // XCDs (8 of them, each with its own L2); give every XCD a contiguous range of
 // tiles, and inside a range walk GROUP tile-rows at a time so the B panels in
@@ -264,6 +275,64 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
           *(float4*)((float*)p.c + (m_lane + i * 32) * p.ldc + n_lane + j * 32 + g * 8) =
               make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
                           acc[i][j][4 * g + 3]);
+  } else if constexpr (EPI == JPP_EPI_SWIGLU) {
+    // a wave's 64 columns are 32 gate features (j = 0) and the same 32 up features (j = 1):
+    // one lane holds both halves of a pair.  Computed from the rounded bf16 values, as the
+    // separate kernel would from C.
+    static_assert(TN == 2 && BN / WN == 64, "gate/up blocks of 32 columns per wave");
+    const long f_lane = (n0 + wn * 64) / 2 + (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const long m = m_lane + i * 32;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint2 gp = make_uint2(pack_bf16x2(acc[i][0][4 * g], acc[i][0][4 * g + 1]),
+                                    pack_bf16x2(acc[i][0][4 * g + 2], acc[i][0][4 * g + 3]));
+        const uint2 up = make_uint2(pack_bf16x2(acc[i][1][4 * g], acc[i][1][4 * g + 1]),
+                                    pack_bf16x2(acc[i][1][4 * g + 2], acc[i][1][4 * g + 3]));
+        *(uint2*)((bf16_t*)p.c + m * p.ldc + n_lane + g * 8) = gp;
+        *(uint2*)((bf16_t*)p.c + m * p.ldc + n_lane + 32 + g * 8) = up;
+        const float2 g01 = rounded(gp.x), g23 = rounded(gp.y), u01 = rounded(up.x), u23 = rounded(up.y);
+        *(uint2*)((bf16_t*)p.c2 + m * p.ldc2 + f_lane + g * 8) =
+            make_uint2(pack_bf16x2(swiglu_f(g01.x, u01.x), swiglu_f(g01.y, u01.y)),
+                       pack_bf16x2(swiglu_f(g23.x, u23.x), swiglu_f(g23.y, u23.y)));
+      }
+    }
+  } else if constexpr (EPI == JPP_EPI_DSWIGLU) {
+    // acc = ds for 64 features per wave (j = 0, 1: two blocks of 32); gate and up of block q
+    // sit at columns 64q.. and 64q+32.. of aux, d(gate) and d(up) go to the same columns of C
+    static_assert(TN == 2 && BN / WN == 64, "gate/up blocks of 32 columns per wave");
+    const long c_lane = 2 * (n0 + wn * 64) + (lane >> 5) * 4;  // column of block j = 0, g = 0
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const long m = m_lane + i * 32;
+      uint2 gg[TN][4], uu[TN][4];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          gg[j][g] = *(const uint2*)(p.aux + m * p.ldaux + c_lane + j * 64 + g * 8);
+          uu[j][g] = *(const uint2*)(p.aux + m * p.ldaux + c_lane + j * 64 + 32 + g * 8);
+        }
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const float2 d01 = rounded(pack_bf16x2(acc[i][j][4 * g], acc[i][j][4 * g + 1]));
+          const float2 d23 = rounded(pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]));
+          const float2 g01 = rounded(gg[j][g].x), g23 = rounded(gg[j][g].y);
+          const float2 u01 = rounded(uu[j][g].x), u23 = rounded(uu[j][g].y);
+          float dg[4], du[4];
+          swiglu_grad_f(g01.x, u01.x, d01.x, dg[0], du[0]);
+          swiglu_grad_f(g01.y, u01.y, d01.y, dg[1], du[1]);
+          swiglu_grad_f(g23.x, u23.x, d23.x, dg[2], du[2]);
+          swiglu_grad_f(g23.y, u23.y, d23.y, dg[3], du[3]);
+          *(uint2*)((bf16_t*)p.c + m * p.ldc + c_lane + j * 64 + g * 8) =
+              make_uint2(pack_bf16x2(dg[0], dg[1]), pack_bf16x2(dg[2], dg[3]));
+          *(uint2*)((bf16_t*)p.c + m * p.ldc + c_lane + j * 64 + 32 + g * 8) =
+              make_uint2(pack_bf16x2(du[0], du[1]), pack_bf16x2(du[2], du[3]));
+        }
+    }
   } else {
     // Operands of the epilogue (bias, residual, GELU pre-activation) are fetched in one
     // batch per row of MFMA tiles before anything is stored: a load issued between stores
@@ -328,7 +397,8 @@ const char* class_name() {
   if (!name[0]) {
     const char* lay = TA ? "tn" : (TB ? "nn" : "nt");
     const char* epi = EPI == JPP_EPI_BF16 ? "bf16" : EPI == JPP_EPI_GELU ? "gelu"
-                    : EPI == JPP_EPI_DGELU ? "dgelu" : EPI == JPP_EPI_ACC_F32 ? "accf32" : "f32";
+                    : EPI == JPP_EPI_DGELU ? "dgelu" : EPI == JPP_EPI_ACC_F32 ? "accf32"
+                    : EPI == JPP_EPI_SWIGLU ? "swiglu" : EPI == JPP_EPI_DSWIGLU ? "dswiglu" : "f32";
     snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d%s", lay, epi, BM, BN, NW == 8 ? "w8" : "");
   }
   return name;
@@ -338,7 +408,8 @@ template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4>
 int launch(hipStream_t stream, GemmParams& p) {
   constexpr int SMEM = 2 * (BM + BN) * 128;
   // algorithmic extent: grouped launches count the non-padding rows when the caller gave them
-  const double cb = EPI == JPP_EPI_ACC_F32 ? 8 : EPI == JPP_EPI_F32 ? 4 : 2;
+  const double cb = EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_DSWIGLU ? 8
+                    : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;
   double am = p.m, ak = p.k, copies = 1;
   if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
   if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
@@ -424,6 +495,14 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     JPP_REQUIRE(a->c2 && a->ldc2 >= a->n && a->ldc2 % 4 == 0, "gemm: GELU epilogue needs c2");
   if (a->epilogue == JPP_EPI_DGELU)
     JPP_REQUIRE(a->aux && a->ldaux >= a->n && a->ldaux % 4 == 0, "gemm: dGELU epilogue needs aux");
+  if (a->epilogue == JPP_EPI_SWIGLU)
+    JPP_REQUIRE(a->c2 && a->ldc2 >= a->n / 2 && a->ldc2 % 4 == 0 && !a->bias && !a->resid &&
+                    a->group_mode == JPP_GROUP_NONE,
+                "gemm: SwiGLU epilogue needs c2 [M, N/2] and takes no bias / residual / groups");
+  if (a->epilogue == JPP_EPI_DSWIGLU)
+    JPP_REQUIRE(a->aux && a->ldaux >= 2 * a->n && a->ldaux % 4 == 0 && a->ldc >= 2 * a->n &&
+                    !a->bias && !a->resid && a->group_mode == JPP_GROUP_NONE,
+                "gemm: dSwiGLU epilogue needs aux and C of width 2N and takes no bias / residual / groups");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
   if (a->group_mode != JPP_GROUP_NONE) tile = 4;  // 256-row segments
@@ -437,8 +516,10 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   JPP_GEMM_CASE(0, 1, JPP_EPI_BF16);     // forward
   JPP_GEMM_CASE(0, 1, JPP_EPI_GELU);     // forward + GELU
   JPP_GEMM_CASE(0, 1, JPP_EPI_F32);      // forward, f32 out (router logits)
+  JPP_GEMM_CASE(0, 1, JPP_EPI_SWIGLU);   // gate/up projection + SwiGLU
   JPP_GEMM_CASE(0, 0, JPP_EPI_BF16);     // input gradient
   JPP_GEMM_CASE(0, 0, JPP_EPI_DGELU);    // input gradient through GELU
+  JPP_GEMM_CASE(0, 0, JPP_EPI_DSWIGLU);  // input gradient through SwiGLU
   JPP_GEMM_CASE(1, 1, JPP_EPI_ACC_F32);  // weight gradient, accumulated
   JPP_GEMM_CASE(1, 1, JPP_EPI_BF16);     // weight gradient, bf16
   JPP_GEMM_CASE(1, 1, JPP_EPI_F32);      // weight gradient, f32

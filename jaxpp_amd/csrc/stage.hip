@@ -253,15 +253,15 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
     RC(jpp_moe_gather(st, &ma, at(L.n2), at(L.xp)));
     RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.xp), h, 0, s->P(chunk, li, X_Wgu), 2 * f, 1, h * 2 * f,
              at(L.gu), 2 * f, 0, s->cap, 2 * f, h, JPP_EPI_BF16, s->T * s->d.top_k));
-    RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), s->cap, f));
+    RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), s->cap, f, 0));
     RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.s), f, 0, s->P(chunk, li, X_Wd), h, 1, f * h, at(L.eo), h,
              0, s->cap, h, f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_fwd(st, &ma, at(L.eo), at(L.h1), y));
     return JPP_OK;
   }
+  // gate and up columns of Wgu are interleaved in blocks of 32: SwiGLU runs in the epilogue
   RC(gemm(st, at(L.n2), h, 0, s->P(chunk, li, L_Wgu), 2 * f, 1, at(L.gu), 2 * f, T, 2 * f, h,
-          JPP_EPI_BF16));
-  RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), T, f));
+          JPP_EPI_SWIGLU, nullptr, nullptr, 0, nullptr, 0, at(L.s), f));
   RC(gemm(st, at(L.s), f, 0, s->P(chunk, li, L_Wd), h, 1, y, h, T, h, f, JPP_EPI_BF16, nullptr,
           at(L.h1), h));
   return JPP_OK;
@@ -319,13 +319,15 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(jpp_moe_bwd_prepare(st, &ma, dy, at(L.eo), (float*)wt(W.dlogits), wt(W.deo)));
     RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.deo), h, 0, s->P(chunk, li, X_Wd), h, 0, f * h, ds, f,
              0, s->cap, f, h, JPP_EPI_BF16, s->T * s->d.top_k));
-    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), s->cap, f));
+    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), s->cap, f, 0));
     RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.dgu), 2 * f, 0, s->P(chunk, li, X_Wgu), 2 * f, 0,
              h * 2 * f, dxp, h, 0, s->cap, h, 2 * f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_bwd(st, &ma, dxp, (const float*)wt(W.dlogits), dn));
   } else {
+    // (JPP_EPI_DSWIGLU would fold the next kernel into this GEMM; measured slower at these
+    // shapes: its epilogue reads gate/up with the matrix cores idle)
     RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, ds, f, T, f, h, JPP_EPI_BF16));
-    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), T, f));
+    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), T, f, 1));
     RC(gemm(st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
             JPP_EPI_BF16));
   }

@@ -76,7 +76,7 @@ class StageDesc(C.Structure):
                 ("two_streams", C.c_int)]
 
 
-EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32 = range(5)
+EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32, EPI_SWIGLU, EPI_DSWIGLU = range(7)
 NORM_PARTIALS = 256
 FAMILY = {"bert": 0, "llama": 1, "mixtral": 2}
 
@@ -140,9 +140,10 @@ def load():
     lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_norm_fwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
     lib.jpp_norm_bwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
-    lib.jpp_swiglu_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]
+    lib.jpp_swiglu_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                   C.c_int]
     lib.jpp_swiglu_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
-                                   C.c_int64]
+                                   C.c_int64, C.c_int]
     lib.jpp_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int,
                              C.c_int, C.c_int, C.c_int, C.c_int]
     lib.jpp_grad_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
@@ -396,11 +397,26 @@ class StageExecutor:
         check(fn(self.handle, chunk, layer, self.index[name], C.byref(p)))
         return p.value
 
+    def _device_columns(self, name: str, cols: int):
+        """Column order of a parameter in device memory, or None when it is the host's.  The
+        Llama layer keeps ``Wgu = [gate | up]`` with the two projections interleaved in blocks
+        of 32 columns (device column 64q+w = gate feature 32q+w for w < 32, up feature 32q+w-32
+        otherwise), which lets the GEMM epilogue apply SwiGLU (JPP_EPI_SWIGLU)."""
+        if self.spec.family != "llama" or name != "Wgu":
+            return None
+        f = cols // 2
+        c = np.arange(cols)
+        q, w = c // 64, c % 64
+        return np.where(w < 32, 32 * q + w, f + 32 * q + w - 32)
+
     def set_params(self, chunk: int, layer: int, params: dict):
         """Upload float32 host arrays as bf16 device parameters."""
         for name, rows, cols in self.params:
             a = np.asarray(params[name], dtype=np.float32)
             assert a.size == rows * cols, (name, a.shape, rows, cols)
+            order = self._device_columns(name, cols)
+            if order is not None:
+                a = np.ascontiguousarray(a.reshape(rows, cols)[:, order])
             upload_ptr(self._ptr(load().jpp_stage_param_ptr, chunk, layer, name),
                        to_bf16_bits(a))
 
@@ -409,8 +425,14 @@ class StageExecutor:
         out = {}
         for name, rows, cols in self.params:
             shape = (cols,) if rows == 1 and not name.startswith("W") else (rows, cols)
-            out[name] = download_ptr(self._ptr(load().jpp_stage_grad_ptr, chunk, layer, name),
-                                     np.float32, shape)
+            g = download_ptr(self._ptr(load().jpp_stage_grad_ptr, chunk, layer, name),
+                             np.float32, shape)
+            order = self._device_columns(name, cols)
+            if order is not None:
+                host = np.empty_like(g)
+                host[:, order] = g
+                g = host
+            out[name] = g
         return out
 
     def zero_grads(self, stream=None):

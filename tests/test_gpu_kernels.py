@@ -35,6 +35,16 @@ def close(got, want, rtol=2e-2, what=""):
     assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
 
 
+def interleave32(gate, up):
+    """[.., f] gate and up -> [.., 2f] with blocks of 32 gate columns followed by their 32 ups."""
+    f = gate.shape[-1]
+    out = np.empty(gate.shape[:-1] + (2 * f,), gate.dtype)
+    o = out.reshape(gate.shape[:-1] + (f // 32, 64))
+    o[..., :32] = gate.reshape(gate.shape[:-1] + (f // 32, 32))
+    o[..., 32:] = up.reshape(up.shape[:-1] + (f // 32, 32))
+    return out
+
+
 GEMM_CASES = [  # (trans_a, trans_b, epilogue)
     (0, 1, rt.EPI_BF16), (0, 1, rt.EPI_GELU), (0, 1, rt.EPI_F32),
     (0, 0, rt.EPI_BF16), (0, 0, rt.EPI_DGELU),
@@ -191,11 +201,20 @@ def test_swiglu_rope_accum_colsum_cast():
     gu, ds = rnd(rng, rows, 2 * f, scale=2.0), rnd(rng, rows, f)
     bgu, bds = dev_bf16(gu), dev_bf16(ds)
     bs, bdgu = rt.DeviceBuffer(rows * f * 2), rt.DeviceBuffer(rows * 2 * f * 2)
-    rt.check(lib.jpp_swiglu_fwd(None, bgu.ptr, bs.ptr, rows, f))
-    rt.check(lib.jpp_swiglu_bwd(None, bgu.ptr, bds.ptr, bdgu.ptr, rows, f))
+    rt.check(lib.jpp_swiglu_fwd(None, bgu.ptr, bs.ptr, rows, f, 0))
+    rt.check(lib.jpp_swiglu_bwd(None, bgu.ptr, bds.ptr, bdgu.ptr, rows, f, 0))
     rt.sync()
     close(bs.download_bf16((rows, f)), L.swiglu(gu, f), 1e-2, "swiglu")
-    close(bdgu.download_bf16((rows, 2 * f)), L.swiglu_bwd(gu, ds, f), 1e-2, "swiglu bwd")
+    dgu_w = L.swiglu_bwd(gu, ds, f)
+    close(bdgu.download_bf16((rows, 2 * f)), dgu_w, 1e-2, "swiglu bwd")
+    # the same through the layout with gate and up interleaved in blocks of 32 columns
+    bgi = dev_bf16(interleave32(gu[:, :f], gu[:, f:]))
+    rt.check(lib.jpp_swiglu_fwd(None, bgi.ptr, bs.ptr, rows, f, 1))
+    rt.check(lib.jpp_swiglu_bwd(None, bgi.ptr, bds.ptr, bdgu.ptr, rows, f, 1))
+    rt.sync()
+    close(bs.download_bf16((rows, f)), L.swiglu(gu, f), 1e-2, "swiglu, interleaved")
+    close(bdgu.download_bf16((rows, 2 * f)), interleave32(dgu_w[:, :f], dgu_w[:, f:]), 1e-2,
+          "swiglu bwd, interleaved")
 
     batch, seq, heads, d, extra = 2, 64, 6, 128, 2
     ld = (heads + extra) * d
@@ -362,3 +381,34 @@ def test_grouped_gemm():
         want = acc0[e] + xp[seg[e]:seg[e + 1]].T @ dy[seg[e]:seg[e + 1]]
         close(got[e], want, 1e-3, f"dW group {e}")
     np.testing.assert_array_equal(got[1], acc0[1])       # empty group: untouched
+
+
+@pytest.mark.parametrize("tile,m,f,k", [(1, 128, 128, 64), (2, 256, 256, 128), (4, 512, 256, 192)])
+def test_gemm_swiglu_epilogues(tile, m, f, k):
+    rng = np.random.default_rng(21)
+    x = rnd(rng, m, k)
+    wg, wu = rnd(rng, k, f, scale=0.2), rnd(rng, k, f, scale=0.2)
+    w = interleave32(wg, wu)                       # device layout of the fused projection
+    gu, s = rt.DeviceBuffer(m * 2 * f * 2), rt.DeviceBuffer(m * f * 2)
+    dx, dw = dev_bf16(x), dev_bf16(w)
+    rt.gemm(dx.ptr, dw.ptr, gu.ptr, m, 2 * f, k, k, 2 * f, 2 * f, 0, 1, rt.EPI_SWIGLU, c2=s.ptr,
+            ldc2=f, tile=tile)
+    rt.sync()
+    g_w, u_w = L.bf16_round(x @ wg), L.bf16_round(x @ wu)
+    gu_h = gu.download_bf16((m, 2 * f))
+    close(gu_h, interleave32(g_w, u_w), 1e-2, "gate/up")
+    # the second output follows from the first exactly as the separate kernel computes it
+    g_h = gu_h.reshape(m, f // 32, 64)[..., :32].reshape(m, f)
+    u_h = gu_h.reshape(m, f // 32, 64)[..., 32:].reshape(m, f)
+    close(s.download_bf16((m, f)), g_h / (1 + np.exp(-g_h)) * u_h, 1e-2, "swiglu")
+    # backward: ds = dy Wd^T, then through SwiGLU, written interleaved
+    n_out = 128
+    dy, wd = rnd(rng, m, n_out), rnd(rng, f, n_out, scale=0.2)
+    ddy, dwd, dgu = dev_bf16(dy), dev_bf16(wd), rt.DeviceBuffer(m * 2 * f * 2)
+    rt.gemm(ddy.ptr, dwd.ptr, dgu.ptr, m, f, n_out, n_out, n_out, 2 * f, 0, 0, rt.EPI_DSWIGLU,
+            aux=gu.ptr, ldaux=2 * f, tile=tile)
+    rt.sync()
+    ds = L.bf16_round(dy @ wd.T)
+    sg = 1 / (1 + np.exp(-g_h))
+    want = interleave32(ds * u_h * sg * (1 + g_h * (1 - sg)), ds * g_h * sg)
+    close(dgu.download_bf16((m, 2 * f)), want, 1e-2, "dgate/dup")
