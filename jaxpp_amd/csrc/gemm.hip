@@ -59,10 +59,6 @@ __device__ __forceinline__ float gelu_grad_f(float u, int tanh_form) {
          u * __expf(-0.5f * u * u) * 0.3989422804014327f;
 }
 
-// bf16 value of two packed elements, as floats (what a later kernel would read back)
-__device__ __forceinline__ float2 rounded(uint32_t packed) {
-  return make_float2(bf16lo_to_f32(packed), bf16hi_to_f32(packed));
-}
 __device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
 __device__ __forceinline__ void swiglu_grad_f(float g, float u, float d, float& dg, float& du) {
   const float sg = 1.0f / (1.0f + __expf(-g));
@@ -275,116 +271,114 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
           *(float4*)((float*)p.c + (m_lane + i * 32) * p.ldc + n_lane + j * 32 + g * 8) =
               make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
                           acc[i][j][4 * g + 3]);
-  } else if constexpr (EPI == JPP_EPI_SWIGLU) {
-    // a wave's 64 columns are 32 gate features (j = 0) and the same 32 up features (j = 1):
-    // one lane holds both halves of a pair.  Computed from the rounded bf16 values, as the
-    // separate kernel would from C.
-    static_assert(TN == 2 && BN / WN == 64, "gate/up blocks of 32 columns per wave");
-    const long f_lane = (n0 + wn * 64) / 2 + (lane >> 5) * 4;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const long m = m_lane + i * 32;
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const uint2 gp = make_uint2(pack_bf16x2(acc[i][0][4 * g], acc[i][0][4 * g + 1]),
-                                    pack_bf16x2(acc[i][0][4 * g + 2], acc[i][0][4 * g + 3]));
-        const uint2 up = make_uint2(pack_bf16x2(acc[i][1][4 * g], acc[i][1][4 * g + 1]),
-                                    pack_bf16x2(acc[i][1][4 * g + 2], acc[i][1][4 * g + 3]));
-        *(uint2*)((bf16_t*)p.c + m * p.ldc + n_lane + g * 8) = gp;
-        *(uint2*)((bf16_t*)p.c + m * p.ldc + n_lane + 32 + g * 8) = up;
-        const float2 g01 = rounded(gp.x), g23 = rounded(gp.y), u01 = rounded(up.x), u23 = rounded(up.y);
-        *(uint2*)((bf16_t*)p.c2 + m * p.ldc2 + f_lane + g * 8) =
-            make_uint2(pack_bf16x2(swiglu_f(g01.x, u01.x), swiglu_f(g01.y, u01.y)),
-                       pack_bf16x2(swiglu_f(g23.x, u23.x), swiglu_f(g23.y, u23.y)));
-      }
-    }
-  } else if constexpr (EPI == JPP_EPI_DSWIGLU) {
-    // acc = ds for 64 features per wave (j = 0, 1: two blocks of 32); gate and up of block q
-    // sit at columns 64q.. and 64q+32.. of aux, d(gate) and d(up) go to the same columns of C
-    static_assert(TN == 2 && BN / WN == 64, "gate/up blocks of 32 columns per wave");
-    const long c_lane = 2 * (n0 + wn * 64) + (lane >> 5) * 4;  // column of block j = 0, g = 0
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const long m = m_lane + i * 32;
-      uint2 gg[TN][4], uu[TN][4];
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          gg[j][g] = *(const uint2*)(p.aux + m * p.ldaux + c_lane + j * 64 + g * 8);
-          uu[j][g] = *(const uint2*)(p.aux + m * p.ldaux + c_lane + j * 64 + 32 + g * 8);
-        }
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float2 d01 = rounded(pack_bf16x2(acc[i][j][4 * g], acc[i][j][4 * g + 1]));
-          const float2 d23 = rounded(pack_bf16x2(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]));
-          const float2 g01 = rounded(gg[j][g].x), g23 = rounded(gg[j][g].y);
-          const float2 u01 = rounded(uu[j][g].x), u23 = rounded(uu[j][g].y);
-          float dg[4], du[4];
-          swiglu_grad_f(g01.x, u01.x, d01.x, dg[0], du[0]);
-          swiglu_grad_f(g01.y, u01.y, d01.y, dg[1], du[1]);
-          swiglu_grad_f(g23.x, u23.x, d23.x, dg[2], du[2]);
-          swiglu_grad_f(g23.y, u23.y, d23.y, dg[3], du[3]);
-          *(uint2*)((bf16_t*)p.c + m * p.ldc + c_lane + j * 64 + g * 8) =
-              make_uint2(pack_bf16x2(dg[0], dg[1]), pack_bf16x2(dg[2], dg[3]));
-          *(uint2*)((bf16_t*)p.c + m * p.ldc + c_lane + j * 64 + 32 + g * 8) =
-              make_uint2(pack_bf16x2(du[0], du[1]), pack_bf16x2(du[2], du[3]));
-        }
-    }
   } else {
-    // Operands of the epilogue (bias, residual, GELU pre-activation) are fetched in one
-    // batch per row of MFMA tiles before anything is stored: a load issued between stores
-    // would have to wait for those stores as well (one counter orders both).
-    uint2 bb[TN][4];
-    if (p.bias) {
+    // bf16 outputs.  An accumulator lane holds one row and 4 consecutive columns, so storing
+    // from that layout scatters 8-byte pieces over 32 rows per instruction.  Instead the tile
+    // goes through LDS (free after the K loop) half at a time - fp32, [BM/2 rows][BN + 4]
+    // - and is taken back out by rows: a thread owns 8 consecutive columns of a row, so
+    // every global access of the epilogue (output, residual, pre-activation, gate/up) is a
+    // 16-byte piece of a contiguous run, and the arithmetic runs in fp32 exactly as before.
+    constexpr int HALF = BM / 2, PITCH = BN * 4 + 16, NT = NW * 64;
+    const int hh = lane >> 5;
+    const bf16_t* bias = p.bias;
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+      __syncthreads();  // fragments of the last K-step / the previous half are out of LDS
+      if (wm == half) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) bb[j][g] = *(const uint2*)(p.bias + n_lane + j * 32 + g * 8);
-    }
+          for (int j = 0; j < TN; ++j)
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const long m = m_lane + i * 32;
-      uint2 xx[TN][4];  // residual, or the pre-activation of the GELU gradient
-      const bf16_t* extra = EPI == JPP_EPI_DGELU ? p.aux : (EPI == JPP_EPI_BF16 ? p.resid : nullptr);
-      const long ldx = EPI == JPP_EPI_DGELU ? p.ldaux : p.ldresid;
-      if (extra) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-            xx[j][g] = *(const uint2*)(extra + m * ldx + n_lane + j * 32 + g * 8);
+            for (int g = 0; g < 4; ++g)
+              *(float4*)(smem + (i * 32 + (lane & 31)) * PITCH +
+                         (wn * (BN / WN) + j * 32 + g * 8 + hh * 4) * 4) =
+                  make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                              acc[i][j][4 * g + 3]);
       }
+      __syncthreads();
+      const long mrow0 = m0 + half * HALF;
+      if constexpr (EPI == JPP_EPI_SWIGLU) {
+        // a thread owns 8 features of a row: gate at columns 64q + w, up at 64q + 32 + w
+        constexpr int TPR = BN / 16, RPI = NT / TPR;  // threads per row, rows per sweep
+        const int fc = tid % TPR, q = fc >> 2, w = (fc & 3) * 8;
+        for (int r = tid / TPR; r < HALF; r += RPI) {
+          const uint8_t* row = smem + r * PITCH + (q * 64 + w) * 4;
+          const float4 g0 = *(const float4*)row, g1 = *(const float4*)(row + 16);
+          const float4 u0 = *(const float4*)(row + 128), u1 = *(const float4*)(row + 144);
+          const uint4 gp = make_uint4(pack_bf16x2(g0.x, g0.y), pack_bf16x2(g0.z, g0.w),
+                                      pack_bf16x2(g1.x, g1.y), pack_bf16x2(g1.z, g1.w));
+          const uint4 up = make_uint4(pack_bf16x2(u0.x, u0.y), pack_bf16x2(u0.z, u0.w),
+                                      pack_bf16x2(u1.x, u1.y), pack_bf16x2(u1.z, u1.w));
+          bf16_t* crow = (bf16_t*)p.c + (mrow0 + r) * p.ldc + n0 + q * 64 + w;
+          *(uint4*)crow = gp;
+          *(uint4*)(crow + 32) = up;
+          // from the rounded values, as a separate kernel would read them back
+          float gv[8], uv[8];
+          unpack8(gp, gv);
+          unpack8(up, uv);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
+          for (int e = 0; e < 8; ++e) gv[e] = swiglu_f(gv[e], uv[e]);
+          *(uint4*)((bf16_t*)p.c2 + (mrow0 + r) * p.ldc2 + n0 / 2 + q * 32 + w) = pack8(gv);
+        }
+      } else if constexpr (EPI == JPP_EPI_DSWIGLU) {
+        // the tile holds ds for BN features; gate / up of block q at columns 64q.., 64q+32..
+        constexpr int TPR = BN / 8, RPI = NT / TPR;
+        const int fc = tid % TPR, q = fc >> 2, w = (fc & 3) * 8;
+        for (int r = tid / TPR; r < HALF; r += RPI) {
+          const uint8_t* row = smem + r * PITCH + fc * 32;
+          const float4 d0 = *(const float4*)row, d1 = *(const float4*)(row + 16);
+          const long col = 2 * n0 + q * 64 + w;
+          const bf16_t* arow = p.aux + (mrow0 + r) * p.ldaux + col;
+          float gv[8], uv[8], dv[8];
+          unpack8(*(const uint4*)arow, gv);
+          unpack8(*(const uint4*)(arow + 32), uv);
+          unpack8(make_uint4(pack_bf16x2(d0.x, d0.y), pack_bf16x2(d0.z, d0.w),
+                             pack_bf16x2(d1.x, d1.y), pack_bf16x2(d1.z, d1.w)), dv);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const long n = n_lane + j * 32 + g * 8;
-          float v0 = acc[i][j][4 * g + 0], v1 = acc[i][j][4 * g + 1];
-          float v2 = acc[i][j][4 * g + 2], v3 = acc[i][j][4 * g + 3];
-          if (p.bias) {
-            v0 += bf16lo_to_f32(bb[j][g].x); v1 += bf16hi_to_f32(bb[j][g].x);
-            v2 += bf16lo_to_f32(bb[j][g].y); v3 += bf16hi_to_f32(bb[j][g].y);
+          for (int e = 0; e < 8; ++e) {
+            float dg, du;
+            swiglu_grad_f(gv[e], uv[e], dv[e], dg, du);
+            gv[e] = dg;
+            uv[e] = du;
+          }
+          bf16_t* crow = (bf16_t*)p.c + (mrow0 + r) * p.ldc + col;
+          *(uint4*)crow = pack8(gv);
+          *(uint4*)(crow + 32) = pack8(uv);
+        }
+      } else {
+        constexpr int TPR = BN / 8, RPI = NT / TPR;
+        const int c8 = (tid % TPR) * 8;
+        float bv[8];
+        if (bias) unpack8(*(const uint4*)(bias + n0 + c8), bv);
+        for (int r = tid / TPR; r < HALF; r += RPI) {
+          const uint8_t* row = smem + r * PITCH + c8 * 4;
+          const float4 a0 = *(const float4*)row, a1 = *(const float4*)(row + 16);
+          float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+          const long at = (mrow0 + r) * p.ldc + n0 + c8;
+          if (bias) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += bv[e];
           }
           if constexpr (EPI == JPP_EPI_BF16) {
-            if (extra) {
-              v0 += bf16lo_to_f32(xx[j][g].x); v1 += bf16hi_to_f32(xx[j][g].x);
-              v2 += bf16lo_to_f32(xx[j][g].y); v3 += bf16hi_to_f32(xx[j][g].y);
+            if (p.resid) {
+              float rv[8];
+              unpack8(*(const uint4*)(p.resid + (mrow0 + r) * p.ldresid + n0 + c8), rv);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] += rv[e];
             }
           } else if constexpr (EPI == JPP_EPI_GELU) {
-            *(uint2*)((bf16_t*)p.c2 + m * p.ldc2 + n) =
-                make_uint2(pack_bf16x2(gelu_f(v0, p.gelu_tanh), gelu_f(v1, p.gelu_tanh)),
-                           pack_bf16x2(gelu_f(v2, p.gelu_tanh), gelu_f(v3, p.gelu_tanh)));
+            float gl[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) gl[e] = gelu_f(v[e], p.gelu_tanh);
+            *(uint4*)((bf16_t*)p.c2 + (mrow0 + r) * p.ldc2 + n0 + c8) = pack8(gl);
           } else if constexpr (EPI == JPP_EPI_DGELU) {
-            v0 *= gelu_grad_f(bf16lo_to_f32(xx[j][g].x), p.gelu_tanh);
-            v1 *= gelu_grad_f(bf16hi_to_f32(xx[j][g].x), p.gelu_tanh);
-            v2 *= gelu_grad_f(bf16lo_to_f32(xx[j][g].y), p.gelu_tanh);
-            v3 *= gelu_grad_f(bf16hi_to_f32(xx[j][g].y), p.gelu_tanh);
+            float uv[8];
+            unpack8(*(const uint4*)(p.aux + (mrow0 + r) * p.ldaux + n0 + c8), uv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] *= gelu_grad_f(uv[e], p.gelu_tanh);
           }
-          *(uint2*)((bf16_t*)p.c + m * p.ldc + n) =
-              make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+          *(uint4*)((bf16_t*)p.c + at) = pack8(v);
         }
       }
     }
@@ -406,7 +400,10 @@ const char* class_name() {
 
 template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4>
 int launch(hipStream_t stream, GemmParams& p) {
-  constexpr int SMEM = 2 * (BM + BN) * 128;
+  // two operand stages; the bf16 epilogues stage half a tile in fp32 with padded rows
+  constexpr int SMEM_LOOP = 2 * (BM + BN) * 128, SMEM_EPI = (BM / 2) * (BN * 4 + 16);
+  constexpr int SMEM = (EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_F32 || SMEM_LOOP > SMEM_EPI)
+                           ? SMEM_LOOP : SMEM_EPI;
   // algorithmic extent: grouped launches count the non-padding rows when the caller gave them
   const double cb = EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_DSWIGLU ? 8
                     : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;

@@ -16,16 +16,6 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
   return v;
 }
-__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
-  f[0] = bf16lo_to_f32(v.x); f[1] = bf16hi_to_f32(v.x);
-  f[2] = bf16lo_to_f32(v.y); f[3] = bf16hi_to_f32(v.y);
-  f[4] = bf16lo_to_f32(v.z); f[5] = bf16hi_to_f32(v.z);
-  f[6] = bf16lo_to_f32(v.w); f[7] = bf16hi_to_f32(v.w);
-}
-__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
-  return make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                    pack_bf16x2(f[6], f[7]));
-}
 
 // logits = x Wr (fp32), top-2 by value (ties -> lower index), gates = softmax
 // over the two selected logits.  One wave per token.
