@@ -324,10 +324,8 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
              h * 2 * f, dxp, h, 0, s->cap, h, 2 * f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_bwd(st, &ma, dxp, (const float*)wt(W.dlogits), dn));
   } else {
-    // (JPP_EPI_DSWIGLU would fold the next kernel into this GEMM; measured slower at these
-    // shapes: its epilogue reads gate/up with the matrix cores idle)
-    RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, ds, f, T, f, h, JPP_EPI_BF16));
-    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), T, f, 1));
+    RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, wt(W.dgu), 2 * f, T, f, h, JPP_EPI_DSWIGLU,
+            nullptr, nullptr, 0, at(L.gu), 2 * f));
     RC(gemm(st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
             JPP_EPI_BF16));
   }
