@@ -262,15 +262,35 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   dma_wait_all();   // the refetches of the last two K-steps must not outlive the block's LDS
 
   if constexpr (EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_F32) {
+    // fp32 outputs leave through LDS as well (see below), a quarter of the tile per pass:
+    // 16-byte stores of contiguous rows instead of 32-byte pieces of 32 rows
+    constexpr int IPP = TM >= 2 ? TM / 2 : 1, RP = IPP * 32, PITCH = BN * 4 + 16, NT = NW * 64;
+    constexpr int TPR = BN / 4, RPI = NT / TPR;
+#pragma unroll 1
+    for (int pass = 0; pass < 2 * (TM / IPP); ++pass) {
+      const int half = pass / (TM / IPP), i0 = (pass % (TM / IPP)) * IPP;
+      __syncthreads();
+      if (wm == half) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
+          if (i >= i0 && i < i0 + IPP) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
-          *(float4*)((float*)p.c + (m_lane + i * 32) * p.ldc + n_lane + j * 32 + g * 8) =
-              make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                          acc[i][j][4 * g + 3]);
+              for (int g = 0; g < 4; ++g)
+                *(float4*)(smem + ((i - i0) * 32 + (lane & 31)) * PITCH +
+                           (wn * (BN / WN) + j * 32 + g * 8 + (lane >> 5) * 4) * 4) =
+                    make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                                acc[i][j][4 * g + 3]);
+          }
+      }
+      __syncthreads();
+      const long mrow0 = m0 + half * (BM / 2) + i0 * 32;
+      const int c4 = (tid % TPR) * 4;
+      for (int r = tid / TPR; r < RP; r += RPI)
+        *(float4*)((float*)p.c + (mrow0 + r) * p.ldc + n0 + c4) =
+            *(const float4*)(smem + r * PITCH + c4 * 4);
+    }
   } else {
     // bf16 outputs.  An accumulator lane holds one row and 4 consecutive columns, so storing
     // from that layout scatters 8-byte pieces over 32 rows per instruction.  Instead the tile
