@@ -126,21 +126,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   const long m_lane = m0 + wm * (BM / 2) + (lane & 31);
   const long n_lane = n0 + wn * (BN / WN) + (lane >> 5) * 4;
   f32x16 acc[TM][TN];
-  // C += A B (EPI_ACC_F32): the fp32 tile in memory is read in TM batches (one row of MFMA
-  // tiles each) during the first K-steps - requested at the end of K-step t, folded into the
-  // accumulators at the end of K-step t+1, where the wave waits for its operand copies
-  // anyway - and the epilogue only stores.  A read-modify-write epilogue would wait for HBM
-  // with the matrix cores idle.  Short K loops read the tile up front instead.
-  const bool stream_c = EPI == JPP_EPI_ACC_F32 && kt_n > TM;
-  float4 cbuf[TN][4];
-  auto load_c_row = [&](int i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-        cbuf[j][g] = *(const float4*)((const float*)p.c + (m_lane + i * 32) * p.ldc + n_lane +
-                                      j * 32 + g * 8);
-  };
+  // C += A B (EPI_ACC_F32): the epilogue only stores; the fp32 tile in memory is folded into
+  // the accumulators during the first K-steps.  It travels HBM -> LDS like the operands, NW
+  // whole rows (BN * 4 bytes each, one per wave) at a time, into one of two buffers behind
+  // the operand stages: batch b is requested at the end of K-step b, after that K-step's
+  // operand copies, and read out of LDS at the wait point of K-step b+2.  The wait of
+  // K-step b+1 leaves the youngest request in flight (vmcnt counts in order), so a batch has
+  // two K-steps to arrive and no K-step waits for HBM on its account; reading whole rows
+  // keeps HBM on long bursts where a lane-per-row layout would touch 32 rows at once.  K
+  // loops too short for that read the tile into the accumulators up front.
+  static_assert(BN * 4 <= 1024, "a row of the fp32 tile is one 64-lane copy");
+  constexpr int NBT = BM / NW, C_LDS = 2 * (BM + BN) * 128, C_PITCH = 1024 + 16;  // a copy is 1 KB
+  const bool stream_c = EPI == JPP_EPI_ACC_F32 && kt_n >= NBT + 2;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -150,18 +147,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   if constexpr (EPI == JPP_EPI_ACC_F32) {
     if (!stream_c) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        load_c_row(i);
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            acc[i][j][4 * g] = cbuf[j][g].x; acc[i][j][4 * g + 1] = cbuf[j][g].y;
-            acc[i][j][4 * g + 2] = cbuf[j][g].z; acc[i][j][4 * g + 3] = cbuf[j][g].w;
+            const float4 c = *(const float4*)((const float*)p.c + (m_lane + i * 32) * p.ldc +
+                                              n_lane + j * 32 + g * 8);
+            acc[i][j][4 * g] = c.x; acc[i][j][4 * g + 1] = c.y;
+            acc[i][j][4 * g + 2] = c.z; acc[i][j][4 * g + 3] = c.w;
           }
-      }
     }
   }
+  // byte offset, from the start of C, of this lane's 16 bytes of tile row `wave`
+  // (lanes past the end of a narrow row repeat its last piece)
+  const uint32_t c_off0 =
+      (uint32_t)(((m0 + wave) * p.ldc + n0 + min(lane, BN / 4 - 1) * 4) * 4);
   const uint32_t lds0 = lds_address(smem);
   typename TileA::Offsets offa;
   typename TileB::Offsets offb;
@@ -217,25 +218,33 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
       } else {
         // every fragment of this stage is in registers: once all waves are here (and the
         // other stage, requested one K-step ago, has landed) this stage can be refilled
-        dma_wait_all();
+        if (EPI == JPP_EPI_ACC_F32 && stream_c && kt >= 1 && kt <= NBT)
+          dma_wait<1>();  // all but the accumulator row requested at the end of K-step kt-1
+        else
+          dma_wait_all();
         lds_wait_all();
         __syncthreads();
         if constexpr (EPI == JPP_EPI_ACC_F32) {
-          if (stream_c && kt <= TM) {
-            // everything this wave had in flight has landed: fold in the row requested one
-            // K-step ago, request the next one
+          if (stream_c && kt >= 2 && kt <= NBT + 1) {
+            // batch kt-2 (tile rows NW (kt-2) .. + NW-1) is in LDS: the lanes that hold those
+            // rows in their accumulators add them in
+            const int row0 = (kt - 2) * NW, rl = (lane & 31) - (row0 & 31);
+            if (wm == row0 / (BM / 2) && rl >= 0 && rl < NW) {
+              const uint8_t* src = smem + C_LDS + ((kt & 1) * NW + rl) * C_PITCH +
+                                   (wn * (BN / WN) + (lane >> 5) * 4) * 4;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-              if (kt == i + 1) {
+              for (int i = 0; i < TM; ++i)
+                if (i == (row0 % (BM / 2)) / 32) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                  for (int j = 0; j < TN; ++j)
 #pragma unroll
-                  for (int g = 0; g < 4; ++g) {
-                    acc[i][j][4 * g] += cbuf[j][g].x; acc[i][j][4 * g + 1] += cbuf[j][g].y;
-                    acc[i][j][4 * g + 2] += cbuf[j][g].z; acc[i][j][4 * g + 3] += cbuf[j][g].w;
-                  }
-              }
-            if (kt < TM) load_c_row(kt);
+                    for (int g = 0; g < 4; ++g) {
+                      const float4 c = *(const float4*)(src + (j * 32 + g * 8) * 4);
+                      acc[i][j][4 * g] += c.x; acc[i][j][4 * g + 1] += c.y;
+                      acc[i][j][4 * g + 2] += c.z; acc[i][j][4 * g + 3] += c.w;
+                    }
+                }
+            }
           }
         }
 #pragma unroll
@@ -257,6 +266,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cur][j], fx[cur][i], acc[i][j],
                                                               0, 0, 0);
       }
+    }
+    if constexpr (EPI == JPP_EPI_ACC_F32) {
+      if (stream_c && kt < NBT)
+        dma_load16(uniform_ptr((const bf16_t*)p.c), c_off0 + (uint32_t)(kt * NW * p.ldc * 4),
+                   lds0 + C_LDS + ((kt & 1) * NW + wave) * C_PITCH);
     }
   }
   dma_wait_all();   // the refetches of the last two K-steps must not outlive the block's LDS
@@ -422,8 +436,9 @@ template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4>
 int launch(hipStream_t stream, GemmParams& p) {
   // two operand stages; the bf16 epilogues stage half a tile in fp32 with padded rows
   constexpr int SMEM_LOOP = 2 * (BM + BN) * 128, SMEM_EPI = (BM / 2) * (BN * 4 + 16);
-  constexpr int SMEM = (EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_F32 || SMEM_LOOP > SMEM_EPI)
-                           ? SMEM_LOOP : SMEM_EPI;
+  // + two buffers of NW rows of the fp32 tile (padded) for C += A B
+  constexpr int SMEM = EPI == JPP_EPI_ACC_F32 ? SMEM_LOOP + 2 * NW * (1024 + 16)
+                       : (EPI == JPP_EPI_F32 || SMEM_LOOP > SMEM_EPI) ? SMEM_LOOP : SMEM_EPI;
   // algorithmic extent: grouped launches count the non-padding rows when the caller gave them
   const double cb = EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_DSWIGLU ? 8
                     : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;
@@ -520,6 +535,9 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     JPP_REQUIRE(a->aux && a->ldaux >= 2 * a->n && a->ldaux % 4 == 0 && a->ldc >= 2 * a->n &&
                     !a->bias && !a->resid && a->group_mode == JPP_GROUP_NONE,
                 "gemm: dSwiGLU epilogue needs aux and C of width 2N and takes no bias / residual / groups");
+  if (a->epilogue == JPP_EPI_ACC_F32)
+    JPP_REQUIRE((double)a->m * a->ldc * 4 < 4294967296.0,
+                "gemm: an accumulated output must span less than 4 GiB (32-bit offsets)");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
   if (a->group_mode != JPP_GROUP_NONE) tile = 4;  // 256-row segments
