@@ -118,7 +118,7 @@ def dominant_gemm_class(wl) -> str:
     # weight-gradient GEMM with the fp32 accumulate epilogue: a third of the
     # FLOPs and the longest kernel per call
     big = wl.layer.hidden >= 4096
-    return "gemm_tn_accf32_256x256w8" if big else "gemm_tn_accf32_128x128"
+    return "gemm_tn_accf32_256x256w8" if big else "gemm_tn_accf32_128x128w8"
 
 
 def cpu_baseline(wl, budget_layers: int = 1):

@@ -466,10 +466,15 @@ int launch(hipStream_t stream, GemmParams& p) {
 template <bool TA, bool TB, int EPI>
 int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
   switch (tile) {
-    case 1: return launch<128, 128, TA, TB, EPI>(stream, p);
     case 2: return launch<256, 128, TA, TB, EPI>(stream, p);
     case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
-    default: return launch<128, 128, TA, TB, EPI>(stream, p);
+    default:
+      // 128x128: 8 waves (64x32 each, two workgroups per CU = 4 waves per SIMD) except for
+      // the SwiGLU epilogues, which need a wave to span 64 columns
+      if constexpr (EPI != JPP_EPI_SWIGLU && EPI != JPP_EPI_DSWIGLU)
+        return launch<128, 128, TA, TB, EPI, 8>(stream, p);
+      else
+        return launch<128, 128, TA, TB, EPI>(stream, p);
   }
 }
 
