@@ -82,7 +82,7 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = (pid % width) / gsize;
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI, int NW>
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   using TileA = DmaTile<BM, TA, NW>;
   using TileB = DmaTile<BN, TB, NW>;
@@ -128,16 +128,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   f32x16 acc[TM][TN];
   // C += A B (EPI_ACC_F32): the epilogue only stores; the fp32 tile in memory is folded into
   // the accumulators during the first K-steps.  It travels HBM -> LDS like the operands, NW
-  // whole rows (BN * 4 bytes each, one per wave) at a time, into one of two buffers behind
+  // whole rows (BN * 4 bytes each, one per wave) at a time, into one of NS+1 buffers behind
   // the operand stages: batch b is requested at the end of K-step b, after that K-step's
-  // operand copies, and read out of LDS at the wait point of K-step b+2.  The wait of
-  // K-step b+1 leaves the youngest request in flight (vmcnt counts in order), so a batch has
-  // two K-steps to arrive and no K-step waits for HBM on its account; reading whole rows
+  // operand copies, and read out of LDS at the wait point of K-step b+NS.  The waits in
+  // between leave the youngest requests in flight (vmcnt counts in order), so a batch has
+  // NS K-steps to arrive and no K-step waits for HBM on its account; reading whole rows
   // keeps HBM on long bursts where a lane-per-row layout would touch 32 rows at once.  K
   // loops too short for that read the tile into the accumulators up front.
   static_assert(BN * 4 <= 1024, "a row of the fp32 tile is one 64-lane copy");
-  constexpr int NBT = BM / NW, C_LDS = 2 * (BM + BN) * 128, C_PITCH = 1024 + 16;  // a copy is 1 KB
-  const bool stream_c = EPI == JPP_EPI_ACC_F32 && kt_n >= NBT + 2;
+  constexpr int NBT = BM / NW, C_LDS = NS * (BM + BN) * 128, C_PITCH = 1024 + 16;  // a copy is 1 KB
+  const bool stream_c = EPI == JPP_EPI_ACC_F32 && kt_n >= NBT + NS;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -171,19 +171,25 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   constexpr int IA = TileA::INSTS, IB = TileB::INSTS;
   const int row_w = wn * (BN / WN), row_x = wm * (BM / 2);
 
-  // Software pipeline over K-steps of 64 with two LDS stages:
-  //   * the HBM -> LDS copy of K-step t+2 is issued inside K-step t, right after the
-  //     barrier that retires stage t&1's readers, so it has a whole K-step to land;
+  // Software pipeline over K-steps of 64 with NS LDS stages:
+  //   * the HBM -> LDS copy of K-step t+NS is issued inside K-step t, right after the
+  //     barrier that retires stage t % NS's readers, so it has NS-1 K-steps to land;
   //   * that barrier sits in front of the last of the four MFMA blocks of a K-step and the
   //     first fragments of K-step t+1 are read from LDS behind it, under those MFMAs.
+  // Waits count requests from the youngest (vmcnt is in order): at the wait point of K-step
+  // t the copies of K-steps t+2 .. t+NS-1 and the accumulator rows requested during the last
+  // NS-1 K-steps may stay in flight.
+  constexpr int OPB = IA + IB;  // operand copies per wave and K-step
   bf16x8 fw[2][TN], fx[2][TM];
   if (kt_n > 0) {
-    TileA::template issue<0, IA>(uniform_ptr(a_src), offa, lds0, wave);
-    TileB::template issue<0, IB>(uniform_ptr(b_src), offb, lds0 + A_BYTES, wave);
-    const int k1 = min(1, kt_n - 1);
-    TileA::template issue<0, IA>(uniform_ptr(a_src + k1 * a_step), offa, lds0 + STAGE, wave);
-    TileB::template issue<0, IB>(uniform_ptr(b_src + k1 * b_step), offb, lds0 + STAGE + A_BYTES, wave);
-    dma_wait<IA + IB>();   // stage 0 has landed; stage 1 may still be in flight
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int k = min(s, kt_n - 1);
+      TileA::template issue<0, IA>(uniform_ptr(a_src + k * a_step), offa, lds0 + s * STAGE, wave);
+      TileB::template issue<0, IB>(uniform_ptr(b_src + k * b_step), offb, lds0 + s * STAGE + A_BYTES,
+                                   wave);
+    }
+    dma_wait<(NS - 1) * OPB>();  // stage 0 has landed; the others may still be in flight
   }
   if constexpr (EPI == JPP_EPI_ACC_F32) {
     // the compiler waits for up-front reads of C here, not at their first use inside the K
@@ -199,12 +205,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 #pragma unroll
   for (int i = 0; i < TM; ++i) fx[0][i] = TileA::frag(smem, row_x + i * 32, 0, lane);
 
+  int st = 0;   // stage of K-step kt: kt % NS
+  int cbi = 0;  // accumulator-row buffer of K-step kt: kt % (NS + 1)
   for (int kt = 0; kt < kt_n; ++kt) {
-    const uint8_t* sa = smem + (kt & 1) * STAGE;
+    const int nst = st + 1 == NS ? 0 : st + 1;
+    const uint8_t* sa = smem + st * STAGE;
     const uint8_t* sb = sa + A_BYTES;
-    const uint8_t* na = smem + ((kt + 1) & 1) * STAGE;
+    const uint8_t* na = smem + nst * STAGE;
     // past the end the last K-step is fetched again, unused
-    const int kn = min(kt + 2, kt_n - 1);
+    const int kn = min(kt + NS, kt_n - 1);
     const bf16_t* ga = uniform_ptr(a_src + (long)kn * a_step);
     const bf16_t* gb = uniform_ptr(b_src + (long)kn * b_step);
 #pragma unroll
@@ -217,20 +226,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
         for (int i = 0; i < TM; ++i) fx[nxt][i] = TileA::frag(sa, row_x + i * 32, ks + 1, lane);
       } else {
         // every fragment of this stage is in registers: once all waves are here (and the
-        // other stage, requested one K-step ago, has landed) this stage can be refilled
-        if (EPI == JPP_EPI_ACC_F32 && stream_c && kt >= 1 && kt <= NBT)
-          dma_wait<1>();  // all but the accumulator row requested at the end of K-step kt-1
-        else
-          dma_wait_all();
+        // next stage has landed) this stage can be refilled
+        {
+          // accumulator rows requested during K-steps kt+1-NS .. kt-1 that may stay in flight
+          int cin = 0;
+          if (EPI == JPP_EPI_ACC_F32 && stream_c)
+            cin = max(0, min(kt - 1, NBT - 1) - max(0, kt + 1 - NS) + 1);
+          if (cin <= 0) dma_wait<(NS - 2) * OPB>();
+          else if (cin == 1) dma_wait<(NS - 2) * OPB + 1>();
+          else if (cin == 2) dma_wait<(NS - 2) * OPB + 2>();
+          else dma_wait<(NS - 2) * OPB + 3>();
+          static_assert(NS <= 4, "the wait above distinguishes up to three rows in flight");
+        }
         lds_wait_all();
         __syncthreads();
         if constexpr (EPI == JPP_EPI_ACC_F32) {
-          if (stream_c && kt >= 2 && kt <= NBT + 1) {
-            // batch kt-2 (tile rows NW (kt-2) .. + NW-1) is in LDS: the lanes that hold those
-            // rows in their accumulators add them in
-            const int row0 = (kt - 2) * NW, rl = (lane & 31) - (row0 & 31);
+          if (stream_c && kt >= NS && kt < NBT + NS) {
+            // batch kt-NS (tile rows NW (kt-NS) .. + NW-1) is in LDS: the lanes that hold
+            // those rows add them in.  Buffers are used round robin over NS+1, so the one
+            // read here is written again only behind the next K-step's barrier.
+            const int row0 = (kt - NS) * NW, rl = (lane & 31) - (row0 & 31);
+            const int fold_buf = cbi + 1 == NS + 1 ? 0 : cbi + 1;  // (kt - NS) % (NS + 1)
             if (wm == row0 / (BM / 2) && rl >= 0 && rl < NW) {
-              const uint8_t* src = smem + C_LDS + ((kt & 1) * NW + rl) * C_PITCH +
+              const uint8_t* src = smem + C_LDS + (fold_buf * NW + rl) * C_PITCH +
                                    (wn * (BN / WN) + (lane >> 5) * 4) * 4;
 #pragma unroll
               for (int i = 0; i < TM; ++i)
@@ -258,8 +276,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         if (ks == 3) {
-          TileA::template issue_part<IA / TM>(i, ga, offa, lds0 + (kt & 1) * STAGE, wave);
-          TileB::template issue_part<IB / TM>(i, gb, offb, lds0 + (kt & 1) * STAGE + A_BYTES, wave);
+          TileA::template issue_part<IA / TM>(i, ga, offa, lds0 + st * STAGE, wave);
+          TileB::template issue_part<IB / TM>(i, gb, offb, lds0 + st * STAGE + A_BYTES, wave);
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
@@ -270,8 +288,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     if constexpr (EPI == JPP_EPI_ACC_F32) {
       if (stream_c && kt < NBT)
         dma_load16(uniform_ptr((const bf16_t*)p.c), c_off0 + (uint32_t)(kt * NW * p.ldc * 4),
-                   lds0 + C_LDS + ((kt & 1) * NW + wave) * C_PITCH);
+                   lds0 + C_LDS + (cbi * NW + wave) * C_PITCH);
     }
+    st = nst;
+    cbi = cbi + 1 == NS + 1 ? 0 : cbi + 1;
   }
   dma_wait_all();   // the refetches of the last two K-steps must not outlive the block's LDS
 
@@ -419,7 +439,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   }
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI, int NW>
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS>
 const char* class_name() {
   static char name[64] = "";
   if (!name[0]) {
@@ -427,17 +447,18 @@ const char* class_name() {
     const char* epi = EPI == JPP_EPI_BF16 ? "bf16" : EPI == JPP_EPI_GELU ? "gelu"
                     : EPI == JPP_EPI_DGELU ? "dgelu" : EPI == JPP_EPI_ACC_F32 ? "accf32"
                     : EPI == JPP_EPI_SWIGLU ? "swiglu" : EPI == JPP_EPI_DSWIGLU ? "dswiglu" : "f32";
-    snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d%s", lay, epi, BM, BN, NW == 8 ? "w8" : "");
+    snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d%s%s", lay, epi, BM, BN, NW == 8 ? "w8" : "",
+             NS == 2 ? "" : NS == 3 ? "s3" : "s4");
   }
   return name;
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4>
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4, int NS = 2>
 int launch(hipStream_t stream, GemmParams& p) {
   // two operand stages; the bf16 epilogues stage half a tile in fp32 with padded rows
-  constexpr int SMEM_LOOP = 2 * (BM + BN) * 128, SMEM_EPI = (BM / 2) * (BN * 4 + 16);
-  // + two buffers of NW rows of the fp32 tile (padded) for C += A B
-  constexpr int SMEM = EPI == JPP_EPI_ACC_F32 ? SMEM_LOOP + 2 * NW * (1024 + 16)
+  constexpr int SMEM_LOOP = NS * (BM + BN) * 128, SMEM_EPI = (BM / 2) * (BN * 4 + 16);
+  // + NS+1 buffers of NW rows of the fp32 tile (padded) for C += A B
+  constexpr int SMEM = EPI == JPP_EPI_ACC_F32 ? SMEM_LOOP + (NS + 1) * NW * (1024 + 16)
                        : (EPI == JPP_EPI_F32 || SMEM_LOOP > SMEM_EPI) ? SMEM_LOOP : SMEM_EPI;
   // algorithmic extent: grouped launches count the non-padding rows when the caller gave them
   const double cb = EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_DSWIGLU ? 8
@@ -446,9 +467,10 @@ int launch(hipStream_t stream, GemmParams& p) {
   if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
   if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
   const double b_bytes = 2.0 * p.n * ak * (p.group_mode == JPP_GROUP_M ? p.n_seg : 1);
-  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW>(), 2.0 * am * p.n * ak,
+  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW, NS>(), 2.0 * am * p.n * ak,
                    2.0 * am * ak + b_bytes + copies * am * p.n * cb);
-  auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW>;
+  auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW, NS>;
+  static_assert(SMEM <= 160 * 1024, "LDS of one CU");
   static bool configured = false;  // per instantiation; attribute is sticky
   if (!configured) {
     JPP_CHECK_HIP(hipFuncSetAttribute((const void*)kern,
@@ -469,12 +491,19 @@ int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
     case 2: return launch<256, 128, TA, TB, EPI>(stream, p);
     case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
     default:
-      // 128x128: 8 waves (64x32 each, two workgroups per CU = 4 waves per SIMD) except for
-      // the SwiGLU epilogues, which need a wave to span 64 columns
-      if constexpr (EPI != JPP_EPI_SWIGLU && EPI != JPP_EPI_DSWIGLU)
-        return launch<128, 128, TA, TB, EPI, 8>(stream, p);
-      else
+      // 128x128: 8 waves (64x32 each) except for the SwiGLU epilogues, which need a wave to
+      // span 64 columns.  With more tiles than two per CU, two stages and two workgroups per
+      // CU; with fewer (and a K loop long enough to pay for the longer prologue) the one
+      // workgroup a CU gets prefetches deeper instead (4 stages, 3 where the accumulator
+      // rows need room too).
+      if constexpr (EPI == JPP_EPI_SWIGLU || EPI == JPP_EPI_DSWIGLU) {
         return launch<128, 128, TA, TB, EPI>(stream, p);
+      } else {
+        const long tiles = (long)(p.m / 128) * (p.n / 128) *
+                           (p.group_mode == JPP_GROUP_K ? p.n_seg : 1);
+        if (tiles > 2 * 256 || p.k < 2048) return launch<128, 128, TA, TB, EPI, 8>(stream, p);
+        return launch<128, 128, TA, TB, EPI, 8, EPI == JPP_EPI_ACC_F32 ? 3 : 4>(stream, p);
+      }
   }
 }
 
