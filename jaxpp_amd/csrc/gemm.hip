@@ -563,12 +563,12 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     JPP_REQUIRE(a->aux && a->ldaux >= a->n && a->ldaux % 4 == 0, "gemm: dGELU epilogue needs aux");
   if (a->epilogue == JPP_EPI_SWIGLU)
     JPP_REQUIRE(a->c2 && a->ldc2 >= a->n / 2 && a->ldc2 % 4 == 0 && !a->bias && !a->resid &&
-                    a->group_mode == JPP_GROUP_NONE,
-                "gemm: SwiGLU epilogue needs c2 [M, N/2] and takes no bias / residual / groups");
+                    a->group_mode != JPP_GROUP_K,
+                "gemm: SwiGLU epilogue needs c2 [M, N/2] and takes no bias / residual");
   if (a->epilogue == JPP_EPI_DSWIGLU)
     JPP_REQUIRE(a->aux && a->ldaux >= 2 * a->n && a->ldaux % 4 == 0 && a->ldc >= 2 * a->n &&
-                    !a->bias && !a->resid && a->group_mode == JPP_GROUP_NONE,
-                "gemm: dSwiGLU epilogue needs aux and C of width 2N and takes no bias / residual / groups");
+                    !a->bias && !a->resid && a->group_mode != JPP_GROUP_K,
+                "gemm: dSwiGLU epilogue needs aux and C of width 2N and takes no bias / residual");
   if (a->epilogue == JPP_EPI_ACC_F32)
     JPP_REQUIRE((double)a->m * a->ldc * 4 < 4294967296.0,
                 "gemm: an accumulated output must span less than 4 GiB (32-bit offsets)");

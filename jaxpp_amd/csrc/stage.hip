@@ -119,13 +119,15 @@ enum MixtralP { X_rms1, X_Wqkv, X_Wo, X_rms2, X_Wr, X_Wgu, X_Wd };
 
 int ggemm(hipStream_t st, int mode, const int* seg, int n_seg, const void* a, int64_t lda, int ta,
           const void* b, int64_t ldb, int tb, int64_t stride_b, void* c, int64_t ldc,
-          int64_t stride_c, int64_t m, int64_t n, int64_t k, int epi, int64_t rows) {
+          int64_t stride_c, int64_t m, int64_t n, int64_t k, int epi, int64_t rows,
+          const void* aux = nullptr, int64_t ldaux = 0, void* c2 = nullptr, int64_t ldc2 = 0) {
   jpp_gemm_args g;
   memset(&g, 0, sizeof(g));
   g.a = a; g.b = b; g.c = c; g.m = m; g.n = n; g.k = k;
   g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.trans_a = ta; g.trans_b = tb; g.epilogue = epi;
   g.seg = seg; g.n_seg = n_seg; g.group_mode = mode; g.stride_b = stride_b; g.stride_c = stride_c;
   g.group_rows = rows;
+  g.aux = aux; g.ldaux = ldaux; g.c2 = c2; g.ldc2 = ldc2;
   return jpp_gemm_bf16(st, &g);
 }
 
@@ -251,9 +253,11 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
     const int* seg = ma.seg;
     RC(jpp_moe_route(st, &ma));
     RC(jpp_moe_gather(st, &ma, at(L.n2), at(L.xp)));
+    // gate and up columns of each expert's Wgu are interleaved in blocks of 32, as in the
+    // dense layer: SwiGLU runs in the epilogue
     RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.xp), h, 0, s->P(chunk, li, X_Wgu), 2 * f, 1, h * 2 * f,
-             at(L.gu), 2 * f, 0, s->cap, 2 * f, h, JPP_EPI_BF16, s->T * s->d.top_k));
-    RC(jpp_swiglu_fwd(st, at(L.gu), at(L.s), s->cap, f, 0));
+             at(L.gu), 2 * f, 0, s->cap, 2 * f, h, JPP_EPI_SWIGLU, s->T * s->d.top_k, nullptr, 0,
+             at(L.s), f));
     RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.s), f, 0, s->P(chunk, li, X_Wd), h, 1, f * h, at(L.eo), h,
              0, s->cap, h, f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_fwd(st, &ma, at(L.eo), at(L.h1), y));
@@ -308,7 +312,6 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     return JPP_OK;
   }
   // llama
-  void* ds = s->S<>(s->s_t1);
   void* dn = s->S<>(s->s_t2);   // dn2, later dn1
   void* dctx = s->S<>(s->s_t3);
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
@@ -317,9 +320,8 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     const int E = s->d.n_experts;
     void* dxp = s->S<>(s->s_t4);
     RC(jpp_moe_bwd_prepare(st, &ma, dy, at(L.eo), (float*)wt(W.dlogits), wt(W.deo)));
-    RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.deo), h, 0, s->P(chunk, li, X_Wd), h, 0, f * h, ds, f,
-             0, s->cap, f, h, JPP_EPI_BF16, s->T * s->d.top_k));
-    RC(jpp_swiglu_bwd(st, at(L.gu), ds, wt(W.dgu), s->cap, f, 0));
+    RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.deo), h, 0, s->P(chunk, li, X_Wd), h, 0, f * h,
+             wt(W.dgu), 2 * f, 0, s->cap, f, h, JPP_EPI_DSWIGLU, s->T * s->d.top_k, at(L.gu), 2 * f));
     RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.dgu), 2 * f, 0, s->P(chunk, li, X_Wgu), 2 * f, 0,
              h * 2 * f, dxp, h, 0, s->cap, h, 2 * f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_bwd(st, &ma, dxp, (const float*)wt(W.dlogits), dn));
@@ -524,7 +526,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   s->s_dx[0] = sc.take(T * h * e);
   s->s_dx[1] = sc.take(T * h * e);
   const size_t rows_t = d->family == JPP_FAMILY_MIXTRAL ? (size_t)s->cap : (size_t)T;
-  s->s_t1 = sc.take(rows_t * (d->family == JPP_FAMILY_BERT ? h : f) * e);
+  s->s_t1 = sc.take(d->family == JPP_FAMILY_BERT ? rows_t * h * e : 256);  // BERT: dx1
   s->s_t4 = sc.take(d->family == JPP_FAMILY_MIXTRAL ? rows_t * h * e : 256);
   s->s_moework = sc.take(d->family == JPP_FAMILY_MIXTRAL
                              ? (size_t)2 * ((T + 255) / 256) * d->n_experts * 4 + 256 : 256);

@@ -399,10 +399,10 @@ class StageExecutor:
 
     def _device_columns(self, name: str, cols: int):
         """Column order of a parameter in device memory, or None when it is the host's.  The
-        Llama layer keeps ``Wgu = [gate | up]`` with the two projections interleaved in blocks
+        Llama and Mixtral layers keep ``Wgu = [gate | up]`` with the two projections interleaved in blocks
         of 32 columns (device column 64q+w = gate feature 32q+w for w < 32, up feature 32q+w-32
         otherwise), which lets the GEMM epilogue apply SwiGLU (JPP_EPI_SWIGLU)."""
-        if self.spec.family != "llama" or name != "Wgu":
+        if self.spec.family not in ("llama", "mixtral") or name != "Wgu":
             return None
         f = cols // 2
         c = np.arange(cols)
