@@ -187,9 +187,9 @@ struct TileLoader {
 //               is the swizzled slab read by slab_frag().
 //   MC = true   memory [64][ROWS..], contraction index is the slow one.  LDS
 //               image keeps that orientation, chunk c of row k stored at
-//               c ^ ((k & 3) << 2); fragments come out through the LDS
-//               transpose read (ds_read_b64_tr_b16), which hands lane i of a
-//               16-lane group the column i of a 4 x 16 block.
+//               c ^ mc_swz(k); fragments come out through the LDS transpose
+//               read (ds_read_b64_tr_b16), which hands lane i of a 16-lane
+//               group the column i of a 4 x 16 block.
 // ---------------------------------------------------------------------------
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -228,6 +228,12 @@ __device__ __forceinline__ void dma_wait() {
 // waits for this wave's LDS reads, so that what they read may be overwritten
 __device__ __forceinline__ void lds_wait_all() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
+// Chunk permutation of row k of an MC tile.  A transpose read has lanes 0-15 on rows
+// k .. k+3 and lanes 16-31 on rows k+8 .. k+11 (8 rows are a multiple of the bank span
+// apart): bits 0-1 of k move a chunk by 64 bytes, bit 3 by 32, so those 32 lanes touch
+// every bank once.
+__device__ __forceinline__ int mc_swz(int k) { return ((k & 3) << 2) ^ (((k >> 3) & 1) << 1); }
+
 template <int ROWS, bool MC, int NW = 4>
 struct DmaTile {
   static constexpr int BYTES = ROWS * 128;
@@ -247,7 +253,7 @@ struct DmaTile {
       } else {
         constexpr int CPR = ROWS / 8, RPI = 64 / CPR;
         const int k = inst * RPI + lane / CPR;
-        off[i] = (uint32_t)(((long)k * ld + ((((lane % CPR) ^ ((k & 3) << 2))) << 3)) * 2);
+        off[i] = (uint32_t)(((long)k * ld + (((lane % CPR) ^ mc_swz(k)) << 3)) * 2);
       }
     }
   }
@@ -270,16 +276,18 @@ struct DmaTile {
       dma_load16(src, off[part * COUNT + i], tile + (wave * INSTS + part * COUNT + i) * 1024);
   }
 
-  // MFMA operand fragment: rows row0 .. row0+31 of the operand, K-step ks
-  static __device__ __forceinline__ bf16x8 frag(const uint8_t* tile, int row0, int ks, int lane) {
+  // Operand fragment for v_mfma_f32_16x16x32_bf16: rows row0 .. row0+15 of the operand and
+  // the contraction elements 32 k32 .. 32 k32 + 31 of the tile; lane l supplies row l & 15
+  // and the 8 elements of chunk l >> 4.
+  static __device__ __forceinline__ bf16x8 frag16(const uint8_t* tile, int row0, int k32, int lane) {
+    const int g = lane >> 4, s = lane & 15;
     if constexpr (!MC) {
-      return slab_frag(tile, row0, ks, lane);
+      return *(const bf16x8*)(tile + slab_off(row0 + s, k32 * 4 + g));
     } else {
-      const int g = lane >> 4, s = lane & 15;
-      const int n = row0 + ((g & 1) << 4) + ((s & 3) << 2);
-      const int kq = s >> 2;  // == k & 3
-      const int k = ks * 16 + ((g >> 1) << 3) + kq;
-      const uint8_t* p = tile + k * (ROWS * 2) + ((((n >> 3) ^ (kq << 2))) << 4) + ((n & 7) << 1);
+      // two transpose reads of 4 contraction rows x 16 operand rows per 16-lane group
+      const int n = row0 + ((s & 3) << 2);
+      const int k = k32 * 32 + (g << 3) + (s >> 2);
+      const uint8_t* p = tile + k * (ROWS * 2) + (((n >> 3) ^ mc_swz(k)) << 4) + ((n & 7) << 1);
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (__attribute__((address_space(3))) s16x4*)JPP_LDS_PTR(p));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(

@@ -88,7 +88,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   using TileB = DmaTile<BN, TB, NW>;
   constexpr int A_BYTES = TileA::BYTES, STAGE = TileA::BYTES + TileB::BYTES;
   constexpr int WN = NW / 2;                        // waves: 2 along m, NW/2 along n
-  constexpr int TM = BM / 64, TN = BN / (32 * WN);  // 32x32 MFMA tiles per wave
+  // 16x16 MFMA tiles per wave.  A K-step runs them in 2 HS blocks of TMH x TN (32 contraction
+  // elements each); large wave tiles take the rows in two halves so that the fragments of
+  // two blocks fit in registers beside the accumulators
+  constexpr int TM = BM / 32, TN = BN / (16 * WN), HS = TM * TN >= 32 ? 2 : 1, TMH = TM / HS;
+  constexpr int NB = 2 * HS;
   extern __shared__ __align__(1024) uint8_t smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -122,10 +126,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   const long a_step = TA ? 64 * p.lda : 64;
   const long b_step = TB ? 64 * p.ldb : 64;
 
-  // lane holds m = m_lane + 32 i, and for g = 0..3 the four columns n_lane + 32 j + 8 g + {0..3}
-  const long m_lane = m0 + wm * (BM / 2) + (lane & 31);
-  const long n_lane = n0 + wn * (BN / WN) + (lane >> 5) * 4;
-  f32x16 acc[TM][TN];
+  // lane holds, of tile (i, j), m = m_lane + 16 i and the four columns n_lane + 16 j + {0..3}
+  const long m_lane = m0 + wm * (BM / 2) + (lane & 15);
+  const long n_lane = n0 + wn * (BN / WN) + (lane >> 4) * 4;
+  f32x4 acc[TM][TN];
   // C += A B (EPI_ACC_F32): the epilogue only stores; the fp32 tile in memory is folded into
   // the accumulators during the first K-steps.  It travels HBM -> LDS like the operands, NW
   // whole rows (BN * 4 bytes each, one per wave) at a time, into one of NS+1 buffers behind
@@ -141,22 +145,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   if constexpr (EPI == JPP_EPI_ACC_F32) {
     if (!stream_c) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const float4 c = *(const float4*)((const float*)p.c + (m_lane + i * 32) * p.ldc +
-                                              n_lane + j * 32 + g * 8);
-            acc[i][j][4 * g] = c.x; acc[i][j][4 * g + 1] = c.y;
-            acc[i][j][4 * g + 2] = c.z; acc[i][j][4 * g + 3] = c.w;
-          }
+          acc[i][j] = *(const f32x4*)((const float*)p.c + (m_lane + i * 16) * p.ldc + n_lane +
+                                      j * 16);
     }
   }
   // byte offset, from the start of C, of this lane's 16 bytes of tile row `wave`
@@ -174,13 +171,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   // Software pipeline over K-steps of 64 with NS LDS stages:
   //   * the HBM -> LDS copy of K-step t+NS is issued inside K-step t, right after the
   //     barrier that retires stage t % NS's readers, so it has NS-1 K-steps to land;
-  //   * that barrier sits in front of the last of the four MFMA blocks of a K-step and the
-  //     first fragments of K-step t+1 are read from LDS behind it, under those MFMAs.
+  //   * that barrier sits in front of the last MFMA block of a K-step and the first
+  //     fragments of K-step t+1 are read from LDS behind it, under those MFMAs.
+  // Block q of a K-step multiplies contraction elements 32 (q / HS) .. + 31 of the stage: the
+  // wave's TN fragments of B (read once per HS blocks) with part q % HS of its TM fragments
+  // of A, each fragment read while the block before it computes.
   // Waits count requests from the youngest (vmcnt is in order): at the wait point of K-step
   // t the copies of K-steps t+2 .. t+NS-1 and the accumulator rows requested during the last
   // NS-1 K-steps may stay in flight.
   constexpr int OPB = IA + IB;  // operand copies per wave and K-step
-  bf16x8 fw[2][TN], fx[2][TM];
+  bf16x8 fw[2][TN], fx[2][TMH];
   if (kt_n > 0) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -201,9 +201,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   }
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag(smem + A_BYTES, row_w + j * 32, 0, lane);
+  for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag16(smem + A_BYTES, row_w + j * 16, 0, lane);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) fx[0][i] = TileA::frag(smem, row_x + i * 32, 0, lane);
+  for (int i = 0; i < TMH; ++i) fx[0][i] = TileA::frag16(smem, row_x + i * 16, 0, lane);
 
   int st = 0;   // stage of K-step kt: kt % NS
   int cbi = 0;  // accumulator-row buffer of K-step kt: kt % (NS + 1)
@@ -217,13 +217,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     const bf16_t* ga = uniform_ptr(a_src + (long)kn * a_step);
     const bf16_t* gb = uniform_ptr(b_src + (long)kn * b_step);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks < 3) {
+    for (int ks = 0; ks < NB; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1, curw = ks / HS, part = ks % HS;
+      if (ks < NB - 1) {
+        if ((ks + 1) % HS == 0) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fw[nxt][j] = TileB::frag(sb, row_w + j * 32, ks + 1, lane);
+          for (int j = 0; j < TN; ++j) fw[1][j] = TileB::frag16(sb, row_w + j * 16, 1, lane);
+        }
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fx[nxt][i] = TileA::frag(sa, row_x + i * 32, ks + 1, lane);
+        for (int i = 0; i < TMH; ++i)
+          fx[nxt][i] = TileA::frag16(sa, row_x + ((ks + 1) % HS * TMH + i) * 16, (ks + 1) / HS, lane);
       } else {
         // every fragment of this stage is in registers: once all waves are here (and the
         // next stage has landed) this stage can be refilled
@@ -245,44 +248,41 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
             // batch kt-NS (tile rows NW (kt-NS) .. + NW-1) is in LDS: the lanes that hold
             // those rows add them in.  Buffers are used round robin over NS+1, so the one
             // read here is written again only behind the next K-step's barrier.
-            const int row0 = (kt - NS) * NW, rl = (lane & 31) - (row0 & 31);
+            const int row0 = (kt - NS) * NW, rl = (lane & 15) - (row0 & 15);
             const int fold_buf = cbi + 1 == NS + 1 ? 0 : cbi + 1;  // (kt - NS) % (NS + 1)
             if (wm == row0 / (BM / 2) && rl >= 0 && rl < NW) {
               const uint8_t* src = smem + C_LDS + (fold_buf * NW + rl) * C_PITCH +
-                                   (wn * (BN / WN) + (lane >> 5) * 4) * 4;
+                                   (wn * (BN / WN) + (lane >> 4) * 4) * 4;
 #pragma unroll
               for (int i = 0; i < TM; ++i)
-                if (i == (row0 % (BM / 2)) / 32) {
+                if (i == (row0 % (BM / 2)) / 16) {
 #pragma unroll
-                  for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                      const float4 c = *(const float4*)(src + (j * 32 + g * 8) * 4);
-                      acc[i][j][4 * g] += c.x; acc[i][j][4 * g + 1] += c.y;
-                      acc[i][j][4 * g + 2] += c.z; acc[i][j][4 * g + 3] += c.w;
-                    }
+                  for (int j = 0; j < TN; ++j) acc[i][j] += *(const f32x4*)(src + j * 64);
                 }
             }
           }
         }
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fw[nxt][j] = TileB::frag(na + A_BYTES, row_w + j * 32, 0, lane);
+        for (int j = 0; j < TN; ++j) fw[0][j] = TileB::frag16(na + A_BYTES, row_w + j * 16, 0, lane);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fx[nxt][i] = TileA::frag(na, row_x + i * 32, 0, lane);
+        for (int i = 0; i < TMH; ++i) fx[0][i] = TileA::frag16(na, row_x + i * 16, 0, lane);
       }
       // the refill of the retired stage is spread over this block's MFMAs: a wave that
       // issues its loads back to back waits on the memory pipeline with its MFMAs behind it
-      static_assert(IA % TM == 0 && IB % TM == 0, "loads per wave must split over the MFMA rows");
+      constexpr int PARTS = TMH < IA && TMH < IB ? TMH : (IA < IB ? IA : IB);
+      static_assert(IA % PARTS == 0 && IB % PARTS == 0 && TMH % PARTS == 0,
+                    "loads per wave must split over the MFMA rows");
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if (ks == 3) {
-          TileA::template issue_part<IA / TM>(i, ga, offa, lds0 + st * STAGE, wave);
-          TileB::template issue_part<IB / TM>(i, gb, offb, lds0 + st * STAGE + A_BYTES, wave);
+      for (int i = 0; i < TMH; ++i) {
+        if (ks == NB - 1 && i % (TMH / PARTS) == 0) {
+          TileA::template issue_part<IA / PARTS>(i / (TMH / PARTS), ga, offa, lds0 + st * STAGE, wave);
+          TileB::template issue_part<IB / PARTS>(i / (TMH / PARTS), gb, offb,
+                                                 lds0 + st * STAGE + A_BYTES, wave);
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cur][j], fx[cur][i], acc[i][j],
-                                                              0, 0, 0);
+          acc[part * TMH + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              fw[curw][j], fx[cur][i], acc[part * TMH + i][j], 0, 0, 0);
       }
     }
     if constexpr (EPI == JPP_EPI_ACC_F32) {
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   if constexpr (EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_F32) {
     // fp32 outputs leave through LDS as well (see below), a quarter of the tile per pass:
     // 16-byte stores of contiguous rows instead of 32-byte pieces of 32 rows
-    constexpr int IPP = TM >= 2 ? TM / 2 : 1, RP = IPP * 32, PITCH = BN * 4 + 16, NT = NW * 64;
+    constexpr int IPP = TM / 2, RP = IPP * 16, PITCH = BN * 4 + 16, NT = NW * 64;
     constexpr int TPR = BN / 4, RPI = NT / TPR;
 #pragma unroll 1
     for (int pass = 0; pass < 2 * (TM / IPP); ++pass) {
@@ -310,16 +310,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
           if (i >= i0 && i < i0 + IPP) {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-#pragma unroll
-              for (int g = 0; g < 4; ++g)
-                *(float4*)(smem + ((i - i0) * 32 + (lane & 31)) * PITCH +
-                           (wn * (BN / WN) + j * 32 + g * 8 + (lane >> 5) * 4) * 4) =
-                    make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                                acc[i][j][4 * g + 3]);
+              *(f32x4*)(smem + ((i - i0) * 16 + (lane & 15)) * PITCH +
+                        (wn * (BN / WN) + j * 16 + (lane >> 4) * 4) * 4) = acc[i][j];
           }
       }
       __syncthreads();
-      const long mrow0 = m0 + half * (BM / 2) + i0 * 32;
+      const long mrow0 = m0 + half * (BM / 2) + i0 * 16;
       const int c4 = (tid % TPR) * 4;
       for (int r = tid / TPR; r < RP; r += RPI)
         *(float4*)((float*)p.c + (mrow0 + r) * p.ldc + n0 + c4) =
@@ -333,7 +329,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     // every global access of the epilogue (output, residual, pre-activation, gate/up) is a
     // 16-byte piece of a contiguous run, and the arithmetic runs in fp32 exactly as before.
     constexpr int HALF = BM / 2, PITCH = BN * 4 + 16, NT = NW * 64;
-    const int hh = lane >> 5;
     const bf16_t* bias = p.bias;
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
@@ -343,12 +338,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g)
-              *(float4*)(smem + (i * 32 + (lane & 31)) * PITCH +
-                         (wn * (BN / WN) + j * 32 + g * 8 + hh * 4) * 4) =
-                  make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                              acc[i][j][4 * g + 3]);
+            *(f32x4*)(smem + (i * 16 + (lane & 15)) * PITCH +
+                      (wn * (BN / WN) + j * 16 + (lane >> 4) * 4) * 4) = acc[i][j];
       }
       __syncthreads();
       const long mrow0 = m0 + half * HALF;
