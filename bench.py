@@ -174,6 +174,11 @@ def main():
                          "otherwise (+1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
                          "include the other stream's kernels)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
+    ap.add_argument("--after-loop", action="store_true",
+                    help="also time the step behind the loop - Adam over the stage's f32 "
+                         "gradient accumulators, rewriting the bf16 parameters - and report it "
+                         "as `after_loop` (not part of `value`; needs 12 more bytes per "
+                         "parameter on the device)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build executes one pipeline rank on one GPU; --gpus > 1 is not "
@@ -238,9 +243,33 @@ def main():
             "launches": pr.launches, "avg_launch_ms": avg_ms,
             "algorithmic_per_launch": (pr.bytes if hbm else pr.flops) / pr.launches,
         }
+    if args.after_loop:
+        rec["after_loop"] = after_loop(wb, wl, args.steps)
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(rec))
+
+
+def after_loop(wb, wl, steps: int) -> dict:
+    """Adam on the accumulators the timed steps left behind, `steps` times; HBM-bound: 34
+    algorithmic bytes per parameter (reads gradient, m, v, f32 weight; writes m, v, weight,
+    the bf16 parameter and the cleared gradient)."""
+    wb.ex.optimizer_init()
+    wb.ex.adam_step(1, grad_scale=1.0 / wl.n_mubatches)    # warm-up
+    rt.sync()
+    start, stop = rt.Event(), rt.Event()
+    with rt.probe("adam") as pr:
+        start.record()
+        for i in range(steps):
+            wb.ex.adam_step(2 + i, grad_scale=1.0 / wl.n_mubatches)
+        stop.record()
+        stop.sync()
+    ms = start.elapsed_ms(stop) / steps
+    ach = pr.bytes / (pr.total_ms * 1e-3)
+    return {"kernel": "adam", "ms": ms, "bound": "hbm", "achieved": ach / 1e9,
+            "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": ach / HBM_PEAK,
+            "launches": pr.launches, "avg_launch_ms": pr.total_ms / pr.launches,
+            "algorithmic_per_launch": pr.bytes / pr.launches}
 
 
 def self_desc(wl, wb) -> str:

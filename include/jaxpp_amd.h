@@ -200,6 +200,32 @@ int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t coun
 int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count);
 int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count);
 
+/* ---- after the loop: the optimizer on the accumulated gradients --------------
+ * The reference's train step applies `optimizer.update(grad, opt_state, pars)` and
+ * `optax.apply_updates` to what `treduce` returns (README.md:90-93; examples/basic.py:234
+ * builds the optimizer with `optax.adam`).  One fused pass over a flat tensor:
+ *   g  = grad_scale * grad
+ *   m  = beta1 m + (1 - beta1) g          v = beta2 v + (1 - beta2) g^2
+ *   w -= lr (m / (1 - beta1^step)) / (sqrt(v / (1 - beta2^step)) + eps)
+ * in f32, then param = bf16(w).  `master` holds the f32 weights; without it the bf16
+ * `param` is the only copy (read, updated in f32, rounded back).  With zero_grad the
+ * accumulator is cleared in the same pass, ready for the next loop. */
+typedef struct {
+  int64_t count;
+  float* grad;        /* f32 [count]: the loop's gradient accumulator */
+  float* master;      /* f32 [count] weights, updated in place; may be NULL */
+  void* param;        /* bf16 [count] weights, rewritten; may be NULL when master is given */
+  float* m;           /* f32 [count] first moment, updated in place */
+  float* v;           /* f32 [count] second moment, updated in place */
+  int64_t step;       /* 1 for the first update */
+  /* doubles, so that 1 - beta and the bias corrections are formed as the reference's
+   * Python floats form them before they meet f32 data */
+  double lr, beta1, beta2, eps;
+  double grad_scale;  /* e.g. 1 / n_mubatches when the loss is not already divided */
+  int zero_grad;
+} jpp_adam_args;
+int jpp_adam_step(void* stream, const jpp_adam_args* args);
+
 /* ---- top-2 mixture of experts: routing around the grouped GEMMs --------------
  * Tokens are assigned to rows of "permuted" buffers, grouped by expert in token
  * order, each group padded to a multiple of 256 rows (padding rows are zero);
@@ -278,6 +304,16 @@ int jpp_stage_zero_grads(jpp_stage* stage, void* stream);
  * gradients, with two_streams).  Call it before reading the accumulators on `stream`;
  * jpp_stage_zero_grads does it by itself.  A no-op without two_streams. */
 int jpp_stage_join(jpp_stage* stage, void* stream);
+/* Optimizer state of a stage: f32 weights (cast up from the bf16 parameters as they are
+ * now) and zeroed moments, laid out like the parameters; allocated by the first call,
+ * reset by later ones (call it again after writing parameters through
+ * jpp_stage_param_ptr).  `which` of jpp_stage_opt_ptr: 0 f32 weights, 1 m, 2 v. */
+int jpp_stage_optimizer_init(jpp_stage* stage, void* stream);
+int jpp_stage_opt_ptr(jpp_stage* stage, int which, int chunk, int layer, int index, float** ptr);
+/* jpp_adam_step over every parameter of the stage (one launch), clearing the gradient
+ * accumulators; joins the stage's second stream first. */
+int jpp_stage_adam_step(jpp_stage* stage, void* stream, int64_t step, double lr, double beta1,
+                        double beta2, double eps, double grad_scale);
 size_t jpp_stage_bytes(const jpp_stage* stage);
 /* One task.  `in` is the incoming boundary activation (FWD) or cotangent
  * (BWD, BWD_I), `out` receives the outgoing activation / cotangent; both are

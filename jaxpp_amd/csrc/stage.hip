@@ -73,6 +73,7 @@ struct jpp_stage {
   size_t layer_elems = 0;
   bf16_t* params = nullptr;        // [chunk][layer][layer_elems] bf16
   float* grads = nullptr;          // same shape, f32
+  float* opt[3] = {nullptr, nullptr, nullptr};  // f32 weights, m, v of the optimizer (same shape)
   std::vector<LayerStash> lay;     // per layer of a chunk, offsets into a slot
   size_t slot_bytes = 0;
   std::vector<uint8_t*> slots;
@@ -618,6 +619,8 @@ int jpp_stage_destroy(jpp_stage* s) {
   if (s->side) hipStreamDestroy(s->side);
   for (auto p : s->slots) hipFree(p);
   if (s->scratch) hipFree(s->scratch);
+  for (auto p : s->opt)
+    if (p) hipFree(p);
   if (s->grads) hipFree(s->grads);
   if (s->params) hipFree(s->params);
   delete s;
@@ -666,6 +669,52 @@ int jpp_stage_zero_grads(jpp_stage* s, void* stream) {
   RC(jpp_stage_join(s, stream));  // weight gradients still in flight accumulate into the old values
   const size_t n = (size_t)s->d.n_chunks * s->d.layers_per_chunk * s->layer_elems;
   return jpp_fill_u32(s->grads, 0u, n, stream);
+}
+
+int jpp_stage_optimizer_init(jpp_stage* s, void* stream) {
+  JPP_REQUIRE(s, "stage: null");
+  const size_t n = (size_t)s->d.n_chunks * s->d.layers_per_chunk * s->layer_elems;
+  for (auto& p : s->opt)
+    if (!p) {
+      if (hipMalloc((void**)&p, n * 4) != hipSuccess) {
+        p = nullptr;
+        (void)hipGetLastError();
+        return jpp_set_error(JPP_ERR_HIP, "optimizer_init: cannot allocate %zu bytes of state", n * 4);
+      }
+      s->total_bytes += n * 4;
+    }
+  RC(jpp_cast_bf16_to_f32(stream, s->params, s->opt[0], (int64_t)n));
+  RC(jpp_fill_u32(s->opt[1], 0u, n, stream));
+  return jpp_fill_u32(s->opt[2], 0u, n, stream);
+}
+
+int jpp_stage_opt_ptr(jpp_stage* s, int which, int chunk, int layer, int i, float** ptr) {
+  RC(check_pli(s, chunk, layer, i));
+  JPP_REQUIRE(which >= 0 && which < 3, "opt_ptr: which = %d, expected 0 (weights), 1 (m) or 2 (v)",
+              which);
+  JPP_REQUIRE(s->opt[which], "opt_ptr: jpp_stage_optimizer_init has not run");
+  *ptr = s->opt[which] + (s->G(chunk, layer, i) - s->grads);
+  return JPP_OK;
+}
+
+int jpp_stage_adam_step(jpp_stage* s, void* stream, int64_t step, double lr, double beta1,
+                        double beta2, double eps, double grad_scale) {
+  JPP_REQUIRE(s, "stage: null");
+  JPP_REQUIRE(s->opt[0] && s->opt[1] && s->opt[2],
+              "adam_step: jpp_stage_optimizer_init has not run");
+  RC(jpp_stage_join(s, stream));  // weight gradients may still be running on the second stream
+  jpp_adam_args a;
+  a.count = (int64_t)s->d.n_chunks * s->d.layers_per_chunk * (int64_t)s->layer_elems;
+  a.grad = s->grads;
+  a.master = s->opt[0];
+  a.param = s->params;
+  a.m = s->opt[1];
+  a.v = s->opt[2];
+  a.step = step;
+  a.lr = lr; a.beta1 = beta1; a.beta2 = beta2; a.eps = eps;
+  a.grad_scale = grad_scale;
+  a.zero_grad = 1;
+  return jpp_adam_step(stream, &a);
 }
 
 size_t jpp_stage_bytes(const jpp_stage* s) { return s ? s->total_bytes : 0; }

@@ -65,6 +65,13 @@ class MoeArgs(C.Structure):
                 ("hidden", C.c_int64), ("n_experts", C.c_int), ("top_k", C.c_int)]
 
 
+class AdamArgs(C.Structure):
+    _fields_ = [("count", C.c_int64), ("grad", C.c_void_p), ("master", C.c_void_p),
+                ("param", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("step", C.c_int64),
+                ("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double),
+                ("eps", C.c_double), ("grad_scale", C.c_double), ("zero_grad", C.c_int)]
+
+
 class StageDesc(C.Structure):
     _fields_ = [("family", C.c_int), ("hidden", C.c_int), ("n_heads", C.c_int),
                 ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("ffn", C.c_int),
@@ -91,7 +98,8 @@ EXPORTS = [
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
-    "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32",
+    "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32", "jpp_adam_step",
+    "jpp_stage_optimizer_init", "jpp_stage_opt_ptr", "jpp_stage_adam_step",
     "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
     "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_join",
     "jpp_stage_bytes",
@@ -179,6 +187,12 @@ def load():
     lib.jpp_stage_run_task.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                        C.c_void_p, C.c_void_p]
     lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
+    lib.jpp_adam_step.argtypes = [C.c_void_p, C.POINTER(AdamArgs)]
+    lib.jpp_stage_optimizer_init.argtypes = [C.c_void_p, C.c_void_p]
+    lib.jpp_stage_opt_ptr.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                      C.POINTER(C.c_void_p)]
+    lib.jpp_stage_adam_step.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_double,
+                                        C.c_double, C.c_double, C.c_double, C.c_double]
     _lib = lib
     return lib
 
@@ -362,6 +376,14 @@ def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, b
     check(load().jpp_gemm_bf16(stream, C.byref(g)))
 
 
+def adam_step(count, grad, m, v, step, master=None, param=None, lr=1e-3, b1=0.9, b2=0.999,
+              eps=1e-8, grad_scale=1.0, zero_grad=False, stream=None):
+    """`optax.adam` + `apply_updates` on flat device tensors (device pointers)."""
+    a = AdamArgs(count, grad, master, param, m, v, step, lr, b1, b2, eps, grad_scale,
+                 int(zero_grad))
+    check(load().jpp_adam_step(stream, C.byref(a)))
+
+
 class StageExecutor:
     """One pipeline rank on one GPU: parameters, fp32 gradient accumulators,
     residual slots, and the FWD / BWD / BWD_I / BWD_W tasks."""
@@ -420,6 +442,23 @@ class StageExecutor:
             upload_ptr(self._ptr(load().jpp_stage_param_ptr, chunk, layer, name),
                        to_bf16_bits(a))
 
+    def get_params(self, chunk: int, layer: int) -> dict:
+        """The bf16 device parameters as float32 host arrays."""
+        self.join()
+        out = {}
+        for name, rows, cols in self.params:
+            shape = (cols,) if rows == 1 and not name.startswith("W") else (rows, cols)
+            bits = download_ptr(self._ptr(load().jpp_stage_param_ptr, chunk, layer, name),
+                                np.uint16, shape)
+            a = from_bf16_bits(bits)
+            order = self._device_columns(name, cols)
+            if order is not None:
+                host = np.empty_like(a)
+                host[:, order] = a
+                a = host
+            out[name] = a
+        return out
+
     def get_grads(self, chunk: int, layer: int) -> dict:
         self.join()          # the copies below run on the null stream
         out = {}
@@ -437,6 +476,39 @@ class StageExecutor:
 
     def zero_grads(self, stream=None):
         check(load().jpp_stage_zero_grads(self.handle, stream))
+
+    def optimizer_init(self, stream=None):
+        """Allocates (first call) and resets the optimizer state: f32 weights cast up from
+        the bf16 parameters as they are now, zero moments."""
+        check(load().jpp_stage_optimizer_init(self.handle, stream))
+
+    def adam_step(self, step: int, lr: float = 1e-3, b1: float = 0.9, b2: float = 0.999,
+                  eps: float = 1e-8, grad_scale: float = 1.0, stream=None):
+        """The update after the loop (README.md:90-93 with `optax.adam`, whose defaults these
+        are): one launch over every parameter of the stage; rewrites the bf16 parameters and
+        clears the gradient accumulators.  `step` counts from 1."""
+        check(load().jpp_stage_adam_step(self.handle, stream, step, lr, b1, b2, eps, grad_scale))
+
+    def get_opt_state(self, chunk: int, layer: int) -> dict:
+        """name -> (f32 weights, m, v) in the host's column order."""
+        self.join()
+        out = {}
+        for name, rows, cols in self.params:
+            shape = (cols,) if rows == 1 and not name.startswith("W") else (rows, cols)
+            order = self._device_columns(name, cols)
+            trio = []
+            for which in range(3):
+                p = C.c_void_p()
+                check(load().jpp_stage_opt_ptr(self.handle, which, chunk, layer, self.index[name],
+                                               C.byref(p)))
+                a = download_ptr(p.value, np.float32, shape)
+                if order is not None:
+                    host = np.empty_like(a)
+                    host[:, order] = a
+                    a = host
+                trio.append(a)
+            out[name] = tuple(trio)
+        return out
 
     def join(self, stream=None):
         """Orders `stream` behind the weight-gradient work on the stage's own stream."""

@@ -36,6 +36,8 @@ def test_error_convention_without_gpu():
     assert lib.jpp_stage_create(None, None) == -1
     assert lib.jpp_norm_fwd(None, None) == -1
     assert lib.jpp_grad_accum_f32(None, None, None, 0, 0) == -1
+    assert lib.jpp_adam_step(None, None) == -1
+    assert lib.jpp_stage_adam_step(None, None, 1, 0.0, 0.0, 0.0, 0.0, 0.0) == -1
 
 
 def test_struct_layouts_match_header_sizes():
@@ -44,3 +46,4 @@ def test_struct_layouts_match_header_sizes():
     assert ctypes.sizeof(rt.AttnArgs) == 10 * 8 + 8 * 8 + 6 * 4
     assert ctypes.sizeof(rt.NormArgs) == 12 * 8 + 2 * 8 + 8
     assert ctypes.sizeof(rt.StageDesc) == 20 * 4
+    assert ctypes.sizeof(rt.AdamArgs) == 8 + 5 * 8 + 8 + 5 * 8 + 8
