@@ -174,6 +174,9 @@ def main():
                          "otherwise (+1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
                          "include the other stream's kernels)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="instead of the workload, print what the matrix cores sustain on a "
+                         "register-only MFMA loop (zero and random operands, both tile shapes)")
     ap.add_argument("--after-loop", action="store_true",
                     help="also time the step behind the loop - Adam over the stage's f32 "
                          "gradient accumulators, rewriting the bf16 parameters - and report it "
@@ -185,6 +188,14 @@ def main():
               "supported (the other ranks' boundary tensors are synthetic).", file=sys.stderr)
         sys.exit(2)
     rt.require_gpu()
+    if args.mfma_ceiling:
+        print(json.dumps({"mfma_sustained_tflops": {
+            "32x32x16_zero_operands": rt.mfma_rate(32, False),
+            "32x32x16_random_operands": rt.mfma_rate(32, True),
+            "16x16x32_zero_operands": rt.mfma_rate(16, False),
+            "16x16x32_random_operands": rt.mfma_rate(16, True)},
+            "published_peak_tflops": MFMA_BF16_PEAK / 1e12}))
+        return
     wl = workloads()[args.workload]
     if args.n_mubatches:
         import dataclasses

@@ -74,10 +74,17 @@ int jpp_mem_info(size_t* free_bytes, size_t* total_bytes);
  * algorithmic FLOPs / HBM bytes the launchers declared.  Class names:
  *   gemm_<nn|nt|tn>_<bf16|gelu|dgelu|accf32|f32>_<BM>x<BN>   (nn: y = x W,
  *       nt: dx = dy W^T, tn: dW = x^T dy)
+ *   (+ "w8" for 8-wave tiles, "s3"/"s4" for 3 or 4 LDS stages),
  *   attn_fwd, attn_bwd_dq, attn_bwd_dkv, norm_fwd, norm_bwd, swiglu_fwd,
- *   swiglu_bwd, rope, grad_accum, colsum */
+ *   swiglu_bwd, rope, grad_accum, colsum, adam */
 int jpp_probe_begin(const char* kernel_class);
 int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, double* total_bytes);
+/* No counterpart in the reference: a measurement aid.  TFLOP/s this device sustains on
+ * a register-only loop of bf16 MFMAs on every SIMD (shape 32: 32x32x16, 16: 16x16x32;
+ * operands all zero, or random and different from one MFMA to the next as in a GEMM).
+ * The clock under load depends on how many operand bits toggle, so the second figure is
+ * the ceiling a real GEMM can approach.  Blocks the host (null stream; two runs of about 0.3 us per iteration, the second timed). */
+int jpp_mfma_rate(int shape, int random_operands, int64_t iters, double* tflops);
 
 /* ---- GEMM: stands in for the `dot_general`s of a stage task ----------------
  * C[M,N] = epilogue( sum_k Aop[m,k] * Bop[n,k] ), bf16 operands, fp32 MFMA

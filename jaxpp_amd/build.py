@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libjaxpp_amd.so")
-SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "elementwise.hip", "moe.hip", "optimizer.hip",
+SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "elementwise.hip", "moe.hip", "optimizer.hip", "diagnostics.hip",
            "stage.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          # packed fp32 ops are kept out of generated code on this hardware pool

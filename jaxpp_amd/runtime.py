@@ -94,7 +94,8 @@ EXPORTS = [
     "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_stream_wait_event",
     "jpp_device_sync",
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
-    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
+    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
+    "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
@@ -187,6 +188,7 @@ def load():
     lib.jpp_stage_run_task.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                        C.c_void_p, C.c_void_p]
     lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
+    lib.jpp_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int64, C.POINTER(C.c_double)]
     lib.jpp_adam_step.argtypes = [C.c_void_p, C.POINTER(AdamArgs)]
     lib.jpp_stage_optimizer_init.argtypes = [C.c_void_p, C.c_void_p]
     lib.jpp_stage_opt_ptr.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
@@ -374,6 +376,13 @@ def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, b
                  int(trans_a), int(trans_b), epilogue, gelu_tanh, tile, seg, n_seg, group_mode,
                  stride_b, stride_c, group_rows)
     check(load().jpp_gemm_bf16(stream, C.byref(g)))
+
+
+def mfma_rate(shape: int, random_operands: bool, iters: int = 200000) -> float:
+    """TFLOP/s of a register-only MFMA loop on every SIMD (see jpp_mfma_rate)."""
+    out = C.c_double(0.0)
+    check(load().jpp_mfma_rate(shape, int(random_operands), iters, C.byref(out)))
+    return out.value
 
 
 def adam_step(count, grad, m, v, step, master=None, param=None, lr=1e-3, b1=0.9, b2=0.999,

@@ -412,3 +412,13 @@ def test_gemm_swiglu_epilogues(tile, m, f, k):
     sg = 1 / (1 + np.exp(-g_h))
     want = interleave32(ds * u_h * sg * (1 + g_h * (1 - sg)), ds * g_h * sg)
     close(dgu.download_bf16((m, 2 * f)), want, 1e-2, "dgate/dup")
+
+
+def test_mfma_rate_diagnostic():
+    """The measurement aid runs and lands between a tenth of and just above the published peak."""
+    for shape in (16, 32):
+        for rnd in (False, True):
+            t = rt.mfma_rate(shape, rnd, iters=4000)
+            assert 250.0 < t < 2600.0, (shape, rnd, t)
+    with pytest.raises(rt.JppError, match="shape is 16"):
+        rt.mfma_rate(8, False)
