@@ -190,10 +190,10 @@ def main():
     rt.require_gpu()
     if args.mfma_ceiling:
         print(json.dumps({"mfma_sustained_tflops": {
-            "32x32x16_zero_operands": rt.mfma_rate(32, False),
-            "32x32x16_random_operands": rt.mfma_rate(32, True),
-            "16x16x32_zero_operands": rt.mfma_rate(16, False),
-            "16x16x32_random_operands": rt.mfma_rate(16, True)},
+            "32x32x16_zero_operands": rt.mfma_rate(32, False, 200000),
+            "32x32x16_random_operands": rt.mfma_rate(32, True, 200000),
+            "16x16x32_zero_operands": rt.mfma_rate(16, False, 100000),
+            "16x16x32_random_operands": rt.mfma_rate(16, True, 100000)},
             "published_peak_tflops": MFMA_BF16_PEAK / 1e12}))
         return
     wl = workloads()[args.workload]

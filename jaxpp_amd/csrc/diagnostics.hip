@@ -12,7 +12,8 @@ __device__ __forceinline__ uint32_t lcg(uint32_t& s) {
   return s;
 }
 
-// SHAPE 32: v_mfma_f32_32x32x16_bf16 on 8 accumulators; 16: v_mfma_f32_16x16x32_bf16 on 16.
+// SHAPE 32: v_mfma_f32_32x32x16_bf16 on 8 accumulators; 16: v_mfma_f32_16x16x32_bf16 on 32
+// (128 accumulator registers either way).
 // Operands differ from one MFMA to the next (as in a GEMM) unless they are all zero.
 template <int SHAPE>
 __global__ __launch_bounds__(512) void mfma_rate_kernel(float* out, int iters, int random_operands) {
@@ -27,14 +28,14 @@ __global__ __launch_bounds__(512) void mfma_rate_kernel(float* out, int iters, i
     }
   float sum = 0.f;
   if constexpr (SHAPE == 16) {
-    f32x4 acc[16];
-    for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[32];
+    for (int i = 0; i < 32; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
+      for (int i = 0; i < 32; ++i)
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i & 7], b[(i * 3 + 1) & 7], acc[i], 0, 0, 0);
     }
-    for (int i = 0; i < 16; ++i) sum += acc[i][0];
+    for (int i = 0; i < 32; ++i) sum += acc[i][0];
   } else {
     f32x16 acc[8];
     for (int i = 0; i < 8; ++i)
@@ -81,7 +82,8 @@ extern "C" int jpp_mfma_rate(int shape, int random_operands, int64_t iters, doub
   hipFree(out);
   if (err != hipSuccess)
     return jpp_set_error(JPP_ERR_HIP, "mfma_rate: %s", hipGetErrorString(err));
-  // 16 MFMAs of 2*16*16*32 or 8 of 2*32*32*16 flops per trip: the same 262144 per wave
-  *tflops = (double)kBlocks * 8 * (double)iters * 262144.0 / (ms * 1e-3) / 1e12;
+  // per trip and wave: 32 MFMAs of 2*16*16*32 flops or 8 of 2*32*32*16
+  const double per_trip = shape == 16 ? 32 * 16384.0 : 8 * 32768.0;
+  *tflops = (double)kBlocks * 8 * (double)iters * per_trip / (ms * 1e-3) / 1e12;
   return JPP_OK;
 }

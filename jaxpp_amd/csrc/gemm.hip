@@ -272,17 +272,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
       constexpr int PARTS = TMH < IA && TMH < IB ? TMH : (IA < IB ? IA : IB);
       static_assert(IA % PARTS == 0 && IB % PARTS == 0 && TMH % PARTS == 0,
                     "loads per wave must split over the MFMA rows");
+      // MFMAs go in 2x2 groups of tiles: of two consecutive MFMAs one operand stays the same
+      // and the other alternates between two fragments, so fewer operand bits toggle per
+      // issue than row by row (the clock under load follows the toggling)
+      static_assert(TMH % 2 == 0 && TN % 2 == 0, "2x2 groups of MFMA tiles");
 #pragma unroll
-      for (int i = 0; i < TMH; ++i) {
-        if (ks == NB - 1 && i % (TMH / PARTS) == 0) {
-          TileA::template issue_part<IA / PARTS>(i / (TMH / PARTS), ga, offa, lds0 + st * STAGE, wave);
-          TileB::template issue_part<IB / PARTS>(i / (TMH / PARTS), gb, offb,
-                                                 lds0 + st * STAGE + A_BYTES, wave);
+      for (int ib = 0; ib < TMH / 2; ++ib) {
+        if (ks == NB - 1) {
+#pragma unroll
+          for (int i = 2 * ib; i < 2 * ib + 2; ++i)
+            if (i % (TMH / PARTS) == 0) {
+              TileA::template issue_part<IA / PARTS>(i / (TMH / PARTS), ga, offa, lds0 + st * STAGE, wave);
+              TileB::template issue_part<IB / PARTS>(i / (TMH / PARTS), gb, offb,
+                                                     lds0 + st * STAGE + A_BYTES, wave);
+            }
         }
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[part * TMH + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              fw[curw][j], fx[cur][i], acc[part * TMH + i][j], 0, 0, 0);
+        for (int jb = 0; jb < TN / 2; ++jb)
+#pragma unroll
+          for (int i = 2 * ib; i < 2 * ib + 2; ++i)
+#pragma unroll
+            for (int j = 2 * jb; j < 2 * jb + 2; ++j)
+              acc[part * TMH + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  fw[curw][j], fx[cur][i], acc[part * TMH + i][j], 0, 0, 0);
       }
     }
     if constexpr (EPI == JPP_EPI_ACC_F32) {

@@ -378,7 +378,7 @@ def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, b
     check(load().jpp_gemm_bf16(stream, C.byref(g)))
 
 
-def mfma_rate(shape: int, random_operands: bool, iters: int = 200000) -> float:
+def mfma_rate(shape: int, random_operands: bool, iters: int = 100000) -> float:
     """TFLOP/s of a register-only MFMA loop on every SIMD (see jpp_mfma_rate)."""
     out = C.c_double(0.0)
     check(load().jpp_mfma_rate(shape, int(random_operands), iters, C.byref(out)))
