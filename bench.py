@@ -117,8 +117,9 @@ MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.133e9}
 def dominant_gemm_class(wl) -> str:
     # weight-gradient GEMM with the fp32 accumulate epilogue: a third of the
     # FLOPs and the longest kernel per call
+    # (narrow layers: 128x128 tiles, at most two per CU, so the 3-stage variant)
     big = wl.layer.hidden >= 4096
-    return "gemm_tn_accf32_256x256w8" if big else "gemm_tn_accf32_128x128w8"
+    return "gemm_tn_accf32_256x256w8" if big else "gemm_tn_accf32_128x128w8s3"
 
 
 def cpu_baseline(wl, budget_layers: int = 1):
