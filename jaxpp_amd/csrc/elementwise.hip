@@ -183,23 +183,32 @@ __global__ __launch_bounds__(kNormBwdWaves * 64) void norm_bwd_kernel(
   }
 }
 
-// acc[j] += sum_b partial[b][j]: a block owns 32 columns; 8 thread groups sum
-// interleaved subsets of the partials, then one combines them in a fixed order
-__global__ __launch_bounds__(256) void partial_reduce_kernel(const float* __restrict__ partial,
-                                                             int nblocks, int cols,
-                                                             float* __restrict__ acc) {
-  __shared__ float red[8][32];
+// acc[j] += sum_b partial[b][j]: a block owns 32 columns; 32 thread groups sum interleaved
+// subsets of the partials (8 independent loads each for 256 partials), then one combines them
+// in a fixed order.  blockIdx.y picks one of two reductions (gamma and beta of a LayerNorm
+// share a launch): the second one's partials follow the first's, its accumulator is acc2.
+__global__ __launch_bounds__(1024) void partial_reduce_kernel(const float* __restrict__ partial,
+                                                              int nblocks, int cols,
+                                                              float* __restrict__ acc,
+                                                              float* __restrict__ acc2) {
+  __shared__ float red[32][33];
   const int c = threadIdx.x & 31, g = threadIdx.x >> 5;
   const int j = blockIdx.x * 32 + c;
+  if (blockIdx.y) {
+    partial += (long)nblocks * cols;
+    acc = acc2;
+  }
   float s = 0.f;
-  if (j < cols)
-    for (int b = g; b < nblocks; b += 8) s += partial[(long)b * cols + j];
+  if (j < cols) {
+#pragma unroll 8
+    for (int b = g; b < nblocks; b += 32) s += partial[(long)b * cols + j];
+  }
   red[g][c] = s;
   __syncthreads();
   if (g == 0 && j < cols) {
     float t = red[0][c];
 #pragma unroll
-    for (int w = 1; w < 8; ++w) t += red[w][c];
+    for (int w = 1; w < 32; ++w) t += red[w][c];
     acc[j] += t;
   }
 }
@@ -431,11 +440,8 @@ int launch_norm_bwd(hipStream_t st, const jpp_norm_args* a) {
 #undef JPP_NB
   JPP_LAUNCH_CHECK();
   const int cb = (int)((a->cols + 31) / 32);
-  hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb), dim3(256), 0, st, a->partial, blocks,
-                     (int)a->cols, a->dgamma);
-  if (LN)
-    hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb), dim3(256), 0, st,
-                       a->partial + (long)blocks * a->cols, blocks, (int)a->cols, a->dbeta);
+  hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb, LN ? 2 : 1), dim3(1024), 0, st, a->partial,
+                     blocks, (int)a->cols, a->dgamma, a->dbeta);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -547,8 +553,8 @@ int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int6
   const int panels = (int)((cols / 8 + 255) / 256);
   hipLaunchKernelGGL(colsum_partial_kernel, dim3(nb, panels), dim3(256), 0, st, (const bf16_t*)x,
                      (long)ld, (long)rows, (int)cols, partial);
-  hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 31) / 32)), dim3(256), 0, st,
-                     partial, nb, (int)cols, acc);
+  hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 31) / 32)), dim3(1024), 0, st,
+                     partial, nb, (int)cols, acc, (float*)nullptr);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
