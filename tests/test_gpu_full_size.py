@@ -1,0 +1,157 @@
+"""Parity at the sizes the bench runs (Llama-3-8B-shaped layer: hidden 4096, 32/8 heads of
+128, SwiGLU 14336, 4096 tokens), where the small cases of the other files do not reach: K
+loops long enough for the accumulate GEMM to stream its output tile and for the deep-stage
+tiles, tile grids of several rounds per CU, attention over 64 key blocks.
+
+* GEMMs: checksums that any dropped, duplicated or misplaced tile breaks - row sums and
+  column sums of the f32 result against matrix-vector products of the operands (f64 on the
+  host), plus a dense comparison of a few full rows and columns.
+* One whole layer (forward, backward, weight gradients) against the numpy oracle, and
+  exact doubling of the accumulators when the same microbatch is run twice.
+
+Tolerances: f32 GEMM results 1e-4 sqrt(K) of the largest magnitude, bf16 GEMM results 1e-2 (as
+for the small cases); bf16 tensors of the layer 2e-2 of the tensor's largest magnitude."""
+import math
+
+import numpy as np
+import pytest
+
+from jaxpp_amd import runtime as rt
+from jaxpp_amd import schedules as S
+from jaxpp_amd.model import LayerSpec
+from jaxpp_amd.plan import make_rank_plan
+from oracle import layers as L
+
+from test_gpu_stage import close, make_params, run_on_gpu, run_on_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    rt.require_gpu()
+
+
+def rnd(rng, *shape, scale=1.0):
+    return L.bf16_round((rng.standard_normal(shape, dtype=np.float32) * np.float32(scale)))
+
+
+# (layout, M, N, K, epilogue, tile): the shapes of the bench's GEMM classes and the tiles
+# that the small cases cannot drive into their long-K code paths
+FULL = [
+    ("nn", 4096, 28672, 4096, rt.EPI_F32, 0),       # gate/up projection
+    ("nt", 4096, 4096, 14336, rt.EPI_BF16, 0),      # input gradient of the down projection
+    ("tn", 4096, 28672, 4096, rt.EPI_ACC_F32, 0),   # weight gradient, streamed accumulator
+    ("tn", 14336, 4096, 4096, rt.EPI_ACC_F32, 0),
+    ("tn", 1024, 1024, 4096, rt.EPI_ACC_F32, 1),    # 128x128, 3 LDS stages
+    ("nn", 1024, 1024, 4096, rt.EPI_F32, 1),        # 128x128, 4 LDS stages
+    ("nt", 2048, 1024, 4096, rt.EPI_BF16, 2),       # 256x128 on 4 waves
+]
+
+
+@pytest.mark.parametrize("lay,m,n,k,epi,tile", FULL, ids=[f"{c[0]}-{c[1]}x{c[2]}x{c[3]}-t{c[5]}" for c in FULL])
+def test_gemm_checksums_at_full_size(lay, m, n, k, epi, tile):
+    print(f"full-size gemm {lay} {m}x{n}x{k} epi={epi} tile={tile}", flush=True)
+    rng = np.random.default_rng(m + n + k)
+    ta, tb = {"nn": (0, 1), "nt": (0, 0), "tn": (1, 1)}[lay]
+    A = rnd(rng, m, k)                       # logical [M, K]
+    B = rnd(rng, n, k, scale=0.05)           # logical [N, K]
+    a_h = np.ascontiguousarray(A.T) if ta else A
+    b_h = np.ascontiguousarray(B.T) if tb else B
+    da, db = rt.DeviceBuffer.from_f32_as_bf16(a_h), rt.DeviceBuffer.from_f32_as_bf16(b_h)
+    prev = None
+    if epi == rt.EPI_ACC_F32:
+        prev = rng.standard_normal((m, n), dtype=np.float32)
+        dc = rt.DeviceBuffer.from_numpy(prev)
+    else:
+        dc = rt.DeviceBuffer(m * n * (2 if epi == rt.EPI_BF16 else 4))
+    rt.gemm(da.ptr, db.ptr, dc.ptr, m, n, k, a_h.shape[1], b_h.shape[1], n, ta, tb, epi, tile=tile)
+    rt.sync()
+    got = (dc.download_bf16((m, n)) if epi == rt.EPI_BF16
+           else dc.download(np.float32, (m, n))).astype(np.float64)
+    assert np.isfinite(got).all()
+    A64, B64 = A.astype(np.float64), B.astype(np.float64)
+    p64 = prev.astype(np.float64) if prev is not None else None
+    # per-element bound, as for the small cases (a bf16 result: 1e-2, of which rounding to
+    # 8 bits takes 2^-8); a sum of n such errors grows like sqrt(n)
+    elem = (1e-2 if epi == rt.EPI_BF16 else 1e-4 * math.sqrt(k)) * float(np.abs(got).max())
+    row_want = A64 @ B64.sum(axis=0) + (p64.sum(axis=1) if prev is not None else 0.0)
+    col_want = B64 @ A64.sum(axis=0) + (p64.sum(axis=0) if prev is not None else 0.0)
+    assert np.abs(got.sum(axis=1) - row_want).max() <= elem * math.sqrt(n), "row checksums"
+    assert np.abs(got.sum(axis=0) - col_want).max() <= elem * math.sqrt(m), "column checksums"
+    rows = sorted(set(int(r) for r in rng.integers(0, m, 6)) | {0, m - 1, 255, 256})
+    cols = sorted(set(int(c) for c in rng.integers(0, n, 6)) | {0, n - 1, 255, 256})
+    want_rows = A64[rows] @ B64.T + (p64[rows] if prev is not None else 0.0)
+    want_cols = A64 @ B64[cols].T + (p64[:, cols] if prev is not None else 0.0)
+    assert np.abs(got[rows] - want_rows).max() <= elem, "dense rows"
+    assert np.abs(got[:, cols] - want_cols).max() <= elem, "dense columns"
+
+
+LLAMA_8B_LAYER = LayerSpec("llama", 4096, 32, 14336, 4096, 1, n_kv_heads=8, head_dim=128,
+                           causal=True, rope_theta=5e5, eps=1e-5)
+
+
+def test_llama_8b_layer_matches_oracle():
+    """One layer of the bench's stage at full size: forward, backward and weight gradients of
+    one microbatch against the oracle; a second pass over the same microbatch must double
+    every accumulator up to f32 rounding (the GEMM folds the old value into its running sums
+    part-way through the K loop, so the second sum is rounded differently from the first)."""
+    spec, lpc = LLAMA_8B_LAYER, 1
+    sched = S.Std1F1B(1)
+    plan1 = make_rank_plan(sched, 1, 0)
+    params = make_params(spec, plan1.stages, lpc)
+    row = S.preprocess_schedule_tasks(sched.tasks(1), 0, False)[0]
+    print("full-size layer: oracle", flush=True)
+    ys_w, dxs_w, acc_w = run_on_oracle(spec, plan1, params, row)
+    print("full-size layer: gpu", flush=True)
+    ys, dxs, grads = run_on_gpu(spec, plan1, lpc, params, two_streams=False)
+    for key in ys_w:
+        close(ys[key], ys_w[key], 2e-2, f"y{key}")
+    for key in dxs_w:
+        close(dxs[key], dxs_w[key], 2e-2, f"dx{key}")
+    for pname, want in acc_w[0][0].items():
+        got = grads[0][0][pname]
+        close(got, want.reshape(got.shape), 2e-2, f"grad {pname}")
+    # the same microbatch twice (boundary tensors depend on the microbatch index, so the
+    # second pass is a second run of microbatch 0 into the same accumulators)
+    shape = (spec.tokens, spec.hidden)
+    from jaxpp_amd.model import boundary_tensor
+    from jaxpp_amd.types import TaskType
+    ex = rt.StageExecutor(spec, 1, lpc, 1, False, True, False)
+    ex.set_params(0, 0, params[0][0])
+    x = rt.DeviceBuffer.from_f32_as_bf16(boundary_tensor("x", 0, 0, shape, 0))
+    dy = rt.DeviceBuffer.from_f32_as_bf16(boundary_tensor("dy", 0, 0, shape, 0))
+    out = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+    for _ in range(2):
+        ex.run_task(TaskType.FWD, 0, 0, x.ptr, out.ptr)
+        ex.run_task(TaskType.BWD, 0, 0, dy.ptr, out.ptr)
+    rt.sync()
+    twice = ex.get_grads(0, 0)
+    ex.close()
+    for pname, once in grads[0][0].items():
+        close(twice[pname], 2.0 * once, 1e-5, f"accumulated twice: {pname}")
+
+
+BERT_LARGE_LAYER = LayerSpec("bert", 1024, 16, 4096, 512, 8, eps=1e-12)
+
+
+@pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
+def test_bert_large_layers_match_oracle(two_streams):
+    """Two layers of the BERT-large stage at full size (8 x 512 tokens, hidden 1024, heads of
+    64), two microbatches of a 1F1B row, against the oracle."""
+    spec, lpc, n = BERT_LARGE_LAYER, 2, 2
+    sched = S.Std1F1B(2)
+    plan = make_rank_plan(sched, n, 1)
+    params = make_params(spec, plan.stages, lpc)
+    row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[1]
+    ys_w, dxs_w, acc_w = run_on_oracle(spec, plan, params, row)
+    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params, two_streams=two_streams)
+    for key in ys_w:
+        close(ys[key], ys_w[key], 2e-2, f"y{key}")
+    for key in dxs_w:
+        close(dxs[key], dxs_w[key], 2e-2, f"dx{key}")
+    for s_ in plan.stages:
+        for li in range(lpc):
+            for pname, want in acc_w[s_][li].items():
+                got = grads[s_][li][pname]
+                close(got, want.reshape(got.shape), 2e-2, f"grad {s_}/{li}/{pname}")
