@@ -491,7 +491,8 @@ int launch(hipStream_t stream, GemmParams& p) {
 template <bool TA, bool TB, int EPI>
 int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
   switch (tile) {
-    case 2: return launch<256, 128, TA, TB, EPI>(stream, p);
+    case 2:  // 8 waves of 128x32; three stages where the accumulator rows leave room
+      return launch<256, 128, TA, TB, EPI, 8, EPI == JPP_EPI_ACC_F32 ? 2 : 3>(stream, p);
     case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
     default:
       // 128x128: 8 waves (64x32 each) except for the SwiGLU epilogues, which need a wave to
@@ -516,6 +517,41 @@ int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
 int choose_tile(long m, long n) {
   const long t256 = (m % 256 == 0 && n % 256 == 0) ? (m / 256) * (n / 256) : 0;
   return t256 >= 192 ? 4 : 1;
+}
+
+
+// sub-problem whose first row / column is (m_off, n_off) of the full one
+void shift_origin(GemmParams& p, bool ta, bool tb, int epi, long m_off, long n_off) {
+  p.a += ta ? m_off : m_off * p.lda;
+  p.b += tb ? n_off : n_off * p.ldb;
+  const long c_cols = epi == JPP_EPI_DSWIGLU ? 2 * n_off : n_off;  // dSwiGLU writes d gate, d up
+  const bool f32 = epi == JPP_EPI_ACC_F32 || epi == JPP_EPI_F32;
+  p.c = f32 ? (void*)((float*)p.c + m_off * p.ldc + c_cols)
+            : (void*)((bf16_t*)p.c + m_off * p.ldc + c_cols);
+  if (p.c2)  // SwiGLU: s has one column per gate/up pair; GELU: as wide as C
+    p.c2 = (bf16_t*)p.c2 + m_off * p.ldc2 + (epi == JPP_EPI_SWIGLU ? n_off / 2 : n_off);
+  if (p.bias) p.bias += n_off;
+  if (p.resid) p.resid += m_off * p.ldresid + n_off;
+  if (p.aux) p.aux += m_off * p.ldaux + c_cols;
+}
+
+int dispatch(hipStream_t stream, const jpp_gemm_args* a, GemmParams& p, int tile) {
+  const int ta = a->trans_a != 0, tb = a->trans_b != 0, e = a->epilogue;
+#define JPP_GEMM_CASE(TA_, TB_, E_) \
+  if (ta == TA_ && tb == TB_ && e == E_) return launch_tiled<TA_, TB_, E_>(stream, p, tile)
+  JPP_GEMM_CASE(0, 1, JPP_EPI_BF16);     // forward
+  JPP_GEMM_CASE(0, 1, JPP_EPI_GELU);     // forward + GELU
+  JPP_GEMM_CASE(0, 1, JPP_EPI_F32);      // forward, f32 out (router logits)
+  JPP_GEMM_CASE(0, 1, JPP_EPI_SWIGLU);   // gate/up projection + SwiGLU
+  JPP_GEMM_CASE(0, 0, JPP_EPI_BF16);     // input gradient
+  JPP_GEMM_CASE(0, 0, JPP_EPI_DGELU);    // input gradient through GELU
+  JPP_GEMM_CASE(0, 0, JPP_EPI_DSWIGLU);  // input gradient through SwiGLU
+  JPP_GEMM_CASE(1, 1, JPP_EPI_ACC_F32);  // weight gradient, accumulated
+  JPP_GEMM_CASE(1, 1, JPP_EPI_BF16);     // weight gradient, bf16
+  JPP_GEMM_CASE(1, 1, JPP_EPI_F32);      // weight gradient, f32
+#undef JPP_GEMM_CASE
+  return jpp_set_error(JPP_ERR_INVALID, "gemm: unsupported combination trans_a=%d trans_b=%d epilogue=%d",
+                       ta, tb, e);
 }
 
 }  // namespace
@@ -582,20 +618,30 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   if (tile >= 2 && a->m % 256) tile = 1;
   if (tile == 4 && a->n % 256) tile = 2;
 
-  const int ta = a->trans_a != 0, tb = a->trans_b != 0, e = a->epilogue;
-#define JPP_GEMM_CASE(TA_, TB_, E_) \
-  if (ta == TA_ && tb == TB_ && e == E_) return launch_tiled<TA_, TB_, E_>(stream, p, tile)
-  JPP_GEMM_CASE(0, 1, JPP_EPI_BF16);     // forward
-  JPP_GEMM_CASE(0, 1, JPP_EPI_GELU);     // forward + GELU
-  JPP_GEMM_CASE(0, 1, JPP_EPI_F32);      // forward, f32 out (router logits)
-  JPP_GEMM_CASE(0, 1, JPP_EPI_SWIGLU);   // gate/up projection + SwiGLU
-  JPP_GEMM_CASE(0, 0, JPP_EPI_BF16);     // input gradient
-  JPP_GEMM_CASE(0, 0, JPP_EPI_DGELU);    // input gradient through GELU
-  JPP_GEMM_CASE(0, 0, JPP_EPI_DSWIGLU);  // input gradient through SwiGLU
-  JPP_GEMM_CASE(1, 1, JPP_EPI_ACC_F32);  // weight gradient, accumulated
-  JPP_GEMM_CASE(1, 1, JPP_EPI_BF16);     // weight gradient, bf16
-  JPP_GEMM_CASE(1, 1, JPP_EPI_F32);      // weight gradient, f32
-#undef JPP_GEMM_CASE
-  return jpp_set_error(JPP_ERR_INVALID, "gemm: unsupported combination trans_a=%d trans_b=%d epilogue=%d",
-                       ta, tb, e);
+  // A grid of 256x256 tiles whose last round fills at most half of the 256 CUs runs that
+  // round as a separate launch of 256x128 tiles over the last rows or columns: a full round
+  // of half-size tiles takes little more than half the time the half-empty round did.
+  // (Only when the choice of tile was left to the library.)
+  if (tile == 4 && a->tile == 0 && a->group_mode == JPP_GROUP_NONE) {
+    const long tm = a->m / 256, tn = a->n / 256, rest = (tm * tn) % 256;
+    if (tm * tn > 256 && rest > 0 && rest <= 128) {
+      const long rows = rest % tn == 0 ? rest / tn * 256 : 0;             // split along M
+      const long cols = !rows && rest % tm == 0 ? rest / tm * 256 : 0;    // split along N
+      if (rows || cols) {
+        GemmParams head = p, tail = p;
+        if (rows) {
+          head.m = p.m - (int)rows;
+          tail.m = (int)rows;
+          shift_origin(tail, a->trans_a != 0, a->trans_b != 0, a->epilogue, head.m, 0);
+        } else {
+          head.n = p.n - (int)cols;
+          tail.n = (int)cols;
+          shift_origin(tail, a->trans_a != 0, a->trans_b != 0, a->epilogue, 0, head.n);
+        }
+        const int rc = dispatch(stream, a, head, 4);
+        return rc != JPP_OK ? rc : dispatch(stream, a, tail, 2);
+      }
+    }
+  }
+  return dispatch(stream, a, p, tile);
 }
