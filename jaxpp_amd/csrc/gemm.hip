@@ -495,11 +495,11 @@ int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
       return launch<256, 128, TA, TB, EPI, 8, EPI == JPP_EPI_ACC_F32 ? 2 : 3>(stream, p);
     case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
     default:
-      // 128x128: 8 waves (64x32 each) except for the SwiGLU epilogues, which need a wave to
-      // span 64 columns.  With more tiles than two per CU, two stages and two workgroups per
-      // CU; with fewer (and a K loop long enough to pay for the longer prologue) the one
-      // workgroup a CU gets prefetches deeper instead (4 stages, 3 where the accumulator
-      // rows need room too).
+      // 128x128: 8 waves (64x32 each); the SwiGLU epilogues, which no measured workload
+      // reaches at this tile size, keep the plain 4-wave form.  With more tiles than two per
+      // CU, two stages and two workgroups per CU; with fewer (and a K loop long enough to pay
+      // for the longer prologue) the one workgroup a CU gets prefetches deeper instead (4
+      // stages, 3 where the accumulator rows need room too).
       if constexpr (EPI == JPP_EPI_SWIGLU || EPI == JPP_EPI_DSWIGLU) {
         return launch<128, 128, TA, TB, EPI>(stream, p);
       } else {
