@@ -92,17 +92,17 @@ class Workbench:
         rt.sync()
         self._keep = (wpool, ones, bpool)
 
-    def step(self):
+    def step(self, stream=None):
         ex = self.ex
-        ex.zero_grads()                       # `Add.state`: accumulators start from zero
+        ex.zero_grads(stream)                 # `Add.state`: accumulators start from zero
 
         def io(pt, lane):
             m = pt.task.mubatch_idx
             src = self.x_in if pt.exec_kind is TaskType.FWD else self.dy_in
             return src[pt.chunk, m].ptr, self.out[lane].ptr
 
-        self.loop.run(io)
-        ex.join()                             # the step ends when the last weight gradient has landed
+        self.loop.run(io, stream=stream)
+        ex.join(stream)                       # the step ends when the last weight gradient has landed
 
     def step_flops(self) -> float:
         wl = self.wl
@@ -175,6 +175,11 @@ def main():
                          "otherwise (+1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
                          "include the other stream's kernels)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
+    ap.add_argument("--graph", action="store_true",
+                    help="record the step into a HIP graph after the warm-up and time replays "
+                         "of it (no host launch work in the timed region); the per-kernel probe "
+                         "cannot see inside a replay, so `roofline` then comes from one more "
+                         "eager step after the timed ones")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="instead of the workload, print what the matrix cores sustain on a "
                          "register-only MFMA loop (zero and random operands, both tile shapes)")
@@ -209,12 +214,32 @@ def main():
         wb.step()
     rt.sync()
     start, stop = rt.Event(), rt.Event()
-    with rt.probe(cls) as pr:
-        start.record()
+    if args.graph:
+        stream = rt.Stream()
+        if not args.warmup:
+            wb.step(stream.ptr)               # first launches configure their kernels
+            stream.sync()
+        wb.ex.quiesce()
+        graph = rt.Graph(stream)
+        with graph:
+            wb.step(stream.ptr)
+        graph.launch()                        # one untimed replay
+        stream.sync()
+        start.record(stream.ptr)
         for _ in range(args.steps):
-            wb.step()
-        stop.record()
+            graph.launch()
+        stop.record(stream.ptr)
         stop.sync()
+        with rt.probe(cls) as pr:
+            wb.step()
+            rt.sync()
+    else:
+        with rt.probe(cls) as pr:
+            start.record()
+            for _ in range(args.steps):
+                wb.step()
+            stop.record()
+            stop.sync()
     rt.sync()
     ms = start.elapsed_ms(stop) / args.steps
     tokens = wl.tokens_per_step
@@ -235,7 +260,7 @@ def main():
             "layers": wl.layers_per_stage * wb.plan.n_chunks,
             "peak_live_microbatches": wb.plan.max_live,
             "fused_wgrad_accumulate": not args.unfused_accumulate,
-            "two_streams": two,
+            "two_streams": two, "hip_graph": bool(args.graph),
             "device_bytes": wb.ex.nbytes,
         },
         "algorithmic_flops_per_step": flops,

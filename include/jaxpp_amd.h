@@ -65,6 +65,20 @@ int jpp_stream_wait_event(void* stream, void* event); /* later work on stream wa
 int jpp_event_sync(void* event);
 int jpp_event_elapsed_ms(void* start, void* stop, float* ms);
 int jpp_mem_info(size_t* free_bytes, size_t* total_bytes);
+/* HIP graphs.  Every entry point of this library only enqueues work on the stream it is
+ * given (and, for a stage with two_streams, on a stream forked from and joined to it with
+ * events), allocates nothing and clears memory with kernels, so a sequence of calls can be
+ * recorded between begin and end and replayed with launch - a rank's whole row of the task
+ * table, for instance.  The reference leaves this to XLA (command buffers); a jax.ffi handler
+ * over these entry points may be marked command-buffer compatible for the same reason.
+ * Record after one eager pass (first launches set kernel attributes) and jpp_stage_quiesce,
+ * on a stream created with jpp_stream_create; call jpp_stage_join on the recording stream
+ * before end; record whole rows of the table (every forward with its backward); probes
+ * (jpp_probe_begin) stay off while recording. */
+int jpp_graph_begin(void* stream);
+int jpp_graph_end(void* stream, void** graph_exec);
+int jpp_graph_launch(void* graph_exec, void* stream);
+int jpp_graph_destroy(void* graph_exec);
 
 /* ---- launch probe: per-kernel timings, the counterpart of the reference's
  * collect_task_times_ms (src/jaxpp/jax_primitives.py:742-773) at kernel
@@ -312,6 +326,10 @@ int jpp_stage_zero_grads(jpp_stage* stage, void* stream);
  * gradients, with two_streams).  Call it before reading the accumulators on `stream`;
  * jpp_stage_zero_grads does it by itself.  A no-op without two_streams. */
 int jpp_stage_join(jpp_stage* stage, void* stream);
+/* Blocks the host until the stage's own stream is idle and forgets the events later tasks
+ * would otherwise wait for.  For use before recording a graph: a recording may not depend on
+ * work that was queued before it began. */
+int jpp_stage_quiesce(jpp_stage* stage);
 /* Optimizer state of a stage: f32 weights (cast up from the bf16 parameters as they are
  * now) and zeroed moments, laid out like the parameters; allocated by the first call,
  * reset by later ones (call it again after writing parameters through

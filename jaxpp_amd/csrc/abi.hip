@@ -127,6 +127,33 @@ int jpp_stream_wait_event(void* stream, void* event) {
   JPP_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0));
   return JPP_OK;
 }
+// ---- HIP graphs: a recorded sequence of calls replayed without host launch work ----
+int jpp_graph_begin(void* stream) {
+  JPP_REQUIRE(stream, "graph_begin: capture needs a stream of its own, not the null stream");
+  JPP_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed));
+  return JPP_OK;
+}
+int jpp_graph_end(void* stream, void** graph_exec) {
+  JPP_REQUIRE(stream && graph_exec, "graph_end: null argument");
+  hipGraph_t graph = nullptr;
+  JPP_CHECK_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+  hipGraphExec_t exec = nullptr;
+  const hipError_t err = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  if (err != hipSuccess)
+    return jpp_set_error(JPP_ERR_HIP, "graph_end: instantiate: %s", hipGetErrorString(err));
+  *graph_exec = exec;
+  return JPP_OK;
+}
+int jpp_graph_launch(void* graph_exec, void* stream) {
+  JPP_REQUIRE(graph_exec, "graph_launch: null graph");
+  JPP_CHECK_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+  return JPP_OK;
+}
+int jpp_graph_destroy(void* graph_exec) {
+  if (graph_exec) JPP_CHECK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+  return JPP_OK;
+}
 int jpp_event_sync(void* event) {
   JPP_CHECK_HIP(hipEventSynchronize((hipEvent_t)event));
   return JPP_OK;

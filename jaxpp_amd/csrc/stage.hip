@@ -664,6 +664,16 @@ int jpp_stage_join(jpp_stage* s, void* stream) {
   return JPP_OK;
 }
 
+int jpp_stage_quiesce(jpp_stage* s) {
+  JPP_REQUIRE(s, "stage: null");
+  if (s->side) JPP_CHECK_HIP(hipStreamSynchronize(s->side));
+  // nothing of the stage's own stream is in flight: no later task has to wait for it
+  std::fill(s->slot_pending.begin(), s->slot_pending.end(), 0);
+  for (auto& p : s->set_pending) p = false;
+  s->tail_pending = false;
+  return JPP_OK;
+}
+
 int jpp_stage_zero_grads(jpp_stage* s, void* stream) {
   JPP_REQUIRE(s, "stage: null");
   RC(jpp_stage_join(s, stream));  // weight gradients still in flight accumulate into the old values

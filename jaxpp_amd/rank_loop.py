@@ -23,26 +23,27 @@ class RankLoop:
             self.aux = rt.Stream()
             self.fork, self.join = rt.Event(), rt.Event()
 
-    def run(self, io):
+    def run(self, io, stream=None):
         """``io(pt, lane)`` -> (in_ptr, out_ptr) for a FWD / BWD / BWD_I task (lane 1: the task
         runs beside another one and needs an output buffer of its own); BWD_W tasks take
-        none.  Everything is queued on the null stream, fused forwards on the second."""
+        none.  Everything is queued on `stream` (a stream pointer; None: the null stream),
+        fused forwards on the loop's second stream."""
         ex = self.ex
         for entry in self.entries:
             beside = self.overlap and len(entry) > 1 and \
                 any(pt.exec_kind is TaskType.FWD for pt in entry) and \
                 any(pt.exec_kind is not TaskType.FWD for pt in entry)
             if beside:
-                self.fork.record(None)
+                self.fork.record(stream)
                 self.aux.wait(self.fork)
             for pt in entry:
                 m = pt.task.mubatch_idx
                 if pt.exec_kind is TaskType.BWD_W:
-                    ex.run_task(pt.exec_kind, pt.chunk, m)
+                    ex.run_task(pt.exec_kind, pt.chunk, m, stream=stream)
                     continue
                 on_aux = beside and pt.exec_kind is TaskType.FWD
                 inp, out = io(pt, 1 if on_aux else 0)
-                ex.run_task(pt.exec_kind, pt.chunk, m, inp, out, self.aux.ptr if on_aux else None)
+                ex.run_task(pt.exec_kind, pt.chunk, m, inp, out, self.aux.ptr if on_aux else stream)
             if beside:
                 self.join.record(self.aux.ptr)
-                rt.stream_wait(None, self.join)
+                rt.stream_wait(stream, self.join)

@@ -94,7 +94,8 @@ EXPORTS = [
     "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_stream_wait_event",
     "jpp_device_sync",
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
-    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
+    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_graph_begin", "jpp_graph_end", "jpp_graph_launch",
+    "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
@@ -103,6 +104,7 @@ EXPORTS = [
     "jpp_stage_optimizer_init", "jpp_stage_opt_ptr", "jpp_stage_adam_step",
     "jpp_stage_create", "jpp_stage_destroy", "jpp_stage_n_params", "jpp_stage_param_info",
     "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_join",
+    "jpp_stage_quiesce",
     "jpp_stage_bytes",
     "jpp_stage_run_task", "jpp_stage_live_slots",
 ]
@@ -141,6 +143,10 @@ def load():
     lib.jpp_event_sync.argtypes = [C.c_void_p]
     lib.jpp_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
     lib.jpp_mem_info.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    lib.jpp_graph_begin.argtypes = [C.c_void_p]
+    lib.jpp_graph_end.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    lib.jpp_graph_launch.argtypes = [C.c_void_p, C.c_void_p]
+    lib.jpp_graph_destroy.argtypes = [C.c_void_p]
     lib.jpp_probe_begin.argtypes = [C.c_char_p]
     lib.jpp_probe_end.argtypes = [C.POINTER(C.c_int64), C.POINTER(C.c_double),
                                   C.POINTER(C.c_double), C.POINTER(C.c_double)]
@@ -185,6 +191,7 @@ def load():
                                        C.POINTER(C.c_void_p)]
     lib.jpp_stage_zero_grads.argtypes = [C.c_void_p, C.c_void_p]
     lib.jpp_stage_join.argtypes = [C.c_void_p, C.c_void_p]
+    lib.jpp_stage_quiesce.argtypes = [C.c_void_p]
     lib.jpp_stage_run_task.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                        C.c_void_p, C.c_void_p]
     lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
@@ -311,6 +318,41 @@ class Stream:
         try:
             if self.ptr:
                 load().jpp_stream_destroy(self.ptr)
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded sequence of calls on `stream` (see jpp_graph_begin in the header)::
+
+        g = Graph(stream)
+        with g:                 # record
+            loop.run(io, stream=stream.ptr); executor.join(stream.ptr)
+        g.launch()              # replay, as often as wanted
+    """
+
+    def __init__(self, stream: Stream):
+        self.stream, self.exec = stream, None
+
+    def __enter__(self):
+        check(load().jpp_graph_begin(self.stream.ptr))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        p = C.c_void_p()
+        rc = load().jpp_graph_end(self.stream.ptr, C.byref(p))
+        if exc_type is None:
+            check(rc)
+            self.exec = p.value
+        return False
+
+    def launch(self, stream=None):
+        check(load().jpp_graph_launch(self.exec, stream if stream is not None else self.stream.ptr))
+
+    def __del__(self):
+        try:
+            if self.exec:
+                load().jpp_graph_destroy(self.exec)
         except Exception:
             pass
 
@@ -522,6 +564,10 @@ class StageExecutor:
     def join(self, stream=None):
         """Orders `stream` behind the weight-gradient work on the stage's own stream."""
         check(load().jpp_stage_join(self.handle, stream))
+
+    def quiesce(self):
+        """Waits (on the host) for the stage's own stream; call before recording a graph."""
+        check(load().jpp_stage_quiesce(self.handle))
 
     def run_task(self, kind: TaskType, chunk: int, mubatch: int, inp=None, out=None,
                  stream=None):

@@ -199,3 +199,69 @@ def test_lifetime_errors():
     ex.close()
     with pytest.raises(rt.JppError, match="head_dim must be 64 or 128"):
         rt.StageExecutor(LayerSpec("bert", 128, 4, 256, 128, 1), 1, 1, 1)
+
+
+@pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
+@pytest.mark.parametrize("spec,sched,n,rank", [(LLAMA, S.Interleaved1F1B(4, 2), 4, 0),
+                                               (MIXTRAL, S.DualPipeV(4, 2), 4, 0)],
+                         ids=["llama-interleaved", "mixtral-dualpipev"])
+def test_rank_row_replays_as_hip_graph(spec, sched, n, rank, two_streams):
+    """The entry points only enqueue, so a rank's row can be recorded into a HIP graph.  Every
+    replay - with eager work and synchronisations between the replays - must reproduce the
+    eager run bit for bit."""
+    plan = make_rank_plan(sched, n, rank)
+    lpc = 1
+    params = make_params(spec, plan.stages, lpc)
+    shape = (spec.tokens, spec.hidden)
+    ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True,
+                          two_streams)
+    for c, stage in enumerate(plan.stages):
+        ex.set_params(c, 0, params[stage][0])
+    bufs = {}
+
+    def io(pt, lane=0):
+        kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
+        key = (kind, pt.task.stage_id, pt.task.mubatch_idx)
+        if key not in bufs:
+            bufs[key] = (rt.DeviceBuffer.from_f32_as_bf16(
+                boundary_tensor(kind, pt.task.stage_id, pt.task.mubatch_idx, shape, 0)),
+                rt.DeviceBuffer(spec.tokens * spec.hidden * 2))
+        return bufs[key][0].ptr, bufs[key][1].ptr
+
+    def results():
+        rt.sync()
+        outs = {k: b[1].download_bf16(shape) for k, b in bufs.items()}
+        grads = [ex.get_grads(c, 0) for c in range(plan.n_chunks)]
+        return outs, grads
+
+    stream = rt.Stream()
+    loop = RankLoop(ex, plan)
+    loop.run(io, stream=stream.ptr)          # eager, also the warm-up the recording needs
+    ex.join(stream.ptr)
+    stream.sync()
+    want_outs, want_grads = results()
+
+    ex.quiesce()
+    graph = rt.Graph(stream)
+    with graph:
+        loop.run(io, stream=stream.ptr)
+        ex.join(stream.ptr)
+    assert ex.live_slots() == 0
+    scratch = rt.DeviceBuffer(1 << 20)
+    for replay in range(3):
+        ex.zero_grads(stream.ptr)            # eager work between the replays
+        for b in bufs.values():
+            rt.check(rt.load().jpp_fill_u32(b[1].ptr, 0x7fc07fc0, spec.tokens * spec.hidden // 2,
+                                            stream.ptr))
+        rt.check(rt.load().jpp_fill_u32(scratch.ptr, replay, 1 << 18, None))
+        stream.sync()
+        graph.launch()
+        stream.sync()
+        outs, grads = results()
+        for k, v in want_outs.items():
+            np.testing.assert_array_equal(outs[k], v, err_msg=f"replay {replay} output {k}")
+        for c in range(plan.n_chunks):
+            for name, v in want_grads[c].items():
+                np.testing.assert_array_equal(grads[c][name], v,
+                                              err_msg=f"replay {replay} grad {c}/{name}")
+    ex.close()
