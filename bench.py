@@ -6,7 +6,8 @@ order the schedule's task table dictates, with synthetic boundary tensors.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3]
 
 A step is one full pass over the rank's row of the task table (all
-microbatches).  Prints one JSON line (see README / DESIGN.md for the fields).
+microbatches).  Prints one JSON line: the metric, its configuration, the roofline of the
+dominant kernel (timed live with HIP events) and a CPU baseline.
 """
 from __future__ import annotations
 
