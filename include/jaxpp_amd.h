@@ -39,7 +39,13 @@ typedef enum {
 /* TaskType of the reference (src/jaxpp/types.py:79-96); same integer values. */
 typedef enum { JPP_FWD = 1, JPP_BWD = 2, JPP_BWD_I = 3, JPP_BWD_W = 4 } jpp_task_kind;
 
-typedef enum { JPP_FAMILY_BERT = 0, JPP_FAMILY_LLAMA = 1, JPP_FAMILY_MIXTRAL = 2 } jpp_family;
+/* Layer families.  BERT: post-LN encoder layer (the README's FlaxBertLayer stack,
+ * README.md:46-72); DECODER: the pre-LN causal block with biases and a GELU feed-forward of
+ * the reference's example model (examples/basic.py:33-91); LLAMA and MIXTRAL: RMSNorm, RoPE,
+ * GQA, SwiGLU / top-2 of 8 experts (the shapes the headline configurations name). */
+typedef enum {
+  JPP_FAMILY_BERT = 0, JPP_FAMILY_LLAMA = 1, JPP_FAMILY_MIXTRAL = 2, JPP_FAMILY_DECODER = 3
+} jpp_family;
 
 const char* jpp_last_error(void);
 int jpp_version(void);

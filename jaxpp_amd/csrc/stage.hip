@@ -57,9 +57,10 @@ struct LayerStash {
   Buf n1, h1, n2, gu, s;
   // mixtral: routing tables and token-permuted expert buffers (gu, s reused, [cap, ..])
   Buf ids, gates, row_of, tok_of, gate_of, seg, xp, eo;
+  // pre-LN decoder block: x, qkv, ctx, lse, mean1, rstd1, n1, h1, mean2, rstd2, n2, u, g
   // cotangents kept for the weight-gradient task
-  Buf dc, du, da, dqkv;   // bert (dqkv shared with llama)
-  Buf dyin, dgu, dh1;     // llama
+  Buf dc, du, da, dqkv;   // bert (dqkv shared with the others, du with the decoder block)
+  Buf dyin, dgu, dh1;     // llama (dyin, dh1 also the decoder block)
   Buf deo, dlogits;       // mixtral
 };
 
@@ -234,6 +235,24 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
               (float*)at(L.mean2), (float*)at(L.rstd2)));
     return JPP_OK;
   }
+  if (s->d.family == JPP_FAMILY_DECODER) {
+    // pre-LN block with biases and a GELU feed-forward; parameters as in the BERT layer
+    RC(norm_f(s, st, at(L.x), s->P(chunk, li, B_ln1g), s->P(chunk, li, B_ln1b), at(L.n1),
+              (float*)at(L.mean1), (float*)at(L.rstd1)));
+    RC(gemm(st, at(L.n1), h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 1, at(L.qkv), 3 * h, T, 3 * h, h,
+            JPP_EPI_BF16, s->P(chunk, li, B_bqkv)));
+    attn_args(s, aa, slot, L);
+    RC(jpp_attn_fwd(st, &aa));
+    RC(gemm(st, at(L.ctx), h, 0, s->P(chunk, li, B_Wo), h, 1, at(L.h1), h, T, h, h, JPP_EPI_BF16,
+            s->P(chunk, li, B_bo), at(L.x), h));
+    RC(norm_f(s, st, at(L.h1), s->P(chunk, li, B_ln2g), s->P(chunk, li, B_ln2b), at(L.n2),
+              (float*)at(L.mean2), (float*)at(L.rstd2)));
+    RC(gemm(st, at(L.n2), h, 0, s->P(chunk, li, B_W1), f, 1, at(L.u), f, T, f, h, JPP_EPI_GELU,
+            s->P(chunk, li, B_b1), nullptr, 0, nullptr, 0, at(L.g), f, s->d.gelu_tanh));
+    RC(gemm(st, at(L.g), f, 0, s->P(chunk, li, B_W2), h, 1, y, h, T, h, f, JPP_EPI_BF16,
+            s->P(chunk, li, B_b2), at(L.h1), h));
+    return JPP_OK;
+  }
   // llama
   RC(norm_f(s, st, at(L.x), s->P(chunk, li, L_rms1), nullptr, at(L.n1), nullptr,
             (float*)at(L.rstd1)));
@@ -312,9 +331,35 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(jpp_colsum_accum(st, dqkv, 3 * h, T, 3 * h, s->G(chunk, li, B_bqkv), partial));
     return JPP_OK;
   }
-  // llama
   void* dn = s->S<>(s->s_t2);   // dn2, later dn1
   void* dctx = s->S<>(s->s_t3);
+  if (s->d.family == JPP_FAMILY_DECODER) {
+    RC(gemm(st, dy, h, 0, s->P(chunk, li, B_W2), h, 0, wt(W.du), f, T, f, h, JPP_EPI_DGELU,
+            nullptr, nullptr, 0, at(L.u), f, nullptr, 0, s->d.gelu_tanh));
+    RC(gemm(st, wt(W.du), f, 0, s->P(chunk, li, B_W1), f, 0, dn, h, T, h, f, JPP_EPI_BF16));
+    RC(norm_b(s, st, dn, at(L.h1), (float*)at(L.mean2), (float*)at(L.rstd2),
+              s->P(chunk, li, B_ln2g), dy, wt(W.dh1), s->G(chunk, li, B_ln2g),
+              s->G(chunk, li, B_ln2b)));
+    RC(gemm(st, wt(W.dh1), h, 0, s->P(chunk, li, B_Wo), h, 0, dctx, h, T, h, h, JPP_EPI_BF16));
+    attn_args(s, aa, slot, L);
+    bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
+    aa.d_o = dctx; aa.lddo = h;
+    aa.dq = dqkv; aa.dk = dqkv + h; aa.dv = dqkv + 2 * h;
+    aa.lddq = aa.lddk = aa.lddv = 3 * h;
+    aa.delta = s->S<float>(s->s_delta);
+    RC(jpp_attn_bwd(st, &aa));
+    RC(gemm(st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dn, h, T, h, 3 * h,
+            JPP_EPI_BF16));
+    RC(norm_b(s, st, dn, at(L.x), (float*)at(L.mean1), (float*)at(L.rstd1),
+              s->P(chunk, li, B_ln1g), wt(W.dh1), dx, s->G(chunk, li, B_ln1g),
+              s->G(chunk, li, B_ln1b)));
+    RC(jpp_colsum_accum(st, dy, h, T, h, s->G(chunk, li, B_b2), partial));
+    RC(jpp_colsum_accum(st, wt(W.du), f, T, f, s->G(chunk, li, B_b1), partial));
+    RC(jpp_colsum_accum(st, wt(W.dh1), h, T, h, s->G(chunk, li, B_bo), partial));
+    RC(jpp_colsum_accum(st, dqkv, 3 * h, T, 3 * h, s->G(chunk, li, B_bqkv), partial));
+    return JPP_OK;
+  }
+  // llama
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
     jpp_moe_args ma;
     moe_args(s, ma, slot, L, chunk, li);
@@ -370,6 +415,13 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(wgrad(s, st, at(L.x), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
     return JPP_OK;
   }
+  if (s->d.family == JPP_FAMILY_DECODER) {
+    RC(wgrad(s, st, at(L.g), f, dy, h, s->G(chunk, li, B_W2), f, h));
+    RC(wgrad(s, st, at(L.n2), h, wt(W.du), f, s->G(chunk, li, B_W1), h, f));
+    RC(wgrad(s, st, at(L.ctx), h, wt(W.dh1), h, s->G(chunk, li, B_Wo), h, h));
+    RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
+    return JPP_OK;
+  }
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
     jpp_moe_args ma;
     moe_args(s, ma, slot, L, chunk, li);
@@ -406,6 +458,14 @@ void carve_layer(jpp_stage* s, Carver& c, LayerStash& L, bool with_w) {
     L.g = c.take(T * f * e);
     L.c = c.take(T * h * e);
     L.mean2 = c.take(T * 4); L.rstd2 = c.take(T * 4);
+  } else if (s->d.family == JPP_FAMILY_DECODER) {
+    L.mean1 = c.take(T * 4); L.rstd1 = c.take(T * 4);
+    L.mean2 = c.take(T * 4); L.rstd2 = c.take(T * 4);
+    L.n1 = c.take(T * h * e);
+    L.h1 = c.take(T * h * e);
+    L.n2 = c.take(T * h * e);
+    L.u = c.take(T * f * e);
+    L.g = c.take(T * f * e);
   } else {
     L.rstd1 = c.take(T * 4); L.rstd2 = c.take(T * 4);
     L.n1 = c.take(T * h * e);
@@ -436,6 +496,10 @@ void carve_w(jpp_stage* s, Carver& c, LayerStash& L) {
     L.dc = c.take(T * h * e);
     L.du = c.take(T * f * e);
     L.da = c.take(T * h * e);
+  } else if (s->d.family == JPP_FAMILY_DECODER) {
+    L.dyin = c.take(T * h * e);
+    L.du = c.take(T * f * e);
+    L.dh1 = c.take(T * h * e);
   } else if (s->d.family == JPP_FAMILY_MIXTRAL) {
     L.dyin = c.take(T * h * e);
     L.dgu = c.take(s->cap * 2 * f * e);
@@ -457,7 +521,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   JPP_REQUIRE(d && out, "stage_create: null");
   *out = nullptr;
   JPP_REQUIRE(d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_LLAMA ||
-                  d->family == JPP_FAMILY_MIXTRAL,
+                  d->family == JPP_FAMILY_MIXTRAL || d->family == JPP_FAMILY_DECODER,
               "stage_create: unknown family %d", d->family);
   if (d->family == JPP_FAMILY_MIXTRAL) {
     JPP_REQUIRE(d->n_experts == 8 && d->top_k == 2,
@@ -482,6 +546,9 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   if (d->family == JPP_FAMILY_BERT)
     JPP_REQUIRE(kvh == d->n_heads && d->n_heads * hd == d->hidden && !d->causal,
                 "stage_create: the BERT layer needs n_heads*head_dim == hidden, no GQA, no mask");
+  if (d->family == JPP_FAMILY_DECODER)
+    JPP_REQUIRE(kvh == d->n_heads && d->n_heads * hd == d->hidden,
+                "stage_create: the decoder block needs n_heads*head_dim == hidden and no GQA");
 
   jpp_stage* s = new jpp_stage();
   s->d = *d;
@@ -496,7 +563,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
     s->pinfo = {{"rms1_g", 1, h}, {"Wqkv", h, s->qkvw}, {"Wo", s->ctxw, h}, {"rms2_g", 1, h},
                 {"Wr", h, d->n_experts}, {"Wgu", d->n_experts * h, 2 * f},
                 {"Wd", d->n_experts * f, h}};
-  else if (d->family == JPP_FAMILY_BERT)
+  else if (d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_DECODER)
     s->pinfo = {{"Wqkv", h, 3 * h}, {"bqkv", 1, 3 * h}, {"Wo", h, h}, {"bo", 1, h},
                 {"ln1_g", 1, h}, {"ln1_b", 1, h}, {"W1", h, f}, {"b1", 1, f},
                 {"W2", f, h}, {"b2", 1, h}, {"ln2_g", 1, h}, {"ln2_b", 1, h}};
@@ -569,7 +636,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   hipMemset(s->params, 0, n_layers * s->layer_elems * 2);
   hipMemset(s->grads, 0, n_layers * s->layer_elems * 4);
 
-  if (d->family != JPP_FAMILY_BERT) {
+  if (d->family == JPP_FAMILY_LLAMA || d->family == JPP_FAMILY_MIXTRAL) {
     // cos/sin of pos * theta^(-2i/d): evaluated in double, stored as f32
     const int half = hd / 2;
     std::vector<float> c((size_t)d->seq * half), sn((size_t)d->seq * half);

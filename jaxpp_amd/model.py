@@ -15,7 +15,7 @@ import numpy as np
 
 @dataclass(frozen=True)
 class LayerSpec:
-    family: str                      # "bert" | "llama" | "mixtral"
+    family: str                      # "bert" | "decoder" | "llama" | "mixtral"
     hidden: int
     n_heads: int
     ffn: int
@@ -51,7 +51,7 @@ class LayerSpec:
 
     def param_shapes(self) -> dict:
         h, f = self.hidden, self.ffn
-        if self.family == "bert":
+        if self.family in ("bert", "decoder"):
             return {"Wqkv": (h, 3 * h), "bqkv": (3 * h,), "Wo": (h, h), "bo": (h,),
                     "ln1_g": (h,), "ln1_b": (h,), "W1": (h, f), "b1": (f,),
                     "W2": (f, h), "b2": (h,), "ln2_g": (h,), "ln2_b": (h,)}
@@ -72,7 +72,7 @@ class LayerSpec:
         qkv = 2.0 * T * h * self.qkv_width
         attn = 4.0 * T * self.seq * self.n_heads * d * (0.5 if self.causal else 1.0)
         out = 2.0 * T * self.n_heads * d * h
-        if self.family == "bert":
+        if self.family in ("bert", "decoder"):
             ffn = 4.0 * T * h * f
         elif self.family == "llama":
             ffn = 6.0 * T * h * f

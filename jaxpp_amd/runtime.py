@@ -85,7 +85,7 @@ class StageDesc(C.Structure):
 
 EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32, EPI_SWIGLU, EPI_DSWIGLU = range(7)
 NORM_PARTIALS = 256
-FAMILY = {"bert": 0, "llama": 1, "mixtral": 2}
+FAMILY = {"bert": 0, "llama": 1, "mixtral": 2, "decoder": 3}
 
 # every symbol include/jaxpp_amd.h declares
 EXPORTS = [

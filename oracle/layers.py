@@ -78,7 +78,7 @@ def identity(x):
 class LayerCfg:
     """Shape of one transformer layer and the conventions it uses."""
 
-    family: str                      # "bert" | "llama" | "mixtral"
+    family: str                      # "bert" | "decoder" | "llama" | "mixtral"
     hidden: int
     n_heads: int
     ffn: int
@@ -112,7 +112,7 @@ class LayerCfg:
 
 def param_shapes(cfg: LayerCfg) -> dict:
     h, f = cfg.hidden, cfg.ffn
-    if cfg.family == "bert":
+    if cfg.family in ("bert", "decoder"):
         return {"Wqkv": (h, 3 * h), "bqkv": (3 * h,), "Wo": (h, h), "bo": (h,),
                 "ln1_g": (h,), "ln1_b": (h,), "W1": (h, f), "b1": (f,),
                 "W2": (f, h), "b2": (h,), "ln2_g": (h,), "ln2_b": (h,)}
@@ -326,6 +326,26 @@ def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics):
         st.update(qkv=qkv, ctx=ctx, lse=lse, a=a, mean1=mean1, rstd1=rstd1, x1=x1,
                   u=u, g=g, c=c, mean2=mean2, rstd2=rstd2)
         return y, st
+    if cfg.family == "decoder":
+        # pre-LN block of the reference's example model (examples/basic.py:72-91): x + attention
+        # of the normalised input, then x + GELU feed-forward of the normalised sum; causal
+        # mask and tanh GELU (jax.nn.gelu's default) are the spec's `causal` / `gelu_tanh`
+        y1, mean1, rstd1 = layernorm_fwd(x, p["ln1_g"], p["ln1_b"], cfg.eps, acc)
+        n1 = rt(y1)
+        qkv = rt(mm(n1, p["Wqkv"], acc) + p["bqkv"].astype(acc))
+        q, k, v = _split_qkv(cfg, qkv)
+        o, lse = attention_fwd(q, k, v, cfg.causal, acc)
+        ctx = rt(o.reshape(T, -1))
+        h1 = rt(mm(ctx, p["Wo"], acc) + p["bo"].astype(acc) + x.astype(acc))
+        y2, mean2, rstd2 = layernorm_fwd(h1, p["ln2_g"], p["ln2_b"], cfg.eps, acc)
+        n2 = rt(y2)
+        u_full = mm(n2, p["W1"], acc) + p["b1"].astype(acc)
+        u = rt(u_full)
+        g = rt(gelu(u_full, cfg.gelu_tanh))
+        y = rt(mm(g, p["W2"], acc) + p["b2"].astype(acc) + h1.astype(acc))
+        st.update(mean1=mean1, rstd1=rstd1, n1=n1, qkv=qkv, ctx=ctx, lse=lse, h1=h1,
+                  mean2=mean2, rstd2=rstd2, n2=n2, u=u, g=g)
+        return y, st
     if cfg.family in ("llama", "mixtral"):
         y1, rstd1 = rmsnorm_fwd(x, p["rms1_g"], cfg.eps, acc)
         n1 = rt(y1)
@@ -381,6 +401,29 @@ def layer_bwd_i(cfg: LayerCfg, p: dict, st: dict, dy, nm: Numerics):
         small["bqkv"] = dqkv.astype(acc).sum(0)
         wst.update(dc=dc, du=du, da=da, dqkv=dqkv)
         return dx, wst, small
+    if cfg.family == "decoder":
+        du = rt(mm(dy, p["W2"].T, acc) * gelu_grad(st["u"].astype(acc), cfg.gelu_tanh))
+        dn2 = rt(mm(du, p["W1"].T, acc))
+        dh1_, small["ln2_g"], small["ln2_b"] = layernorm_bwd(
+            dn2, st["h1"], st["mean2"], st["rstd2"], p["ln2_g"], acc)
+        dh1 = rt(dh1_ + dy.astype(acc))
+        dctx = rt(mm(dh1, p["Wo"].T, acc))
+        q, k, v = _split_qkv(cfg, st["qkv"])
+        B, S, d = cfg.batch, cfg.seq, cfg.d
+        dq, dk, dv = attention_bwd(q, k, v, st["ctx"].reshape(B, S, cfg.n_heads, d),
+                                   dctx.reshape(B, S, cfg.n_heads, d), st["lse"],
+                                   cfg.causal, acc)
+        dqkv = rt(_join_qkv(cfg, dq, dk, dv))
+        dn1 = rt(mm(dqkv, p["Wqkv"].T, acc))
+        dx_, small["ln1_g"], small["ln1_b"] = layernorm_bwd(
+            dn1, st["x"], st["mean1"], st["rstd1"], p["ln1_g"], acc)
+        dx = rt(dx_ + dh1.astype(acc))
+        small["b2"] = dy.astype(acc).sum(0)
+        small["b1"] = du.astype(acc).sum(0)
+        small["bo"] = dh1.astype(acc).sum(0)
+        small["bqkv"] = dqkv.astype(acc).sum(0)
+        wst.update(dy=dy, du=du, dh1=dh1, dqkv=dqkv)
+        return dx, wst, small
     if cfg.family in ("llama", "mixtral"):
         if cfg.family == "llama":
             ds = rt(mm(dy, p["Wd"].T, acc))
@@ -416,6 +459,9 @@ def layer_bwd_w(cfg: LayerCfg, st: dict, wst: dict, nm: Numerics):
     if cfg.family == "bert":
         return {"W2": mm(st["g"].T, wst["dc"], acc), "W1": mm(st["x1"].T, wst["du"], acc),
                 "Wo": mm(st["ctx"].T, wst["da"], acc), "Wqkv": mm(st["x"].T, wst["dqkv"], acc)}
+    if cfg.family == "decoder":
+        return {"W2": mm(st["g"].T, wst["dy"], acc), "W1": mm(st["n2"].T, wst["du"], acc),
+                "Wo": mm(st["ctx"].T, wst["dh1"], acc), "Wqkv": mm(st["n1"].T, wst["dqkv"], acc)}
     if cfg.family == "llama":
         return {"Wd": mm(st["s"].T, wst["dy"], acc), "Wgu": mm(st["n2"].T, wst["dgu"], acc),
                 "Wo": mm(st["ctx"].T, wst["dh1"], acc), "Wqkv": mm(st["n1"].T, wst["dqkv"], acc)}

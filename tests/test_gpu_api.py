@@ -68,3 +68,42 @@ def test_train_step_matches_oracle_pipeline(schedule, n_mb, mpmd):
     np.testing.assert_array_equal(losses, losses2)
     np.testing.assert_array_equal(grad["layers"][0]["Wqkv"], grad2["layers"][0]["Wqkv"])
     pp_train_step.close()
+
+
+def test_example_model_train_step():
+    """The reference's example (examples/basic.py): a stack of pre-LN causal decoder blocks with
+    a stage marker after every `num_layers // pp` layers, loss mean((res - batch)**2) /
+    num_ubatches, Std1F1B over 2 stages - here 4 blocks of hidden 256 in two stages."""
+    rt.require_gpu()
+    spec = LayerSpec("decoder", 256, 2, 512, 128, 1, causal=True, eps=1e-6, gelu_tanh=True)
+    n_mb, pp, n_layers = 4, 2, 4
+    schedule = jaxpp.Std1F1B(pp)
+    model = jaxpp.nn.TransformerStack(spec, n_layers=n_layers, layers_per_stage=n_layers // pp)
+    params = model.init(seed=0, perturb=True)
+    params = {"layers": [{k: L.bf16_round(v) for k, v in p.items()} for p in params["layers"]]}
+    rng = np.random.default_rng(2)
+    batch = L.bf16_round(rng.uniform(size=(n_mb, spec.tokens, spec.hidden)).astype(np.float32))
+    mesh = jaxpp.MpmdMesh(jaxpp.DeviceMesh(np.arange(pp).reshape(pp, 1), ("mpmd", "data")), "mpmd")
+
+    def loss_fn(pars, mb):
+        res = model.apply(pars, mb)
+        return jaxpp.nn.mse_loss(res, mb) / n_mb, (res, 4)
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=mesh)
+    def train_step(pars, batch):
+        mubatch_grad = partial(jaxpp.value_and_grad(loss_fn, has_aux=True), pars)
+        (losses, (pred, _)), grad = jaxpp.treduce(mubatch_grad, batch, schedule=schedule)
+        return losses, pred, grad
+
+    losses, pred, grad = train_step(params, batch)
+    cfg = L.LayerCfg(**spec.as_dict())
+    per = n_layers // pp
+    stages = [params["layers"][s * per:(s + 1) * per] for s in range(pp)]
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16())
+    close(losses, want_loss, "losses")
+    for s in range(pp):
+        for li in range(per):
+            for k, v in want_acc[s][li].items():
+                got = grad["layers"][s * per + li][k]
+                close(got, v.reshape(got.shape), f"grad {s}/{li}/{k}")
+    train_step.close()

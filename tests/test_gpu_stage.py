@@ -24,6 +24,8 @@ LLAMA = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, caus
                   rope_theta=5e5, eps=1e-5)
 MIXTRAL = LayerSpec("mixtral", 256, 2, 256, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
                     rope_theta=5e5, eps=1e-5, n_experts=8, top_k=2)
+DECODER = LayerSpec("decoder", 256, 2, 512, 128, 2, causal=True, eps=1e-6, gelu_tanh=True)
+DECODER_D64 = LayerSpec("decoder", 128, 2, 256, 256, 1, eps=1e-5)
 LLAMA_D64 = LayerSpec("llama", 256, 4, 256, 256, 1, n_kv_heads=2, head_dim=64, causal=True,
                       rope_theta=1e4, eps=1e-5)
 
@@ -106,6 +108,9 @@ def make_params(spec, stages, layers_per_chunk):
 CASES = [
     ("bert-1f1b", BERT, S.Std1F1B(2), 4, 0, 2),
     ("bert-tanh-zb", BERT_TANH, S.ZeroBubble(2), 3, 1, 1),
+    ("decoder-1f1b", DECODER, S.Std1F1B(2), 3, 1, 2),
+    ("decoder-zb", DECODER, S.ZeroBubble(2), 3, 1, 1),
+    ("decoder-d64-zb-first-stage", DECODER_D64, S.ZeroBubble(2), 2, 0, 2),
     ("llama-interleaved", LLAMA, S.Interleaved1F1B(4, 2), 4, 0, 2),
     ("llama-zb-first-stage", LLAMA, S.ZeroBubble(2), 2, 0, 1),
     ("llama-d64-zb", LLAMA_D64, S.ZeroBubble(3), 3, 1, 2),

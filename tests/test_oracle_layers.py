@@ -16,6 +16,9 @@ torch.set_num_threads(4)
 SPECS = {
     "bert": LayerSpec("bert", 32, 4, 64, 8, 2, eps=1e-12),
     "bert_tanh": LayerSpec("bert", 32, 4, 64, 8, 2, eps=1e-6, gelu_tanh=True),
+    # the block of the reference's example model: pre-LN, causal, tanh GELU
+    "decoder": LayerSpec("decoder", 32, 4, 64, 8, 2, causal=True, eps=1e-6, gelu_tanh=True),
+    "decoder_nomask": LayerSpec("decoder", 32, 2, 48, 6, 1, eps=1e-5),
     "llama": LayerSpec("llama", 32, 4, 48, 8, 2, n_kv_heads=2, head_dim=8, causal=True,
                        rope_theta=1e4, eps=1e-5),
     "llama_mha": LayerSpec("llama", 32, 4, 48, 6, 1, n_kv_heads=4, head_dim=8, causal=True,
@@ -62,6 +65,16 @@ def torch_layer(spec, p, x):
                                      approximate="tanh" if spec.gelu_tanh else "none")
         c = g @ p["W2"] + p["b2"] + x1
         return torch.nn.functional.layer_norm(c, (h,), p["ln2_g"], p["ln2_b"], spec.eps)
+
+    if spec.family == "decoder":
+        # written after the data flow of examples/basic.py:72-91 (DecoderBlock.__call__)
+        approx = "tanh" if spec.gelu_tanh else "none"
+        attn_in = torch.nn.functional.layer_norm(x, (h,), p["ln1_g"], p["ln1_b"], spec.eps)
+        q, k, v = (attn_in @ p["Wqkv"] + p["bqkv"]).split(h, -1)
+        x = x + attn(q, k, v) @ p["Wo"] + p["bo"]
+        ffn_in = torch.nn.functional.layer_norm(x, (h,), p["ln2_g"], p["ln2_b"], spec.eps)
+        ffn = torch.nn.functional.gelu(ffn_in @ p["W1"] + p["b1"], approximate=approx)
+        return x + ffn @ p["W2"] + p["b2"]
 
     def rms(t, g):
         return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + spec.eps) * g
@@ -117,7 +130,7 @@ def test_layer_matches_torch_autograd(name):
                                    err_msg=k)
 
 
-@pytest.mark.parametrize("name", ["bert", "llama", "mixtral"])
+@pytest.mark.parametrize("name", ["bert", "decoder", "llama", "mixtral"])
 def test_layer_finite_differences(name):
     spec = SPECS[name]
     cfg = cfg_of(spec)
