@@ -144,7 +144,8 @@ typedef struct {
   int epilogue;      /* jpp_epilogue */
   int gelu_tanh;     /* 0: erf form, 1: tanh approximation */
   int tile;          /* 0: choose (may run the last, half-empty round of 256x256 tiles as a second
-                        launch of 256x128 tiles); 1: 128x128; 2: 256x128; 4: 256x256 (8 waves each) */
+                        launch of 128x256 tiles); 1: 128x128; 2: 256x128; 3: 128x256; 4: 256x256
+                        (8 waves each) */
   /* grouped GEMM over experts (0 = plain).  seg: device int32 [n_seg + 1], row
    * offsets of the expert groups in the token-permuted buffers, multiples of 256.
    *   JPP_GROUP_M: rows of A and C are grouped; group e multiplies b + e * stride_b.

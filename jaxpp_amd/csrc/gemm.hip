@@ -493,6 +493,8 @@ int launch_tiled(hipStream_t stream, GemmParams& p, int tile) {
   switch (tile) {
     case 2:  // 8 waves of 128x32; three stages where the accumulator rows leave room
       return launch<256, 128, TA, TB, EPI, 8, EPI == JPP_EPI_ACC_F32 ? 2 : 3>(stream, p);
+    case 3:  // 8 waves of 64x64
+      return launch<128, 256, TA, TB, EPI, 8, EPI == JPP_EPI_ACC_F32 ? 2 : 3>(stream, p);
     case 4: return launch<256, 256, TA, TB, EPI, 8>(stream, p);
     default:
       // 128x128: 8 waves (64x32 each); the SwiGLU epilogues, which no measured workload
@@ -614,12 +616,12 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
   if (a->group_mode != JPP_GROUP_NONE) tile = 4;  // 256-row segments
-  JPP_REQUIRE(tile == 1 || tile == 2 || tile == 4, "gemm: unknown tile %d", tile);
-  if (tile >= 2 && a->m % 256) tile = 1;
-  if (tile == 4 && a->n % 256) tile = 2;
+  JPP_REQUIRE(tile >= 1 && tile <= 4, "gemm: unknown tile %d", tile);
+  if ((tile == 2 || tile == 4) && a->m % 256) tile = a->n % 256 ? 1 : 3;
+  if ((tile == 3 || tile == 4) && a->n % 256) tile = a->m % 256 ? 1 : 2;
 
   // A grid of 256x256 tiles whose last round fills at most half of the 256 CUs runs that
-  // round as a separate launch of 256x128 tiles over the last rows or columns: a full round
+  // round as a separate launch of 128x256 tiles over the last rows or columns: a full round
   // of half-size tiles takes little more than half the time the half-empty round did.
   // (Only when the choice of tile was left to the library.)
   if (tile == 4 && a->tile == 0 && a->group_mode == JPP_GROUP_NONE) {
@@ -639,7 +641,7 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
           shift_origin(tail, a->trans_a != 0, a->trans_b != 0, a->epilogue, 0, head.n);
         }
         const int rc = dispatch(stream, a, head, 4);
-        return rc != JPP_OK ? rc : dispatch(stream, a, tail, 2);
+        return rc != JPP_OK ? rc : dispatch(stream, a, tail, 3);
       }
     }
   }

@@ -45,7 +45,9 @@ FULL = [
     ("tn", 14336, 4096, 4096, rt.EPI_ACC_F32, 0),
     ("tn", 1024, 1024, 4096, rt.EPI_ACC_F32, 1),    # 128x128, 3 LDS stages
     ("nn", 1024, 1024, 4096, rt.EPI_F32, 1),        # 128x128, 4 LDS stages
-    ("nt", 2048, 1024, 4096, rt.EPI_BF16, 2),       # 256x128 on 4 waves
+    ("nt", 2048, 1024, 4096, rt.EPI_BF16, 2),       # 256x128
+    ("tn", 1024, 2048, 4096, rt.EPI_ACC_F32, 3),    # 128x256, streamed accumulator
+    ("nn", 1152, 2048, 4096, rt.EPI_F32, 3),
 ]
 
 

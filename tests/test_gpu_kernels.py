@@ -54,9 +54,10 @@ GEMM_CASES = [  # (trans_a, trans_b, epilogue)
 
 @pytest.mark.parametrize("ta,tb,epi", GEMM_CASES)
 @pytest.mark.parametrize("tile,m,n,k", [(1, 128, 384, 192), (2, 512, 128, 64), (4, 256, 512, 320), (4, 512, 256, 192),
+                                        (3, 384, 512, 192),
                                         (0, 768, 256, 128),
                                         # 384 tiles of 256x256: the half-filled second round runs as
-                                        # a launch of 256x128 tiles over the last columns / rows
+                                        # a launch of 128x256 tiles over the last columns / rows
                                         (0, 4096, 6144, 128), (0, 6144, 4096, 192)])
 def test_gemm(ta, tb, epi, tile, m, n, k):
     print(f"gemm ta={ta} tb={tb} epi={epi} tile={tile} {m}x{n}x{k}", flush=True)
@@ -387,7 +388,8 @@ def test_grouped_gemm():
 
 
 @pytest.mark.parametrize("tile,m,f,k", [(1, 128, 128, 64), (2, 256, 256, 128), (4, 512, 256, 192),
-                                        # split into 256x256 + 256x128 launches: the forward at
+                                        (3, 384, 256, 128),
+                                        # split into 256x256 + 128x256 launches: the forward at
                                         # f = 3072 (N = 6144), the backward at f = 6144
                                         (0, 4096, 3072, 128), (0, 4096, 6144, 64)])
 def test_gemm_swiglu_epilogues(tile, m, f, k):
