@@ -172,8 +172,8 @@ def main():
     ap.add_argument("--two-streams", choices=["auto", "on", "off"], default="auto",
                     help="weight gradients on the stage's second stream and the forward of a "
                          "fused entry beside its backward.  auto: on when the layers are too "
-                         "narrow for one kernel to fill the chip (hidden < 2048: +20%% at cfg2), off "
-                         "otherwise (+1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
+                         "narrow for one kernel to fill the chip (hidden < 2048: +7%% at cfg2), off "
+                         "otherwise (-1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
                          "include the other stream's kernels)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
     ap.add_argument("--graph", action="store_true",
