@@ -121,6 +121,10 @@ def test_gemm_rejects_bad_shapes():
 @pytest.mark.parametrize("d,causal,hq,hkv,batch,seq", [
     (64, 0, 4, 4, 2, 256), (64, 1, 2, 2, 1, 384), (128, 1, 8, 2, 1, 512),
     (128, 0, 2, 1, 2, 128), (128, 1, 4, 4, 1, 256),
+    # shortest causal sequence with grouped heads; an odd number of 128-query blocks; head
+    # counts that switch on the per-XCD work order (8 kv heads); the BERT-large head shape
+    (128, 1, 4, 1, 2, 128), (64, 1, 8, 2, 2, 640), (128, 1, 32, 8, 1, 512), (64, 0, 16, 16, 2, 512),
+    (64, 1, 16, 8, 1, 1024),
 ])
 def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
     print(f"attention d={d} causal={causal} hq={hq} hkv={hkv} b={batch} s={seq}", flush=True)
