@@ -158,6 +158,9 @@ typedef struct {
   int64_t stride_b, stride_c;
   int64_t group_rows; /* non-padding rows over all groups, for the probe's FLOP and byte
                        * accounting only (0: the padded extent is counted) */
+  const int32_t* seg_rows; /* device int32 [n_seg] or NULL: rows of each group that hold data;
+                            * the rest of a group is zero padding, which JPP_GROUP_K then leaves
+                            * out of the contraction (whole 64-row steps of it) */
 } jpp_gemm_args;
 
 enum { JPP_GROUP_NONE = 0, JPP_GROUP_M = 1, JPP_GROUP_K = 2 };
@@ -267,7 +270,8 @@ typedef struct {
   int32_t* row_of;   /* [tokens, 2] row of each assignment */
   int32_t* tok_of;   /* [capacity] token of each row, -1 for padding */
   float* gate_of;    /* [capacity] gate of each row */
-  int32_t* seg;      /* [n_experts + 1] */
+  int32_t* seg;      /* [2 n_experts + 1]: first row of each group and the end of the last,
+                        then the number of rows of each group that hold tokens */
   void* work;        /* int32 [2 * ceil(tokens / 256) * n_experts] scratch */
   int64_t tokens, hidden;
   int n_experts, top_k; /* 8, 2 */

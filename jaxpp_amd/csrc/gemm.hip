@@ -36,6 +36,7 @@ struct GemmParams {
   int tiles_m, tiles_n;
   // grouped (mixture-of-experts) problems: seg[0..n_seg] are row offsets, multiples of 256
   const int* seg;
+  const int* seg_rows;
   int n_seg, group_mode;
   int64_t group_rows;
   long stride_b, stride_c;
@@ -116,7 +117,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     // one output per expert; the contraction runs over the expert's rows
     const int e = blockIdx.x / tiles;
     const long r0 = p.seg[e];
-    kt_n = (p.seg[e + 1] - p.seg[e]) / 64;
+    // rows past the group's data are zero padding: steps made of nothing else are skipped
+    const int rows = p.seg_rows ? min(p.seg_rows[e], p.seg[e + 1] - p.seg[e]) : p.seg[e + 1] - p.seg[e];
+    kt_n = (rows + 63) / 64;
     a_src += r0 * p.lda;
     b_src += r0 * p.ldb;
     p.c = EPI == JPP_EPI_BF16 ? (void*)((bf16_t*)p.c + (long)e * p.stride_c)
@@ -126,9 +129,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   const long a_step = TA ? 64 * p.lda : 64;
   const long b_step = TB ? 64 * p.ldb : 64;
 
-  // lane holds, of tile (i, j), m = m_lane + 16 i and the four columns n_lane + 16 j + {0..3}
-  const long m_lane = m0 + wm * (BM / 2) + (lane & 15);
-  const long n_lane = n0 + wn * (BN / WN) + (lane >> 4) * 4;
+  // of tile (i, j) a lane holds row wm BM/2 + 16 i + lane % 16 and the four columns
+  // wn BN/WN + 16 j + 4 (lane / 16) + {0..3}
   f32x4 acc[TM][TN];
   // C += A B (EPI_ACC_F32): the epilogue only stores; the fp32 tile in memory is folded into
   // the accumulators during the first K-steps.  It travels HBM -> LDS like the operands, NW
@@ -137,8 +139,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   // operand copies, and read out of LDS at the wait point of K-step b+NS.  The waits in
   // between leave the youngest requests in flight (vmcnt counts in order), so a batch has
   // NS K-steps to arrive and no K-step waits for HBM on its account; reading whole rows
-  // keeps HBM on long bursts where a lane-per-row layout would touch 32 rows at once.  K
-  // loops too short for that read the tile into the accumulators up front.
+  // keeps HBM on long bursts where a lane-per-row layout would touch 16 rows at once.  K
+  // loops too short for that add the old values in the epilogue, where rows are whole too.
   static_assert(BN * 4 <= 1024, "a row of the fp32 tile is one 64-lane copy");
   constexpr int NBT = BM / NW, C_LDS = NS * (BM + BN) * 128, C_PITCH = 1024 + 16;  // a copy is 1 KB
   const bool stream_c = EPI == JPP_EPI_ACC_F32 && kt_n >= NBT + NS;
@@ -146,16 +148,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  if constexpr (EPI == JPP_EPI_ACC_F32) {
-    if (!stream_c) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = *(const f32x4*)((const float*)p.c + (m_lane + i * 16) * p.ldc + n_lane +
-                                      j * 16);
-    }
-  }
   // byte offset, from the start of C, of this lane's 16 bytes of tile row `wave`
   // (lanes past the end of a narrow row repeat its last piece)
   const uint32_t c_off0 =
@@ -190,14 +182,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
                                    wave);
     }
     dma_wait<(NS - 1) * OPB>();  // stage 0 has landed; the others may still be in flight
-  }
-  if constexpr (EPI == JPP_EPI_ACC_F32) {
-    // the compiler waits for up-front reads of C here, not at their first use inside the K
-    // loop (where its wait would also cover the operand copies in flight)
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(acc[i][j]));
   }
   __syncthreads();
 #pragma unroll
@@ -329,9 +313,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
       __syncthreads();
       const long mrow0 = m0 + half * (BM / 2) + i0 * 16;
       const int c4 = (tid % TPR) * 4;
-      for (int r = tid / TPR; r < RP; r += RPI)
-        *(float4*)((float*)p.c + (mrow0 + r) * p.ldc + n0 + c4) =
-            *(const float4*)(smem + r * PITCH + c4 * 4);
+      static_assert(RP % RPI == 0, "rows of a pass split evenly over the threads");
+      float4 v[RP / RPI];
+      if (EPI == JPP_EPI_ACC_F32 && !stream_c) {
+        // a K loop too short to stream the old values in: they are read here, by rows, all of
+        // a thread's rows before the first is used
+        float4 old[RP / RPI];
+#pragma unroll
+        for (int it = 0; it < RP / RPI; ++it)
+          old[it] = *(const float4*)((const float*)p.c + (mrow0 + tid / TPR + it * RPI) * p.ldc +
+                                     n0 + c4);
+#pragma unroll
+        for (int it = 0; it < RP / RPI; ++it) {
+          const float4 t = *(const float4*)(smem + (tid / TPR + it * RPI) * PITCH + c4 * 4);
+          v[it] = make_float4(old[it].x + t.x, old[it].y + t.y, old[it].z + t.z, old[it].w + t.w);
+        }
+      } else {
+#pragma unroll
+        for (int it = 0; it < RP / RPI; ++it)
+          v[it] = *(const float4*)(smem + (tid / TPR + it * RPI) * PITCH + c4 * 4);
+      }
+#pragma unroll
+      for (int it = 0; it < RP / RPI; ++it)
+        *(float4*)((float*)p.c + (mrow0 + tid / TPR + it * RPI) * p.ldc + n0 + c4) = v[it];
     }
   } else {
     // bf16 outputs.  An accumulator lane holds one row and 4 consecutive columns, so storing
@@ -588,7 +592,7 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   p.lda = a->lda; p.ldb = a->ldb; p.ldc = a->ldc;
   p.ldc2 = a->ldc2; p.ldresid = a->ldresid; p.ldaux = a->ldaux;
   p.gelu_tanh = a->gelu_tanh;
-  p.seg = a->seg; p.n_seg = a->n_seg; p.group_mode = a->group_mode;
+  p.seg = a->seg; p.seg_rows = a->seg_rows; p.n_seg = a->n_seg; p.group_mode = a->group_mode;
   p.group_rows = a->group_rows;
   p.stride_b = a->stride_b; p.stride_c = a->stride_c;
   if (a->group_mode != JPP_GROUP_NONE) {

@@ -70,8 +70,8 @@ __global__ __launch_bounds__(256) void count_kernel(const int* __restrict__ ids,
   if (threadIdx.x < kE) cnt[blockIdx.x * kE + threadIdx.x] = hist[threadIdx.x];
 }
 
-// seg[e]: first row of expert e (multiple of 256); base[blk][e]: first row of
-// the block's assignments to e.  One thread per expert.
+// seg[e]: first row of expert e (multiple of 256), seg[kE + 1 + e]: its number of tokens;
+// base[blk][e]: first row of the block's assignments to e.  One thread per expert.
 __global__ void scan_kernel(const int* __restrict__ cnt, int nblk, int* __restrict__ seg,
                             int* __restrict__ base) {
   __shared__ int total[kE];
@@ -92,6 +92,7 @@ __global__ void scan_kernel(const int* __restrict__ cnt, int nblk, int* __restri
       at += (total[i] + kPad - 1) / kPad * kPad;
     }
     seg[kE] = at;
+    for (int i = 0; i < kE; ++i) seg[kE + 1 + i] = total[i];
   }
   __syncthreads();
   if (e < kE)

@@ -129,6 +129,7 @@ int ggemm(hipStream_t st, int mode, const int* seg, int n_seg, const void* a, in
   g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.trans_a = ta; g.trans_b = tb; g.epilogue = epi;
   g.seg = seg; g.n_seg = n_seg; g.group_mode = mode; g.stride_b = stride_b; g.stride_c = stride_c;
   g.group_rows = rows;
+  g.seg_rows = seg + n_seg + 1;   // the routing kernels leave the token counts behind the offsets
   g.aux = aux; g.ldaux = ldaux; g.c2 = c2; g.ldc2 = ldc2;
   return jpp_gemm_bf16(st, &g);
 }

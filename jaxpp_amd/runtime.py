@@ -36,7 +36,8 @@ class GemmArgs(C.Structure):
                 ("trans_a", C.c_int), ("trans_b", C.c_int), ("epilogue", C.c_int),
                 ("gelu_tanh", C.c_int), ("tile", C.c_int),
                 ("seg", C.c_void_p), ("n_seg", C.c_int), ("group_mode", C.c_int),
-                ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("group_rows", C.c_int64)]
+                ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("group_rows", C.c_int64),
+                ("seg_rows", C.c_void_p)]
 
 
 class AttnArgs(C.Structure):
@@ -413,10 +414,11 @@ class probe:
 # ---------------------------------------------------------------------------
 def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, bias=None,
          resid=None, ldresid=0, aux=None, ldaux=0, c2=None, ldc2=0, gelu_tanh=0, tile=0,
-         stream=None, seg=None, n_seg=0, group_mode=0, stride_b=0, stride_c=0, group_rows=0):
+         stream=None, seg=None, n_seg=0, group_mode=0, stride_b=0, stride_c=0, group_rows=0,
+         seg_rows=None):
     g = GemmArgs(a, b, c, c2, bias, resid, aux, m, n, k, lda, ldb, ldc, ldc2, ldresid, ldaux,
                  int(trans_a), int(trans_b), epilogue, gelu_tanh, tile, seg, n_seg, group_mode,
-                 stride_b, stride_c, group_rows)
+                 stride_b, stride_c, group_rows, seg_rows)
     check(load().jpp_gemm_bf16(stream, C.byref(g)))
 
 

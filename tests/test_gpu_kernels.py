@@ -301,7 +301,9 @@ def test_moe_routing_and_permutation():
         assert min(top3[0] - top3[1], top3[1] - top3[2]) < 1e-4, (t, top3)
     same = np.setdiff1d(np.arange(T), diff)
     np.testing.assert_allclose(gates[same], gates_w[same], rtol=1e-4, atol=1e-6)
-    seg = b["seg"].download(np.int32, (E + 1,))
+    seg_all = b["seg"].download(np.int32, (2 * E + 1,))
+    seg, seg_rows = seg_all[:E + 1], seg_all[E + 1:]
+    np.testing.assert_array_equal(seg_rows, [(ids == e).any(1).sum() for e in range(E)])
     row_of = b["row_of"].download(np.int32, (T, 2))
     tok_of = b["tok_of"].download(np.int32, (cap,))
     gate_of = b["gate_of"].download(np.float32, (cap,))
@@ -389,6 +391,17 @@ def test_grouped_gemm():
         want = acc0[e] + xp[seg[e]:seg[e + 1]].T @ dy[seg[e]:seg[e + 1]]
         close(got[e], want, 1e-3, f"dW group {e}")
     np.testing.assert_array_equal(got[1], acc0[1])       # empty group: untouched
+    # with the groups' row counts, steps of the contraction that hold only padding are left out
+    b_acc2, b_rows = rt.DeviceBuffer.from_numpy(acc0), rt.DeviceBuffer.from_numpy(
+        np.array(counts, np.int32))
+    rt.gemm(b_xp.ptr, b_dy.ptr, b_acc2.ptr, h, f, 0, h, f, f, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
+            n_seg=E, group_mode=2, stride_c=h * f, seg_rows=b_rows.ptr)
+    rt.sync()
+    got2 = b_acc2.download(np.float32, (E, h, f))
+    for e in range(E):
+        want = acc0[e] + xp[seg[e]:seg[e + 1]].T @ dy[seg[e]:seg[e + 1]]
+        close(got2[e], want, 1e-3, f"dW group {e}, padding steps skipped")
+    np.testing.assert_array_equal(got2[1], acc0[1])
 
 
 @pytest.mark.parametrize("tile,m,f,k", [(1, 128, 128, 64), (2, 256, 256, 128), (4, 512, 256, 192),
