@@ -378,6 +378,14 @@ def test_grouped_gemm():
         if counts[e]:
             close(got[seg[e]:seg[e + 1]], xp[seg[e]:seg[e + 1]] @ w[e], 1e-2, f"group {e}")
     assert not got[seg[E]:].any(), "tiles past the last group must not be written"
+    # row counts change nothing for row-grouped products: same bits
+    b_rows = rt.DeviceBuffer.from_numpy(np.array(counts, np.int32))
+    out2 = rt.DeviceBuffer(cap * f * 2)
+    out2.zero()
+    rt.gemm(b_xp.ptr, b_w.ptr, out2.ptr, cap, f, h, h, f, f, 0, 1, rt.EPI_BF16, seg=b_seg.ptr, n_seg=E,
+            group_mode=1, stride_b=h * f, seg_rows=b_rows.ptr)
+    rt.sync()
+    np.testing.assert_array_equal(out2.download_bf16((cap, f)), got)
     # weight gradients: per-expert contraction over the expert's rows, accumulated
     dy = np.zeros((cap, f), np.float32)
     dy[:seg[E]] = rnd(rng, int(seg[E]), f)
@@ -392,8 +400,7 @@ def test_grouped_gemm():
         close(got[e], want, 1e-3, f"dW group {e}")
     np.testing.assert_array_equal(got[1], acc0[1])       # empty group: untouched
     # with the groups' row counts, steps of the contraction that hold only padding are left out
-    b_acc2, b_rows = rt.DeviceBuffer.from_numpy(acc0), rt.DeviceBuffer.from_numpy(
-        np.array(counts, np.int32))
+    b_acc2 = rt.DeviceBuffer.from_numpy(acc0)
     rt.gemm(b_xp.ptr, b_dy.ptr, b_acc2.ptr, h, f, 0, h, f, f, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
             n_seg=E, group_mode=2, stride_c=h * f, seg_rows=b_rows.ptr)
     rt.sync()
