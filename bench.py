@@ -112,7 +112,7 @@ class Workbench:
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size)
-MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.009e9}
+MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.005e9}
 
 
 def dominant_gemm_class(wl) -> str:
