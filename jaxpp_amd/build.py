@@ -14,11 +14,18 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libjaxpp_amd.so")
-SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "elementwise.hip", "moe.hip", "optimizer.hip", "diagnostics.hip",
-           "stage.hip"]
+SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "attention_dkv.hip", "elementwise.hip",
+           "moe.hip", "optimizer.hip", "diagnostics.hip", "stage.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          # packed fp32 ops are kept out of generated code on this hardware pool
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+# Per-file additions.  The causal dK/dV attention kernel runs one wave per SIMD and depends on
+# the order of its own instructions; LLVM's iterative ILP scheduler orders it 9 % faster than
+# the default (measured on MI355X).  If a compiler does not know the option the file is built
+# without it.
+EXTRA_FLAGS = {"attention_dkv.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"]}
 
 
 def _hipcc() -> str:
@@ -43,7 +50,18 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
 
     def compile_one(src):
         obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
-        _run([hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        extra = EXTRA_FLAGS.get(src)
+        if extra:
+            try:
+                _run(cmd[:1] + extra + cmd[1:])
+            except RuntimeError:
+                if verbose:
+                    print(f"[jaxpp_amd.build] {src}: {' '.join(extra)} not accepted, "
+                          "building without", flush=True)
+                _run(cmd)
+        else:
+            _run(cmd)
         if verbose:
             print(f"[jaxpp_amd.build] compiled {src}", flush=True)
         return obj

@@ -1,0 +1,103 @@
+// Pieces shared by the attention kernels: parameters, fragment helpers, the HBM -> LDS tile
+// copy and the per-XCD work order.
+#ifndef JAXPP_AMD_ATTENTION_COMMON_H_
+#define JAXPP_AMD_ATTENTION_COMMON_H_
+
+#include <math.h>
+
+#include "common.h"
+
+namespace jpp_attn {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct AttnParams {
+  const bf16_t* q; const bf16_t* k; const bf16_t* v;
+  bf16_t* o; float* lse;
+  const bf16_t* d_o;
+  bf16_t* dq; bf16_t* dk; bf16_t* dv;
+  float* delta;
+  long ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv;
+  int batch, seq, n_heads, n_kv_heads;
+  float scale;
+};
+
+// 8 consecutive accumulator registers -> one bf16 MFMA operand
+__device__ __forceinline__ bf16x8 acc_to_frag(const f32x16& a, int base) {
+  bf16x8 f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (__bf16)a[base + e];
+  return f;
+}
+
+// row-major operand fragment straight from HBM (lane: row = lane&31, 8
+// contraction elements of step ks)
+__device__ __forceinline__ bf16x8 global_frag(const bf16_t* base, long ld, int ks, int lane) {
+  return *(const bf16x8*)(base + (long)(lane & 31) * ld + ks * 16 + (lane >> 5) * 8);
+}
+
+// a [64][D] tile lives in LDS as D/64 slabs of [64][64]
+template <int D>
+__device__ __forceinline__ bf16x8 slabs_frag(const uint8_t* slabs, int row0, int ks, int lane) {
+  return slab_frag(slabs + (ks >> 2) * 8192, row0, ks & 3, lane);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Makes the compiler wait here for the loads that produce these registers.  Without it the
+// wait lands at their first use inside the main loop as a vmcnt count, and there it also
+// waits for the HBM -> LDS copies of the next tile, which the wave has just issued (vmcnt
+// counts every vector memory operation of the wave, in order).
+template <int N>
+__device__ __forceinline__ void settle(bf16x8 (&f)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i]));
+}
+__device__ __forceinline__ void settle(float& x) { asm volatile("" : "+v"(x)); }
+
+// HBM -> LDS copy of a [64][D] tile (row stride ld) by the 4 waves of a
+// workgroup, as D/64 swizzled slabs; no registers involved.
+using Tile64 = DmaTile<64, false>;
+template <int D>
+__device__ __forceinline__ void dma_tile(const bf16_t* src, const Tile64::Offsets& off,
+                                         uint32_t lds, int wave) {
+#pragma unroll
+  for (int c = 0; c < D / 64; ++c)
+    Tile64::issue<0, Tile64::INSTS>(uniform_ptr(src + c * 64), off, lds + c * 8192, wave);
+}
+
+// Which (block, head, batch) a workgroup works on.  Workgroups are handed to the 8 XCDs
+// round robin in launch order, and each XCD has its own L2: the launch order is rearranged
+// so that one XCD sees only 1/8 of the (head, batch) pairs - adjacent heads, which share
+// their K/V under grouped-query attention - and its K/V working set stays in its L2.
+// Within an XCD blocks still go out in increasing x for all its heads (heavy first).
+struct Work { int x, h, b; };
+__device__ __forceinline__ Work xcd_work() {
+  const int gx = gridDim.x, gy = gridDim.y;
+  const int pairs = gy * gridDim.z;
+  int x = blockIdx.x, pair = blockIdx.y + gy * blockIdx.z;
+  if ((pairs & 7) == 0) {
+    const int l = x + gx * pair, per = pairs >> 3;
+    const int xcd = l & 7, j = l >> 3;
+    x = j / per;
+    pair = xcd * per + j % per;
+  }
+  return {x, pair % gy, pair / gy};
+}
+
+// sets the kernel's dynamic LDS limit (sticky per kernel)
+template <class K>
+int set_smem(K kern, int bytes) {
+  JPP_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    bytes));
+  return JPP_OK;
+}
+
+// dK/dV under a causal mask (attention_dkv.hip, a translation unit of its own: it is built
+// with another instruction scheduler than the other kernels); grid (seq/128, kv heads, batch)
+int launch_dkv_causal(hipStream_t stream, const AttnParams& p, int head_dim, dim3 grid);
+
+}  // namespace jpp_attn
+
+#endif  // JAXPP_AMD_ATTENTION_COMMON_H_
