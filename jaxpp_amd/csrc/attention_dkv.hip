@@ -1,6 +1,6 @@
 // dK/dV of causal attention (see attention.hip for the conventions).  This kernel has one
 // wave per SIMD and nothing to hide its latencies behind but its own instruction order; it
-// is compiled with LLVM's iterative ILP scheduler, which orders it 9 % faster than the
+// is compiled with LLVM's iterative ILP scheduler, which orders it 4 % faster than the
 // default one does (and the other attention kernels slower, hence the separate file).
 #include "attention_common.h"
 
