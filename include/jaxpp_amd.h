@@ -223,6 +223,15 @@ int jpp_grad_accum_f32(void* stream, float* acc, const void* g, int64_t count, i
 /* acc[j] += sum_t x[t,j] (bias gradients); partial: f32 [JPP_NORM_PARTIALS*cols]. */
 int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int64_t cols,
                      float* acc, float* partial);
+/* The same for up to 4 tensors of `rows` rows in one pair of launches (the bias gradients of
+ * a layer); partial: f32 [JPP_NORM_PARTIALS * sum of cols]. */
+typedef struct {
+  const void* x;     /* bf16 [rows, cols], leading dimension ld */
+  int64_t ld, cols;  /* multiples of 8 */
+  float* acc;        /* f32 [cols], added to */
+} jpp_colsum_item;
+int jpp_colsum_accum_multi(void* stream, int n, const jpp_colsum_item* items, int64_t rows,
+                           float* partial);
 /* Loss of the last stage as in the reference's examples (README.md:76-78):
  * loss[0] = scale * mean((out - target)^2) over `count` bf16 elements, and its
  * cotangent dout = scale * 2 (out - target) / count (bf16).  partial: f32

@@ -234,6 +234,60 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const bf16_t* __res
   *(float4*)(dst + 4) = make_float4(s[4], s[5], s[6], s[7]);
 }
 
+// Several column sums in one launch: the tensors' columns are laid side by side in one virtual
+// row of `total` columns (each tensor's share a multiple of 8), and so are the partial sums.
+struct ColsumBatch {
+  const bf16_t* x[4];
+  long ld[4];
+  float* acc[4];
+  int start[5];  // first virtual column of each tensor; start[n] = total
+  int n;
+};
+
+__global__ __launch_bounds__(256) void colsum_multi_partial_kernel(ColsumBatch b, long rows,
+                                                                   float* __restrict__ partial) {
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;  // virtual column of this thread's chunk
+  const int total = b.start[b.n];
+  if (c >= total) return;
+  int i = 0;
+  while (c >= b.start[i + 1]) ++i;
+  const bf16_t* x = b.x[i] + (c - b.start[i]);
+  const long ld = b.ld[i];
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (long row = blockIdx.x; row < rows; row += gridDim.x) {
+    float f[8];
+    unpack8(*(const uint4*)(x + row * ld), f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[e] += f[e];
+  }
+  float* dst = partial + (long)blockIdx.x * total + c;
+  *(float4*)dst = make_float4(s[0], s[1], s[2], s[3]);
+  *(float4*)(dst + 4) = make_float4(s[4], s[5], s[6], s[7]);
+}
+
+// as partial_reduce_kernel, the result scattered to the tensors' accumulators
+__global__ __launch_bounds__(1024) void colsum_multi_reduce_kernel(const float* __restrict__ partial,
+                                                                   int nblocks, ColsumBatch b) {
+  __shared__ float red[32][33];
+  const int c = threadIdx.x & 31, g = threadIdx.x >> 5;
+  const int j = blockIdx.x * 32 + c, total = b.start[b.n];
+  float s = 0.f;
+  if (j < total) {
+#pragma unroll 8
+    for (int k = g; k < nblocks; k += 32) s += partial[(long)k * total + j];
+  }
+  red[g][c] = s;
+  __syncthreads();
+  if (g == 0 && j < total) {
+    float t = red[0][c];
+#pragma unroll
+    for (int w = 1; w < 32; ++w) t += red[w][c];
+    int i = 0;
+    while (j >= b.start[i + 1]) ++i;
+    b.acc[i][j - b.start[i]] += t;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // SwiGLU
 // ---------------------------------------------------------------------------
@@ -555,6 +609,39 @@ int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int6
                      (long)ld, (long)rows, (int)cols, partial);
   hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 31) / 32)), dim3(1024), 0, st,
                      partial, nb, (int)cols, acc, (float*)nullptr);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_colsum_accum_multi(void* stream, int n, const jpp_colsum_item* items, int64_t rows,
+                           float* partial) {
+  JPP_REQUIRE(items && partial && n >= 1 && n <= 4 && rows > 0,
+              "colsum_multi: 1 to 4 tensors and a partial-sum buffer are required");
+  ColsumBatch b;
+  b.n = n;
+  int at = 0;
+  double bytes = 0;
+  for (int i = 0; i < n; ++i) {
+    const jpp_colsum_item& it = items[i];
+    JPP_REQUIRE(it.x && it.acc && it.cols > 0 && it.cols % 8 == 0 && it.ld % 8 == 0 &&
+                    it.ld >= it.cols && (uintptr_t)it.x % 16 == 0,
+                "colsum_multi: tensor %d: cols and ld must be multiples of 8, ld >= cols", i);
+    b.x[i] = (const bf16_t*)it.x;
+    b.ld[i] = it.ld;
+    b.acc[i] = it.acc;
+    b.start[i] = at;
+    at += (int)it.cols;
+    bytes += 2.0 * rows * it.cols;
+  }
+  b.start[n] = at;
+  hipStream_t st = (hipStream_t)stream;
+  ProbeScope probe(st, "colsum", 0, bytes);
+  const int nb = (int)(rows < JPP_NORM_PARTIALS ? rows : JPP_NORM_PARTIALS);
+  const int panels = (at / 8 + 255) / 256;
+  hipLaunchKernelGGL(colsum_multi_partial_kernel, dim3(nb, panels), dim3(256), 0, st, b, (long)rows,
+                     partial);
+  hipLaunchKernelGGL(colsum_multi_reduce_kernel, dim3((at + 31) / 32), dim3(1024), 0, st, partial, nb,
+                     b);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }

@@ -326,10 +326,11 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(jpp_attn_bwd(st, &aa));
     RC(gemm(st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dx, h, T, h, 3 * h,
             JPP_EPI_BF16, nullptr, wt(W.da), h));
-    RC(jpp_colsum_accum(st, wt(W.dc), h, T, h, s->G(chunk, li, B_b2), partial));
-    RC(jpp_colsum_accum(st, wt(W.du), f, T, f, s->G(chunk, li, B_b1), partial));
-    RC(jpp_colsum_accum(st, wt(W.da), h, T, h, s->G(chunk, li, B_bo), partial));
-    RC(jpp_colsum_accum(st, dqkv, 3 * h, T, 3 * h, s->G(chunk, li, B_bqkv), partial));
+    const jpp_colsum_item bias_grads[4] = {{wt(W.dc), h, h, s->G(chunk, li, B_b2)},
+                                           {wt(W.du), f, f, s->G(chunk, li, B_b1)},
+                                           {wt(W.da), h, h, s->G(chunk, li, B_bo)},
+                                           {dqkv, 3 * h, 3 * h, s->G(chunk, li, B_bqkv)}};
+    RC(jpp_colsum_accum_multi(st, 4, bias_grads, T, partial));
     return JPP_OK;
   }
   void* dn = s->S<>(s->s_t2);   // dn2, later dn1
@@ -354,10 +355,11 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(norm_b(s, st, dn, at(L.x), (float*)at(L.mean1), (float*)at(L.rstd1),
               s->P(chunk, li, B_ln1g), wt(W.dh1), dx, s->G(chunk, li, B_ln1g),
               s->G(chunk, li, B_ln1b)));
-    RC(jpp_colsum_accum(st, dy, h, T, h, s->G(chunk, li, B_b2), partial));
-    RC(jpp_colsum_accum(st, wt(W.du), f, T, f, s->G(chunk, li, B_b1), partial));
-    RC(jpp_colsum_accum(st, wt(W.dh1), h, T, h, s->G(chunk, li, B_bo), partial));
-    RC(jpp_colsum_accum(st, dqkv, 3 * h, T, 3 * h, s->G(chunk, li, B_bqkv), partial));
+    const jpp_colsum_item bias_grads[4] = {{dy, h, h, s->G(chunk, li, B_b2)},
+                                           {wt(W.du), f, f, s->G(chunk, li, B_b1)},
+                                           {wt(W.dh1), h, h, s->G(chunk, li, B_bo)},
+                                           {dqkv, 3 * h, 3 * h, s->G(chunk, li, B_bqkv)}};
+    RC(jpp_colsum_accum_multi(st, 4, bias_grads, T, partial));
     return JPP_OK;
   }
   // llama
@@ -602,8 +604,10 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   s->s_t2 = sc.take(T * h * e);
   s->s_t3 = sc.take(T * s->ctxw * e);
   const size_t widest = (size_t)std::max<int64_t>(std::max<int64_t>(s->qkvw, 2 * f), h);
-  s->s_partial = sc.take(std::max((size_t)2 * JPP_NORM_PARTIALS * widest * 4,
-                                  (size_t)64 * h * 8 * 4));
+  // norm-gradient partial sums (two vectors), the router's, or a layer's four bias gradients
+  s->s_partial = sc.take(std::max({(size_t)2 * JPP_NORM_PARTIALS * widest * 4,
+                                   (size_t)64 * h * 8 * 4,
+                                   (size_t)JPP_NORM_PARTIALS * (size_t)(5 * h + f) * 4}));
   s->s_partial_side = sc.take(d->two_streams ? (size_t)64 * h * 8 * 4 : 256);
   s->s_delta = sc.take((size_t)d->batch * d->n_heads * d->seq * 4);
   size_t max_w = 0;

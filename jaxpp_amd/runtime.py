@@ -73,6 +73,10 @@ class AdamArgs(C.Structure):
                 ("eps", C.c_double), ("grad_scale", C.c_double), ("zero_grad", C.c_int)]
 
 
+class ColsumItem(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("ld", C.c_int64), ("cols", C.c_int64), ("acc", C.c_void_p)]
+
+
 class StageDesc(C.Structure):
     _fields_ = [("family", C.c_int), ("hidden", C.c_int), ("n_heads", C.c_int),
                 ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("ffn", C.c_int),
@@ -99,7 +103,7 @@ EXPORTS = [
     "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
-    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
+    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_colsum_accum_multi", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
     "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32", "jpp_adam_step",
     "jpp_stage_optimizer_init", "jpp_stage_opt_ptr", "jpp_stage_adam_step",
@@ -165,6 +169,8 @@ def load():
     lib.jpp_grad_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
     lib.jpp_colsum_accum.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                      C.c_void_p, C.c_void_p]
+    lib.jpp_colsum_accum_multi.argtypes = [C.c_void_p, C.c_int, C.POINTER(ColsumItem), C.c_int64,
+                                           C.c_void_p]
     lib.jpp_mse_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float,
                                  C.c_void_p, C.c_void_p, C.c_void_p]
     lib.jpp_moe_capacity.restype = C.c_int64

@@ -259,6 +259,20 @@ def test_swiglu_rope_accum_colsum_cast():
     rt.check(lib.jpp_colsum_accum(None, bx.ptr, cols, rows, cols, bacc.ptr, part.ptr))
     rt.sync()
     close(bacc.download(np.float32, (cols,)), acc + xx.sum(0), 1e-4, "colsum")
+    # several tensors at once (a layer's bias gradients): widths 256 / 1024 / 8 / 3072, one of
+    # them a column slice of a wider tensor
+    widths, lds = [256, 1024, 8, 3072], [256, 1024, 64, 3072]
+    xs = [rnd(rng, rows, ld) for ld in lds]
+    accs = [rng.standard_normal(w).astype(np.float32) for w in widths]
+    bxs, baccs = [dev_bf16(x) for x in xs], [rt.DeviceBuffer.from_numpy(a) for a in accs]
+    items = (rt.ColsumItem * 4)(*[rt.ColsumItem(bx.ptr, ld, w, ba.ptr)
+                                  for bx, ld, w, ba in zip(bxs, lds, widths, baccs)])
+    part = rt.DeviceBuffer(rt.NORM_PARTIALS * sum(widths) * 4)
+    rt.check(lib.jpp_colsum_accum_multi(None, 4, items, rows, part.ptr))
+    rt.sync()
+    for x, w, a, ba in zip(xs, widths, accs, baccs):
+        close(ba.download(np.float32, (w,)), a + x[:, :w].sum(0), 1e-4, f"colsum of {w} columns")
+    assert lib.jpp_colsum_accum_multi(None, 5, items, rows, part.ptr) == -1
 
     src = rng.standard_normal(1001).astype(np.float32)
     bsrc, bdst = rt.DeviceBuffer.from_numpy(src), rt.DeviceBuffer(1001 * 2)
