@@ -151,7 +151,9 @@ typedef struct {
    *   JPP_GROUP_M: rows of A and C are grouped; group e multiplies b + e * stride_b.
    *                m is the capacity of the permuted buffer; tiles past seg[n_seg] exit.
    *   JPP_GROUP_K: (weight gradients) C_e = c + e * stride_c gets the product over the
-   *                rows seg[e] .. seg[e+1] of A and B; k is ignored. */
+   *                rows seg[e] .. seg[e+1] (multiples of 64) of A and B; k is ignored.  Also
+   *                the way to split one long contraction over workgroups: equal ranges, an
+   *                f32 epilogue into scratch, then jpp_sum_accum_f32. */
   const int32_t* seg;
   int n_seg;
   int group_mode;
@@ -220,6 +222,10 @@ int jpp_rope(void* stream, void* x, int64_t ld, const float* cos_tab, const floa
 /* acc[i] += g[i]; g is bf16 (g_is_f32 == 0) or f32.  The gradient accumulation
  * of `treduce`'s Add (src/jaxpp/training.py:112-123) as a standalone pass. */
 int jpp_grad_accum_f32(void* stream, float* acc, const void* g, int64_t count, int g_is_f32);
+/* acc[i] += parts[0][i] + parts[1][i] + ... + parts[n_parts-1][i], summed in that order;
+ * parts: f32 [n_parts, count].  Closes a contraction that was split over workgroups
+ * (JPP_GROUP_K with an f32 epilogue into `parts`) without making the result depend on timing. */
+int jpp_sum_accum_f32(void* stream, float* acc, const float* parts, int n_parts, int64_t count);
 /* acc[j] += sum_t x[t,j] (bias gradients); partial: f32 [JPP_NORM_PARTIALS*cols]. */
 int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int64_t cols,
                      float* acc, float* partial);

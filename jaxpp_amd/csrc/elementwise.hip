@@ -400,6 +400,23 @@ __global__ __launch_bounds__(256) void grad_accum_kernel(float* __restrict__ acc
   }
 }
 
+// acc += parts[0] + parts[1] + ... (in that order): the partial products of a contraction
+// that was split over workgroups
+__global__ __launch_bounds__(256) void sum_accum_kernel(float* __restrict__ acc,
+                                                        const float* __restrict__ parts,
+                                                        int n_parts, long n4) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n4; i += (long)gridDim.x * 256) {
+    float4 s = ((const float4*)parts)[i];
+    for (int k = 1; k < n_parts; ++k) {
+      const float4 t = ((const float4*)parts)[(long)k * n4 + i];
+      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    float4 a = ((float4*)acc)[i];
+    a.x += s.x; a.y += s.y; a.z += s.z; a.w += s.w;
+    ((float4*)acc)[i] = a;
+  }
+}
+
 template <bool G_F32>
 __global__ void grad_accum_tail_kernel(float* acc, const void* g, long start, long count) {
   const long i = start + blockIdx.x * 256 + threadIdx.x;
@@ -609,6 +626,18 @@ int jpp_colsum_accum(void* stream, const void* x, int64_t ld, int64_t rows, int6
                      (long)ld, (long)rows, (int)cols, partial);
   hipLaunchKernelGGL(partial_reduce_kernel, dim3((int)((cols + 31) / 32)), dim3(1024), 0, st,
                      partial, nb, (int)cols, acc, (float*)nullptr);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_sum_accum_f32(void* stream, float* acc, const float* parts, int n_parts, int64_t count) {
+  JPP_REQUIRE(acc && parts && n_parts >= 1 && count > 0 && count % 4 == 0,
+              "sum_accum: bad arguments (count must be a positive multiple of 4)");
+  JPP_REQUIRE((uintptr_t)acc % 16 == 0 && (uintptr_t)parts % 16 == 0,
+              "sum_accum: operands must be 16-byte aligned");
+  ProbeScope probe((hipStream_t)stream, "sum_accum", 0, (4.0 * n_parts + 8.0) * count);
+  hipLaunchKernelGGL(sum_accum_kernel, dim3(grid_for(count / 4)), dim3(256), 0, (hipStream_t)stream,
+                     acc, parts, n_parts, (long)(count / 4));
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }

@@ -599,7 +599,9 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     JPP_REQUIRE(a->group_mode == JPP_GROUP_M || a->group_mode == JPP_GROUP_K,
                 "gemm: unknown group_mode %d", a->group_mode);
     JPP_REQUIRE(a->seg && a->n_seg > 0 && a->n_seg <= 256, "gemm: grouped problem needs seg[n_seg+1]");
-    JPP_REQUIRE(a->m % 256 == 0 && a->n % 256 == 0, "gemm: grouped problems need M, N multiples of 256");
+    JPP_REQUIRE((a->m % 256 == 0 && a->n % 256 == 0) || (a->group_mode == JPP_GROUP_K && a->tile),
+                "gemm: grouped problems need M, N multiples of 256 (a grouped contraction with "
+                "a tile of the caller's choice: of that tile)");
     JPP_REQUIRE(!a->bias && !a->resid, "gemm: grouped problems take no bias / residual");
   }
   if (a->epilogue == JPP_EPI_GELU)
@@ -619,7 +621,8 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
                 "gemm: an accumulated output must span less than 4 GiB (32-bit offsets)");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
-  if (a->group_mode != JPP_GROUP_NONE) tile = 4;  // 256-row segments
+  // row groups come in 256-row segments; a contraction split into groups takes any tile
+  if (a->group_mode == JPP_GROUP_M || (a->group_mode == JPP_GROUP_K && !a->tile)) tile = 4;
   JPP_REQUIRE(tile >= 1 && tile <= 4, "gemm: unknown tile %d", tile);
   if ((tile == 2 || tile == 4) && a->m % 256) tile = a->n % 256 ? 1 : 3;
   if ((tile == 3 || tile == 4) && a->n % 256) tile = a->m % 256 ? 1 : 2;

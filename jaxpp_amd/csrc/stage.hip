@@ -89,8 +89,8 @@ struct jpp_stage {
   // layer l+1 read set (l+1)%3 while layer l's input-gradient chain writes set l%3 and
   // hands its result to layer l-1 in set (l-1)%3.
   LayerStash wsets[3];
-  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_partial_side, s_delta, s_wg, s_cos, s_sin,
-      s_moework;
+  Buf s_dx[2], s_t1, s_t2, s_t3, s_t4, s_partial, s_partial_side, s_delta, s_wg, s_split, s_cos,
+      s_sin, s_moework;
   size_t total_bytes = 0;
   // second stream (two_streams): weight gradients trail the input-gradient chain
   hipStream_t side = nullptr;
@@ -171,8 +171,31 @@ int gemm(hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int6
 // dW[rows, cols] (+)= X^T dY, X: [T, rows], dY: [T, cols]
 int wgrad(jpp_stage* s, hipStream_t st, const void* x, int64_t ldx, const void* dy, int64_t lddy,
           float* acc, int64_t rows, int64_t cols) {
-  if (s->d.fused_wgrad_accum)
+  if (s->d.fused_wgrad_accum) {
+    // A weight matrix of at most 128 tiles of 128x128 leaves half of the CUs without work:
+    // the contraction over the tokens is then split over `parts` workgroups per tile, which
+    // leave f32 partial products in scratch, and an ordered sum adds them to the accumulator
+    // (the order is fixed, so the result does not depend on timing).
+    const int64_t tiles = (rows / 128) * (cols / 128);
+    int parts = 1;
+    while (parts < 8 && tiles * parts * 2 <= 256 && s->T % (parts * 2 * 64) == 0 &&
+           s->T / (parts * 2) >= 512)
+      parts *= 2;
+    if (parts > 1 && (size_t)parts * rows * cols * 4 <= s->s_wg.bytes) {
+      float* ws = s->S<float>(s->s_wg);
+      jpp_gemm_args g;
+      memset(&g, 0, sizeof(g));
+      g.a = x; g.b = dy; g.c = ws; g.m = rows; g.n = cols; g.k = 0;
+      g.lda = ldx; g.ldb = lddy; g.ldc = cols; g.trans_a = 1; g.trans_b = 1;
+      g.epilogue = JPP_EPI_F32; g.tile = 1;
+      g.seg = s->S<int32_t>(s->s_split) + 16 * (parts == 2 ? 0 : parts == 4 ? 1 : 2);
+      g.n_seg = parts; g.group_mode = JPP_GROUP_K; g.stride_c = rows * cols;
+      g.group_rows = s->T;
+      RC(jpp_gemm_bf16(st, &g));
+      return jpp_sum_accum_f32(st, acc, ws, parts, rows * cols);
+    }
     return gemm(st, x, ldx, 1, dy, lddy, 1, acc, cols, rows, cols, s->T, JPP_EPI_ACC_F32);
+  }
   void* g = s->S<>(s->s_wg);
   RC(gemm(st, x, ldx, 1, dy, lddy, 1, g, cols, rows, cols, s->T, JPP_EPI_BF16));
   return jpp_grad_accum_f32(st, acc, g, rows * cols, 0);
@@ -612,7 +635,10 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   s->s_delta = sc.take((size_t)d->batch * d->n_heads * d->seq * 4);
   size_t max_w = 0;
   for (auto& p : s->pinfo) max_w = std::max(max_w, (size_t)(p.rows * p.cols));
-  s->s_wg = sc.take(d->fused_wgrad_accum ? 256 : max_w * e);
+  // unfused path: a bf16 weight gradient; fused path: partial products of a split contraction
+  // (at most 256 tiles of 128x128 in all)
+  s->s_wg = sc.take(d->fused_wgrad_accum ? (size_t)256 * 128 * 128 * 4 : max_w * e);
+  s->s_split = sc.take(3 * 16 * 4);  // token offsets of a contraction split in 2, 4, 8
   s->s_cos = sc.take((size_t)d->seq * (hd / 2) * 4);
   s->s_sin = sc.take((size_t)d->seq * (hd / 2) * 4);
   s->scratch_bytes = sc.total;
@@ -641,6 +667,12 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   hipMemset(s->params, 0, n_layers * s->layer_elems * 2);
   hipMemset(s->grads, 0, n_layers * s->layer_elems * 4);
 
+  {
+    int32_t split[3 * 16] = {};
+    for (int k = 0; k < 3; ++k)
+      for (int i = 0; i <= (2 << k); ++i) split[16 * k + i] = (int32_t)(T / (2 << k) * i);
+    hipMemcpy(s->S<>(s->s_split), split, sizeof(split), hipMemcpyHostToDevice);
+  }
   if (d->family == JPP_FAMILY_LLAMA || d->family == JPP_FAMILY_MIXTRAL) {
     // cos/sin of pos * theta^(-2i/d): evaluated in double, stored as f32
     const int half = hd / 2;

@@ -103,7 +103,7 @@ EXPORTS = [
     "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
-    "jpp_grad_accum_f32", "jpp_colsum_accum", "jpp_colsum_accum_multi", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
+    "jpp_grad_accum_f32", "jpp_sum_accum_f32", "jpp_colsum_accum", "jpp_colsum_accum_multi", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
     "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32", "jpp_adam_step",
     "jpp_stage_optimizer_init", "jpp_stage_opt_ptr", "jpp_stage_adam_step",
@@ -169,6 +169,7 @@ def load():
     lib.jpp_grad_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
     lib.jpp_colsum_accum.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                      C.c_void_p, C.c_void_p]
+    lib.jpp_sum_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64]
     lib.jpp_colsum_accum_multi.argtypes = [C.c_void_p, C.c_int, C.POINTER(ColsumItem), C.c_int64,
                                            C.c_void_p]
     lib.jpp_mse_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float,

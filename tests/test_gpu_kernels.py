@@ -468,3 +468,31 @@ def test_mfma_rate_diagnostic():
             assert 250.0 < t < 2600.0, (shape, rnd, t)
     with pytest.raises(rt.JppError, match="shape is 16"):
         rt.mfma_rate(8, False)
+
+
+def test_split_contraction():
+    """A contraction split over workgroups: JPP_GROUP_K with an f32 epilogue leaves one partial
+    product per token range, jpp_sum_accum_f32 adds them to the accumulator in order."""
+    rng = np.random.default_rng(31)
+    m, n, T, parts = 256, 384, 2048, 4
+    x, dy = rnd(rng, T, m), rnd(rng, T, n)
+    acc0 = rng.standard_normal((m, n)).astype(np.float32)
+    seg = np.arange(parts + 1, dtype=np.int32) * (T // parts)
+    b_x, b_dy, b_seg = dev_bf16(x), dev_bf16(dy), rt.DeviceBuffer.from_numpy(seg)
+    ws, b_acc = rt.DeviceBuffer(parts * m * n * 4), rt.DeviceBuffer.from_numpy(acc0)
+    rt.gemm(b_x.ptr, b_dy.ptr, ws.ptr, m, n, 0, m, n, n, 1, 1, rt.EPI_F32, tile=1, seg=b_seg.ptr,
+            n_seg=parts, group_mode=2, stride_c=m * n)
+    rt.check(rt.load().jpp_sum_accum_f32(None, b_acc.ptr, ws.ptr, parts, m * n))
+    rt.sync()
+    part_h = ws.download(np.float32, (parts, m, n))
+    for k in range(parts):
+        rows = slice(seg[k], seg[k + 1])
+        close(part_h[k], x[rows].T @ dy[rows], 1e-4 * math.sqrt(T // parts), f"part {k}")
+    got = b_acc.download(np.float32, (m, n))
+    # the sum is taken in the order of the parts, exactly
+    want = part_h[0].copy()
+    for k in range(1, parts):
+        want += part_h[k]
+    np.testing.assert_array_equal(got, acc0 + want)
+    with pytest.raises(rt.JppError, match="multiple of 4"):
+        rt.check(rt.load().jpp_sum_accum_f32(None, b_acc.ptr, ws.ptr, parts, 6))
