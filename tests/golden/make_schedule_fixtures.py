@@ -75,7 +75,7 @@ def digest(obj) -> str:
 
 # (class name, constructor kwargs, n_mubatches, store full table?)
 CASES = [
-    # the five BASELINE configurations
+    # the five benchmark configurations
     ("Std1F1B", {"num_stages": 2}, 8, True),
     ("Std1F1B", {"num_stages": 4}, 16, True),
     ("Interleaved1F1B", {"num_stages": 8, "mpmd_dim": 4}, 32, True),
