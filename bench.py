@@ -160,8 +160,8 @@ def cpu_baseline(wl, budget_layers: int = 1):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--n-mubatches", type=int, default=None,
@@ -284,7 +284,9 @@ def main():
     if args.after_loop:
         rec["after_loop"] = after_loop(wb, wl, args.steps)
     if not args.no_cpu_baseline:
-        rec["cpu_baseline"] = cpu_baseline(wl)
+        # a sample of 10-20 s on the host: about 1.2e13 FLOP at the ~1 TFLOP/s its BLAS reaches
+        layers = int(round(1.2e13 / (3.0 * wl.layer.fwd_flops())))
+        rec["cpu_baseline"] = cpu_baseline(wl, max(1, min(wl.layers_per_stage, layers)))
     print(json.dumps(rec))
 
 
