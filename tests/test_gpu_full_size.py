@@ -48,6 +48,9 @@ FULL = [
     ("nt", 2048, 1024, 4096, rt.EPI_BF16, 2),       # 256x128
     ("tn", 1024, 2048, 4096, rt.EPI_ACC_F32, 3),    # 128x256, streamed accumulator
     ("nn", 1152, 2048, 4096, rt.EPI_F32, 3),
+    # Llama-70B-shaped stage: hidden 8192, 64 + 2 x 8 heads of 128, SwiGLU 28672
+    ("nt", 4096, 8192, 28672, rt.EPI_BF16, 0),      # input gradient of the down projection: 448 K-steps
+    ("tn", 8192, 10240, 4096, rt.EPI_ACC_F32, 0),   # QKV weight gradient: five full rounds of tiles
 ]
 
 
@@ -87,6 +90,72 @@ def test_gemm_checksums_at_full_size(lay, m, n, k, epi, tile):
     want_cols = A64 @ B64[cols].T + (p64[:, cols] if prev is not None else 0.0)
     assert np.abs(got[rows] - want_rows).max() <= elem, "dense rows"
     assert np.abs(got[:, cols] - want_cols).max() <= elem, "dense columns"
+
+
+def test_grouped_gemms_at_full_size():
+    """The expert products of the Mixtral-shaped stage (8 experts, hidden 4096, SwiGLU 14336,
+    2 x 8192 token copies): the down projection over ragged 256-row-padded groups and its
+    weight gradient, one output per expert.  Row checksums per expert (a misplaced or dropped
+    tile, or a group that multiplies another group's weights, breaks them), dense rows at the
+    group edges, untouched padding; for the weight gradient row and column checksums per expert
+    and the bit pattern of an expert without rows."""
+    print("full-size grouped gemms", flush=True)
+    rng = np.random.default_rng(5)
+    E, h, f = 8, 4096, 14336
+    counts = [3000, 1, 2304, 0, 4095, 2048, 2560, 2376]          # 16384 token copies
+    seg = np.zeros(E + 1, np.int32)
+    for e, c in enumerate(counts):
+        seg[e + 1] = seg[e] + (c + 255) // 256 * 256
+    cap = int(seg[E]) + 256
+    s_h = np.zeros((cap, f), np.float32)                          # SwiGLU outputs, grouped rows
+    for e, c in enumerate(counts):
+        s_h[seg[e]:seg[e] + c] = rnd(rng, c, f)
+    w2 = rnd(rng, E, f, h, scale=0.05)
+    b_seg = rt.DeviceBuffer.from_numpy(seg)
+    b_rows = rt.DeviceBuffer.from_numpy(np.array(counts, np.int32))
+    b_s, b_w = rt.DeviceBuffer.from_f32_as_bf16(s_h), rt.DeviceBuffer.from_f32_as_bf16(w2)
+    out = rt.DeviceBuffer(cap * h * 2)
+    out.zero()
+    rt.gemm(b_s.ptr, b_w.ptr, out.ptr, cap, h, f, f, h, h, 0, 1, rt.EPI_BF16, seg=b_seg.ptr, n_seg=E,
+            group_mode=1, stride_b=f * h, seg_rows=b_rows.ptr)
+    rt.sync()
+    got = out.download_bf16((cap, h)).astype(np.float64)
+    assert np.isfinite(got).all()
+    assert not got[seg[E]:].any(), "tiles past the last group must not be written"
+    elem = 1e-2 * float(np.abs(got).max())
+    for e, c in enumerate(counts):
+        if not c:
+            continue
+        rows = slice(int(seg[e]), int(seg[e]) + c)
+        want = s_h[rows].astype(np.float64) @ w2[e].astype(np.float64).sum(axis=1)
+        assert np.abs(got[rows].sum(axis=1) - want).max() <= elem * math.sqrt(h), f"row checksums, expert {e}"
+        edge = [int(seg[e]), int(seg[e]) + c - 1]
+        dense = s_h[edge].astype(np.float64) @ w2[e].astype(np.float64)
+        assert np.abs(got[edge] - dense).max() <= elem, f"dense rows, expert {e}"
+        assert not got[int(seg[e]) + c:int(seg[e + 1])].any(), f"padding rows of expert {e}"
+    # weight gradient of the same projection: dW2[e] += s_e^T dy_e
+    dy = np.zeros((cap, h), np.float32)
+    for e, c in enumerate(counts):
+        dy[seg[e]:seg[e] + c] = rnd(rng, c, h, scale=0.05)
+    del out, b_w
+    acc0 = rng.standard_normal((E, f, h), dtype=np.float32)
+    b_dy, b_acc = rt.DeviceBuffer.from_f32_as_bf16(dy), rt.DeviceBuffer.from_numpy(acc0)
+    rt.gemm(b_s.ptr, b_dy.ptr, b_acc.ptr, f, h, 0, f, h, h, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
+            n_seg=E, group_mode=2, stride_c=f * h, seg_rows=b_rows.ptr)
+    rt.sync()
+    gw = b_acc.download(np.float32, (E, f, h))
+    np.testing.assert_array_equal(gw[3], acc0[3])                 # expert without rows
+    for e, c in enumerate(counts):
+        if not c:
+            continue
+        rows = slice(int(seg[e]), int(seg[e]) + c)
+        se, de = s_h[rows].astype(np.float64), dy[rows].astype(np.float64)
+        d = gw[e].astype(np.float64) - acc0[e]
+        tol = 1e-4 * math.sqrt(max(c, 64)) * max(float(np.abs(gw[e]).max()), 1.0)
+        assert np.abs(d.sum(axis=1) - se.T @ de.sum(axis=1)).max() <= tol * math.sqrt(h), f"dW row checksums, expert {e}"
+        assert np.abs(d.sum(axis=0) - de.T @ se.sum(axis=1)).max() <= tol * math.sqrt(f), f"dW column checksums, expert {e}"
+        cols = [0, 255, 256, h - 1]
+        assert np.abs(d[:, cols] - se.T @ de[:, cols]).max() <= tol, f"dW dense columns, expert {e}"
 
 
 LLAMA_8B_LAYER = LayerSpec("llama", 4096, 32, 14336, 4096, 1, n_kv_heads=8, head_dim=128,
