@@ -211,8 +211,22 @@ def main():
     wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two)
     cls = args.probe or dominant_gemm_class(wl)
 
-    for _ in range(args.warmup):
+    # The host enqueues a step in a fraction of the time the GPU takes to run it.  It is kept at
+    # most two steps ahead (the queue never drains, so the timing is unaffected): tools that
+    # keep a record per dispatch in flight, rocprofv3 among them, do not survive a backlog of
+    # 100 000 launches.
+    ends = []
+
+    def paced_step():
+        if len(ends) >= 2:
+            ends.pop(0).sync()
         wb.step()
+        ev = rt.Event()
+        ev.record()
+        ends.append(ev)
+
+    for _ in range(args.warmup):
+        paced_step()
     rt.sync()
     start, stop = rt.Event(), rt.Event()
     if args.graph:
@@ -238,7 +252,7 @@ def main():
         with rt.probe(cls) as pr:
             start.record()
             for _ in range(args.steps):
-                wb.step()
+                paced_step()
             stop.record()
             stop.sync()
     rt.sync()
