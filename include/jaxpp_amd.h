@@ -247,6 +247,25 @@ int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t coun
 int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count);
 int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count);
 
+/* ---- the same operators on f32 tensors -----------------------------------------
+ * The full-precision flavour of a stage (jpp_stage_desc.dtype = JPP_DTYPE_F32): the
+ * reference's CPU-runnable configuration is float32 end to end (BERT-style stack of
+ * hidden 256; tests/test_transformations.py:44-118 also builds its model in float32).
+ * Same argument structs, every bf16 tensor replaced by an f32 one; plain fp32 arithmetic
+ * in a fixed summation order, sized for small problems (not for the matrix cores).
+ * jpp_gemm_f32: M, N multiples of 64, K of 16; epilogues JPP_EPI_BF16 (= store, with bias
+ * and residual), JPP_EPI_F32, JPP_EPI_GELU, JPP_EPI_DGELU, JPP_EPI_ACC_F32; no groups.
+ * jpp_attn_*_f32: seq a multiple of 64.  jpp_norm_bwd_f32 does not use `partial`. */
+int jpp_gemm_f32(void* stream, const jpp_gemm_args* args);
+int jpp_attn_fwd_f32(void* stream, const jpp_attn_args* args);
+int jpp_attn_bwd_f32(void* stream, const jpp_attn_args* args);
+int jpp_norm_fwd_f32(void* stream, const jpp_norm_args* args);
+int jpp_norm_bwd_f32(void* stream, const jpp_norm_args* args);
+int jpp_colsum_accum_f32(void* stream, const float* x, int64_t ld, int64_t rows, int64_t cols,
+                         float* acc);
+int jpp_mse_loss_f32(void* stream, const float* out, const float* target, int64_t count,
+                     float scale, float* loss, float* dout);
+
 /* ---- after the loop: the optimizer on the accumulated gradients --------------
  * The reference's train step applies `optimizer.update(grad, opt_state, pars)` and
  * `optax.apply_updates` to what `treduce` returns (README.md:90-93; examples/basic.py:234

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libjaxpp_amd.so")
 SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "attention_dkv.hip", "elementwise.hip",
-           "moe.hip", "optimizer.hip", "diagnostics.hip", "stage.hip"]
+           "moe.hip", "optimizer.hip", "diagnostics.hip", "f32_ops.hip", "stage.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          # packed fp32 ops are kept out of generated code on this hardware pool
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -102,6 +102,8 @@ EXPORTS = [
     "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_graph_begin", "jpp_graph_end", "jpp_graph_launch",
     "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
+    "jpp_gemm_f32", "jpp_attn_fwd_f32", "jpp_attn_bwd_f32", "jpp_norm_fwd_f32", "jpp_norm_bwd_f32",
+    "jpp_colsum_accum_f32", "jpp_mse_loss_f32",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_sum_accum_f32", "jpp_colsum_accum", "jpp_colsum_accum_multi", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
@@ -160,6 +162,15 @@ def load():
     lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_norm_fwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
     lib.jpp_norm_bwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
+    lib.jpp_gemm_f32.argtypes = [C.c_void_p, C.POINTER(GemmArgs)]
+    lib.jpp_attn_fwd_f32.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
+    lib.jpp_attn_bwd_f32.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
+    lib.jpp_norm_fwd_f32.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
+    lib.jpp_norm_bwd_f32.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
+    lib.jpp_colsum_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                         C.c_void_p]
+    lib.jpp_mse_loss_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float,
+                                     C.c_void_p, C.c_void_p]
     lib.jpp_swiglu_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                    C.c_int]
     lib.jpp_swiglu_bwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
@@ -422,11 +433,11 @@ class probe:
 def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, bias=None,
          resid=None, ldresid=0, aux=None, ldaux=0, c2=None, ldc2=0, gelu_tanh=0, tile=0,
          stream=None, seg=None, n_seg=0, group_mode=0, stride_b=0, stride_c=0, group_rows=0,
-         seg_rows=None):
+         seg_rows=None, f32=False):
     g = GemmArgs(a, b, c, c2, bias, resid, aux, m, n, k, lda, ldb, ldc, ldc2, ldresid, ldaux,
                  int(trans_a), int(trans_b), epilogue, gelu_tanh, tile, seg, n_seg, group_mode,
                  stride_b, stride_c, group_rows, seg_rows)
-    check(load().jpp_gemm_bf16(stream, C.byref(g)))
+    check((load().jpp_gemm_f32 if f32 else load().jpp_gemm_bf16)(stream, C.byref(g)))
 
 
 def mfma_rate(shape: int, random_operands: bool, iters: int = 100000) -> float:

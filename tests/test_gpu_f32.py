@@ -1,0 +1,189 @@
+"""The f32 operators (jpp_*_f32) against numpy in float64, through the C ABI.
+
+Tolerance 1e-5 of a tensor's largest magnitude for single operators (fp32 arithmetic in a
+fixed order against float64), 1e-4 - the bound stated for fp32 results - for whole stages."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+
+from jaxpp_amd import runtime as rt
+from oracle import layers as L
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    rt.require_gpu()
+
+
+def close(got, want, rtol, what):
+    scale = float(np.abs(want).max()) + 1e-30
+    err = float(np.abs(got.astype(np.float64) - want).max())
+    assert np.isfinite(got).all(), f"{what}: non-finite"
+    assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+
+
+def dev(a):
+    return rt.DeviceBuffer.from_numpy(np.ascontiguousarray(a, dtype=np.float32))
+
+
+GEMMS = [("nn", 128, 192, 64), ("nn", 512, 768, 256), ("nt", 512, 256, 1024), ("tn", 256, 1024, 512)]
+
+
+@pytest.mark.parametrize("lay,m,n,k", GEMMS, ids=[f"{c[0]}-{c[1]}x{c[2]}x{c[3]}" for c in GEMMS])
+def test_gemm_f32_epilogues(lay, m, n, k):
+    print(f"gemm_f32 {lay} {m}x{n}x{k}", flush=True)
+    rng = np.random.default_rng(m + n + k)
+    ta, tb = {"nn": (0, 1), "nt": (0, 0), "tn": (1, 1)}[lay]
+    A = rng.standard_normal((m, k), dtype=np.float32)
+    B = rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.1)
+    bias = rng.standard_normal(n, dtype=np.float32)
+    resid = rng.standard_normal((m, n), dtype=np.float32)
+    aux = rng.standard_normal((m, n), dtype=np.float32)
+    a_h = np.ascontiguousarray(A.T) if ta else A
+    b_h = np.ascontiguousarray(B.T) if tb else B
+    da, db, dbias, dres, daux = dev(a_h), dev(b_h), dev(bias), dev(resid), dev(aux)
+    prod = A.astype(np.float64) @ B.astype(np.float64).T
+    lda, ldb = a_h.shape[1], b_h.shape[1]
+
+    def run(epi, c0=None, **kw):
+        dc = dev(c0 if c0 is not None else np.zeros((m, n), np.float32))
+        rt.gemm(da.ptr, db.ptr, dc.ptr, m, n, k, lda, ldb, n, ta, tb, epi, f32=True, **kw)
+        rt.sync()
+        return dc.download(np.float32, (m, n))
+
+    close(run(rt.EPI_BF16), prod, 1e-5, "store")
+    close(run(rt.EPI_F32), prod, 1e-5, "f32 store")
+    close(run(rt.EPI_BF16, bias=dbias.ptr, resid=dres.ptr, ldresid=n), prod + bias + resid, 1e-5,
+          "bias + residual")
+    c0 = rng.standard_normal((m, n), dtype=np.float32)
+    close(run(rt.EPI_ACC_F32, c0), prod + c0, 1e-5, "accumulate")
+    for tanh_form in (0, 1):
+        u = prod + bias
+        if tanh_form:
+            t = np.tanh(0.7978845608028654 * (u + 0.044715 * u ** 3))
+            g = 0.5 * u * (1 + t)
+        else:
+            erf = np.vectorize(math.erf)
+            g = 0.5 * u * (1 + erf(u / math.sqrt(2)))
+        dc2 = dev(np.zeros((m, n), np.float32))
+        got_u = run(rt.EPI_GELU, bias=dbias.ptr, c2=dc2.ptr, ldc2=n, gelu_tanh=tanh_form)
+        close(got_u, u, 1e-5, "gelu pre-activation")
+        close(dc2.download(np.float32, (m, n)), g, 1e-5, "gelu")
+        x = aux.astype(np.float64)
+        if tanh_form:
+            t = np.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3))
+            gp = 0.5 * (1 + t) + 0.5 * x * (1 - t * t) * 0.7978845608028654 * (1 + 0.134145 * x * x)
+        else:
+            erf = np.vectorize(math.erf)
+            gp = 0.5 * (1 + erf(x / math.sqrt(2))) + x * np.exp(-0.5 * x * x) / math.sqrt(2 * math.pi)
+        close(run(rt.EPI_DGELU, aux=daux.ptr, ldaux=n, gelu_tanh=tanh_form), prod * gp, 1e-5, "dgelu")
+
+
+def test_gemm_f32_rejects_what_it_does_not_do():
+    d = rt.DeviceBuffer(64 * 64 * 4)
+    with pytest.raises(rt.JppError, match="multiples of 64"):
+        rt.gemm(d.ptr, d.ptr, d.ptr, 32, 64, 16, 16, 64, 64, 0, 1, f32=True)
+    with pytest.raises(rt.JppError, match="unsupported epilogue"):
+        rt.gemm(d.ptr, d.ptr, d.ptr, 64, 64, 16, 16, 64, 64, 0, 1, rt.EPI_SWIGLU, f32=True)
+
+
+@pytest.mark.parametrize("ln", [True, False], ids=["layernorm", "rmsnorm"])
+def test_norm_f32(ln):
+    rng = np.random.default_rng(3)
+    rows, cols, eps = 200, 320, 1e-5
+    x = rng.standard_normal((rows, cols), dtype=np.float32) * 2 + 0.5
+    gamma = rng.standard_normal(cols, dtype=np.float32)
+    beta = rng.standard_normal(cols, dtype=np.float32)
+    dy = rng.standard_normal((rows, cols), dtype=np.float32)
+    resid = rng.standard_normal((rows, cols), dtype=np.float32)
+    x64 = x.astype(np.float64)
+    mean = x64.mean(-1, keepdims=True) if ln else np.zeros((rows, 1))
+    var = ((x64 - mean) ** 2).mean(-1, keepdims=True)
+    rstd = 1.0 / np.sqrt(var + eps)
+    xh = (x64 - mean) * rstd
+    y_w = xh * gamma + (beta if ln else 0.0)
+    dg = dy.astype(np.float64) * gamma
+    s1 = dg.mean(-1, keepdims=True) if ln else 0.0
+    s2 = (dg * xh).mean(-1, keepdims=True)
+    dx_w = (dg - s1 - xh * s2) * rstd + resid
+    b = {k: dev(v) for k, v in dict(x=x, gamma=gamma, beta=beta, dy=dy, resid=resid).items()}
+    y, dx = rt.DeviceBuffer(rows * cols * 4), rt.DeviceBuffer(rows * cols * 4)
+    mean_d, rstd_d = rt.DeviceBuffer(rows * 4), rt.DeviceBuffer(rows * 4)
+    g0 = rng.standard_normal(cols, dtype=np.float32)
+    b0 = rng.standard_normal(cols, dtype=np.float32)
+    dgam, dbet = dev(g0), dev(b0)
+    a = rt.NormArgs(b["x"].ptr, b["gamma"].ptr, b["beta"].ptr if ln else None, y.ptr,
+                    mean_d.ptr if ln else None, rstd_d.ptr, b["dy"].ptr, b["resid"].ptr, dx.ptr,
+                    dgam.ptr, dbet.ptr if ln else None, None, rows, cols, eps)
+    lib = rt.load()
+    rt.check(lib.jpp_norm_fwd_f32(None, C.byref(a)))
+    rt.check(lib.jpp_norm_bwd_f32(None, C.byref(a)))
+    rt.sync()
+    close(y.download(np.float32, (rows, cols)), y_w, 1e-5, "y")
+    close(rstd_d.download(np.float32, (rows,)), rstd[:, 0], 1e-5, "rstd")
+    if ln:
+        close(mean_d.download(np.float32, (rows,)), mean[:, 0], 1e-5, "mean")
+    close(dx.download(np.float32, (rows, cols)), dx_w, 1e-5, "dx")
+    close(dgam.download(np.float32, (cols,)), g0 + (dy * xh).sum(0), 1e-5, "dgamma")
+    if ln:
+        close(dbet.download(np.float32, (cols,)), b0 + dy.astype(np.float64).sum(0), 1e-5, "dbeta")
+
+
+ATTN = [(2, 128, 4, 4, 64, False), (1, 256, 4, 2, 128, True), (2, 64, 2, 1, 64, True),
+        (1, 192, 2, 2, 128, False)]
+
+
+@pytest.mark.parametrize("B,S,Hq,Hkv,d,causal", ATTN,
+                         ids=[f"b{c[0]}s{c[1]}h{c[2]}kv{c[3]}d{c[4]}{'c' if c[5] else ''}" for c in ATTN])
+def test_attention_f32(B, S, Hq, Hkv, d, causal):
+    print(f"attention_f32 B{B} S{S} Hq{Hq} Hkv{Hkv} d{d} causal={causal}", flush=True)
+    rng = np.random.default_rng(S + d)
+    w = (Hq + 2 * Hkv) * d
+    qkv = rng.standard_normal((B * S, w), dtype=np.float32)
+    do = rng.standard_normal((B * S, Hq * d), dtype=np.float32)
+    q = qkv[:, :Hq * d].reshape(B, S, Hq, d)
+    k = qkv[:, Hq * d:(Hq + Hkv) * d].reshape(B, S, Hkv, d)
+    v = qkv[:, (Hq + Hkv) * d:].reshape(B, S, Hkv, d)
+    o_w, lse_w = L.attention_fwd(q, k, v, causal, np.float64)
+    dq_w, dk_w, dv_w = L.attention_bwd(q, k, v, o_w, do.reshape(B, S, Hq, d).astype(np.float64),
+                                       lse_w, causal, np.float64)
+    b_qkv, b_do = dev(qkv), dev(do)
+    o, lse = rt.DeviceBuffer(B * S * Hq * d * 4), rt.DeviceBuffer(B * Hq * S * 4)
+    dqkv, delta = rt.DeviceBuffer(B * S * w * 4), rt.DeviceBuffer(B * Hq * S * 4)
+    a = rt.AttnArgs(b_qkv.ptr, b_qkv.ptr + Hq * d * 4, b_qkv.ptr + (Hq + Hkv) * d * 4, o.ptr, lse.ptr,
+                    b_do.ptr, dqkv.ptr, dqkv.ptr + Hq * d * 4, dqkv.ptr + (Hq + Hkv) * d * 4, delta.ptr,
+                    w, w, w, Hq * d, Hq * d, w, w, w, B, S, Hq, Hkv, d, int(causal))
+    lib = rt.load()
+    rt.check(lib.jpp_attn_fwd_f32(None, C.byref(a)))
+    rt.check(lib.jpp_attn_bwd_f32(None, C.byref(a)))
+    rt.sync()
+    close(o.download(np.float32, (B, S, Hq, d)), o_w, 1e-5, "o")
+    close(lse.download(np.float32, (B, Hq, S)), lse_w, 1e-5, "lse")
+    got = dqkv.download(np.float32, (B * S, w))
+    close(got[:, :Hq * d].reshape(B, S, Hq, d), dq_w, 1e-5, "dq")
+    close(got[:, Hq * d:(Hq + Hkv) * d].reshape(B, S, Hkv, d), dk_w, 1e-5, "dk")
+    close(got[:, (Hq + Hkv) * d:].reshape(B, S, Hkv, d), dv_w, 1e-5, "dv")
+
+
+def test_colsum_and_mse_f32():
+    rng = np.random.default_rng(9)
+    rows, cols, ld = 300, 200, 256
+    x = rng.standard_normal((rows, ld), dtype=np.float32)
+    acc0 = rng.standard_normal(cols, dtype=np.float32)
+    bx, acc = dev(x), dev(acc0)
+    lib = rt.load()
+    rt.check(lib.jpp_colsum_accum_f32(None, bx.ptr, ld, rows, cols, acc.ptr))
+    rt.sync()
+    close(acc.download(np.float32, (cols,)), acc0 + x[:, :cols].astype(np.float64).sum(0), 1e-5, "colsum")
+    n = 5000
+    out, tgt = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
+    bo, bt, loss, dout = dev(out), dev(tgt), rt.DeviceBuffer(4), rt.DeviceBuffer(n * 4)
+    rt.check(lib.jpp_mse_loss_f32(None, bo.ptr, bt.ptr, n, 0.125, loss.ptr, dout.ptr))
+    rt.sync()
+    d = out.astype(np.float64) - tgt
+    close(loss.download(np.float32, (1,)), np.array([0.125 * (d * d).mean()]), 1e-5, "loss")
+    close(dout.download(np.float32, (n,)), 0.125 * 2 * d / n, 1e-5, "dout")
