@@ -355,7 +355,12 @@ typedef struct {
                             from and ordered against the caller's stream with events; it may
                             still be running when jpp_stage_run_task returns control of the
                             caller's stream - see jpp_stage_join */
+  int dtype;             /* jpp_dtype of parameters, activations and boundary tensors.
+                            JPP_DTYPE_F32: BERT and decoder-block families, through the *_f32
+                            operators; gradient accumulators are f32 either way */
 } jpp_stage_desc;
+
+enum jpp_dtype { JPP_DTYPE_BF16 = 0, JPP_DTYPE_F32 = 1 };
 
 int jpp_stage_create(const jpp_stage_desc* desc, jpp_stage** out);
 int jpp_stage_destroy(jpp_stage* stage);

@@ -72,7 +72,8 @@ struct jpp_stage {
   std::vector<ParamInfo> pinfo;
   std::vector<size_t> poff;        // element offset of parameter i inside a layer block
   size_t layer_elems = 0;
-  bf16_t* params = nullptr;        // [chunk][layer][layer_elems] bf16
+  size_t es = 2;                   // bytes per element of parameters and activations
+  uint8_t* params = nullptr;       // [chunk][layer][layer_elems] bf16 or f32
   float* grads = nullptr;          // same shape, f32
   float* opt[3] = {nullptr, nullptr, nullptr};  // f32 weights, m, v of the optimizer (same shape)
   std::vector<LayerStash> lay;     // per layer of a chunk, offsets into a slot
@@ -103,8 +104,9 @@ struct jpp_stage {
   hipEvent_t ev_tail = nullptr;          // last work queued on `side`
   bool tail_pending = false;
 
-  bf16_t* P(int chunk, int layer, int i) {
-    return params + ((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i];
+  bool f32() const { return d.dtype == JPP_DTYPE_F32; }
+  void* P(int chunk, int layer, int i) {
+    return params + (((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i]) * es;
   }
   float* G(int chunk, int layer, int i) {
     return grads + ((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i];
@@ -118,6 +120,12 @@ namespace {
 enum BertP { B_Wqkv, B_bqkv, B_Wo, B_bo, B_ln1g, B_ln1b, B_W1, B_b1, B_W2, B_b2, B_ln2g, B_ln2b };
 enum LlamaP { L_rms1, L_Wqkv, L_Wo, L_rms2, L_Wgu, L_Wd };
 enum MixtralP { X_rms1, X_Wqkv, X_Wo, X_rms2, X_Wr, X_Wgu, X_Wd };
+
+#define RC(expr)            \
+  do {                      \
+    int rc_ = (expr);       \
+    if (rc_) return rc_;    \
+  } while (0)
 
 int ggemm(hipStream_t st, int mode, const int* seg, int n_seg, const void* a, int64_t lda, int ta,
           const void* b, int64_t ldb, int tb, int64_t stride_b, void* c, int64_t ldc,
@@ -149,7 +157,7 @@ void moe_args(jpp_stage* s, jpp_moe_args& m, uint8_t* slot, const LayerStash& L,
   m.tokens = s->T; m.hidden = s->h; m.n_experts = s->d.n_experts; m.top_k = s->d.top_k;
 }
 
-int gemm(hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int64_t ldb, int tb,
+int gemm(jpp_stage* s, hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int64_t ldb, int tb,
          void* c, int64_t ldc, int64_t m, int64_t n, int64_t k, int epi, const void* bias = nullptr,
          const void* resid = nullptr, int64_t ldr = 0, const void* aux = nullptr,
          int64_t ldaux = 0, void* c2 = nullptr, int64_t ldc2 = 0, int gelu_tanh = 0) {
@@ -159,18 +167,29 @@ int gemm(hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int6
   g.m = m; g.n = n; g.k = k;
   g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldc2 = ldc2; g.ldresid = ldr; g.ldaux = ldaux;
   g.trans_a = ta; g.trans_b = tb; g.epilogue = epi; g.gelu_tanh = gelu_tanh;
-  return jpp_gemm_bf16(st, &g);
+  return s->f32() ? jpp_gemm_f32(st, &g) : jpp_gemm_bf16(st, &g);
 }
 
-#define RC(expr)            \
-  do {                      \
-    int rc_ = (expr);       \
-    if (rc_) return rc_;    \
-  } while (0)
+int attn_f(jpp_stage* s, hipStream_t st, const jpp_attn_args* a) {
+  return s->f32() ? jpp_attn_fwd_f32(st, a) : jpp_attn_fwd(st, a);
+}
+int attn_b(jpp_stage* s, hipStream_t st, const jpp_attn_args* a) {
+  return s->f32() ? jpp_attn_bwd_f32(st, a) : jpp_attn_bwd(st, a);
+}
+
+// a layer's four bias gradients: column sums of the cotangents, added to the accumulators
+int bias_grads4(jpp_stage* s, hipStream_t st, const jpp_colsum_item* items, float* partial) {
+  if (!s->f32()) return jpp_colsum_accum_multi(st, 4, items, s->T, partial);
+  for (int i = 0; i < 4; ++i)
+    RC(jpp_colsum_accum_f32(st, (const float*)items[i].x, items[i].ld, s->T, items[i].cols,
+                            items[i].acc));
+  return JPP_OK;
+}
 
 // dW[rows, cols] (+)= X^T dY, X: [T, rows], dY: [T, cols]
 int wgrad(jpp_stage* s, hipStream_t st, const void* x, int64_t ldx, const void* dy, int64_t lddy,
           float* acc, int64_t rows, int64_t cols) {
+  if (s->f32()) return gemm(s, st, x, ldx, 1, dy, lddy, 1, acc, cols, rows, cols, s->T, JPP_EPI_ACC_F32);
   if (s->d.fused_wgrad_accum) {
     // A weight matrix of at most 128 tiles of 128x128 leaves half of the CUs without work:
     // the contraction over the tokens is then split over `parts` workgroups per tile, which
@@ -194,10 +213,10 @@ int wgrad(jpp_stage* s, hipStream_t st, const void* x, int64_t ldx, const void* 
       RC(jpp_gemm_bf16(st, &g));
       return jpp_sum_accum_f32(st, acc, ws, parts, rows * cols);
     }
-    return gemm(st, x, ldx, 1, dy, lddy, 1, acc, cols, rows, cols, s->T, JPP_EPI_ACC_F32);
+    return gemm(s, st, x, ldx, 1, dy, lddy, 1, acc, cols, rows, cols, s->T, JPP_EPI_ACC_F32);
   }
   void* g = s->S<>(s->s_wg);
-  RC(gemm(st, x, ldx, 1, dy, lddy, 1, g, cols, rows, cols, s->T, JPP_EPI_BF16));
+  RC(gemm(s, st, x, ldx, 1, dy, lddy, 1, g, cols, rows, cols, s->T, JPP_EPI_BF16));
   return jpp_grad_accum_f32(st, acc, g, rows * cols, 0);
 }
 
@@ -207,7 +226,7 @@ int norm_f(jpp_stage* s, hipStream_t st, const void* x, const void* gamma, const
   memset(&a, 0, sizeof(a));
   a.x = x; a.gamma = gamma; a.beta = beta; a.y = y; a.mean = mean; a.rstd = rstd;
   a.rows = s->T; a.cols = s->h; a.eps = s->d.eps;
-  return jpp_norm_fwd(st, &a);
+  return s->f32() ? jpp_norm_fwd_f32(st, &a) : jpp_norm_fwd(st, &a);
 }
 
 int norm_b(jpp_stage* s, hipStream_t st, const void* dy, const void* x, const float* mean,
@@ -219,15 +238,15 @@ int norm_b(jpp_stage* s, hipStream_t st, const void* dy, const void* x, const fl
   a.resid = resid; a.dx = dx; a.dgamma = dgamma; a.dbeta = dbeta;
   a.partial = s->S<float>(s->s_partial);
   a.rows = s->T; a.cols = s->h; a.eps = s->d.eps;
-  return jpp_norm_bwd(st, &a);
+  return s->f32() ? jpp_norm_bwd_f32(st, &a) : jpp_norm_bwd(st, &a);
 }
 
 void attn_args(jpp_stage* s, jpp_attn_args& a, uint8_t* slot, const LayerStash& L) {
   memset(&a, 0, sizeof(a));
-  bf16_t* qkv = (bf16_t*)(slot + L.qkv.off);
+  uint8_t* qkv = slot + L.qkv.off;
   a.q = qkv;
-  a.k = qkv + (int64_t)s->d.n_heads * s->hd;
-  a.v = qkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd;
+  a.k = qkv + (int64_t)s->d.n_heads * s->hd * s->es;
+  a.v = qkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd * s->es;
   a.ldq = a.ldk = a.ldv = s->qkvw;
   a.o = slot + L.ctx.off;
   a.ldo = s->ctxw;
@@ -243,17 +262,17 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
   auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
   jpp_attn_args aa;
   if (s->d.family == JPP_FAMILY_BERT) {
-    RC(gemm(st, at(L.x), h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 1, at(L.qkv), 3 * h, T, 3 * h, h,
+    RC(gemm(s, st, at(L.x), h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 1, at(L.qkv), 3 * h, T, 3 * h, h,
             JPP_EPI_BF16, s->P(chunk, li, B_bqkv)));
     attn_args(s, aa, slot, L);
-    RC(jpp_attn_fwd(st, &aa));
-    RC(gemm(st, at(L.ctx), h, 0, s->P(chunk, li, B_Wo), h, 1, at(L.a), h, T, h, h, JPP_EPI_BF16,
+    RC(attn_f(s, st, &aa));
+    RC(gemm(s, st, at(L.ctx), h, 0, s->P(chunk, li, B_Wo), h, 1, at(L.a), h, T, h, h, JPP_EPI_BF16,
             s->P(chunk, li, B_bo), at(L.x), h));
     RC(norm_f(s, st, at(L.a), s->P(chunk, li, B_ln1g), s->P(chunk, li, B_ln1b), at(L.x1),
               (float*)at(L.mean1), (float*)at(L.rstd1)));
-    RC(gemm(st, at(L.x1), h, 0, s->P(chunk, li, B_W1), f, 1, at(L.u), f, T, f, h, JPP_EPI_GELU,
+    RC(gemm(s, st, at(L.x1), h, 0, s->P(chunk, li, B_W1), f, 1, at(L.u), f, T, f, h, JPP_EPI_GELU,
             s->P(chunk, li, B_b1), nullptr, 0, nullptr, 0, at(L.g), f, s->d.gelu_tanh));
-    RC(gemm(st, at(L.g), f, 0, s->P(chunk, li, B_W2), h, 1, at(L.c), h, T, h, f, JPP_EPI_BF16,
+    RC(gemm(s, st, at(L.g), f, 0, s->P(chunk, li, B_W2), h, 1, at(L.c), h, T, h, f, JPP_EPI_BF16,
             s->P(chunk, li, B_b2), at(L.x1), h));
     RC(norm_f(s, st, at(L.c), s->P(chunk, li, B_ln2g), s->P(chunk, li, B_ln2b), y,
               (float*)at(L.mean2), (float*)at(L.rstd2)));
@@ -263,30 +282,30 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
     // pre-LN block with biases and a GELU feed-forward; parameters as in the BERT layer
     RC(norm_f(s, st, at(L.x), s->P(chunk, li, B_ln1g), s->P(chunk, li, B_ln1b), at(L.n1),
               (float*)at(L.mean1), (float*)at(L.rstd1)));
-    RC(gemm(st, at(L.n1), h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 1, at(L.qkv), 3 * h, T, 3 * h, h,
+    RC(gemm(s, st, at(L.n1), h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 1, at(L.qkv), 3 * h, T, 3 * h, h,
             JPP_EPI_BF16, s->P(chunk, li, B_bqkv)));
     attn_args(s, aa, slot, L);
-    RC(jpp_attn_fwd(st, &aa));
-    RC(gemm(st, at(L.ctx), h, 0, s->P(chunk, li, B_Wo), h, 1, at(L.h1), h, T, h, h, JPP_EPI_BF16,
+    RC(attn_f(s, st, &aa));
+    RC(gemm(s, st, at(L.ctx), h, 0, s->P(chunk, li, B_Wo), h, 1, at(L.h1), h, T, h, h, JPP_EPI_BF16,
             s->P(chunk, li, B_bo), at(L.x), h));
     RC(norm_f(s, st, at(L.h1), s->P(chunk, li, B_ln2g), s->P(chunk, li, B_ln2b), at(L.n2),
               (float*)at(L.mean2), (float*)at(L.rstd2)));
-    RC(gemm(st, at(L.n2), h, 0, s->P(chunk, li, B_W1), f, 1, at(L.u), f, T, f, h, JPP_EPI_GELU,
+    RC(gemm(s, st, at(L.n2), h, 0, s->P(chunk, li, B_W1), f, 1, at(L.u), f, T, f, h, JPP_EPI_GELU,
             s->P(chunk, li, B_b1), nullptr, 0, nullptr, 0, at(L.g), f, s->d.gelu_tanh));
-    RC(gemm(st, at(L.g), f, 0, s->P(chunk, li, B_W2), h, 1, y, h, T, h, f, JPP_EPI_BF16,
+    RC(gemm(s, st, at(L.g), f, 0, s->P(chunk, li, B_W2), h, 1, y, h, T, h, f, JPP_EPI_BF16,
             s->P(chunk, li, B_b2), at(L.h1), h));
     return JPP_OK;
   }
   // llama
   RC(norm_f(s, st, at(L.x), s->P(chunk, li, L_rms1), nullptr, at(L.n1), nullptr,
             (float*)at(L.rstd1)));
-  RC(gemm(st, at(L.n1), h, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 1, at(L.qkv), s->qkvw, T, s->qkvw,
+  RC(gemm(s, st, at(L.n1), h, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 1, at(L.qkv), s->qkvw, T, s->qkvw,
           h, JPP_EPI_BF16));
   RC(jpp_rope(st, at(L.qkv), s->qkvw, s->S<float>(s->s_cos), s->S<float>(s->s_sin), s->d.batch,
               s->d.seq, s->d.n_heads + s->d.n_kv_heads, (int)s->hd, 0));
   attn_args(s, aa, slot, L);
-  RC(jpp_attn_fwd(st, &aa));
-  RC(gemm(st, at(L.ctx), s->ctxw, 0, s->P(chunk, li, L_Wo), h, 1, at(L.h1), h, T, h, s->ctxw,
+  RC(attn_f(s, st, &aa));
+  RC(gemm(s, st, at(L.ctx), s->ctxw, 0, s->P(chunk, li, L_Wo), h, 1, at(L.h1), h, T, h, s->ctxw,
           JPP_EPI_BF16, nullptr, at(L.x), h));
   RC(norm_f(s, st, at(L.h1), s->P(chunk, li, L_rms2), nullptr, at(L.n2), nullptr,
             (float*)at(L.rstd2)));
@@ -308,9 +327,9 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
     return JPP_OK;
   }
   // gate and up columns of Wgu are interleaved in blocks of 32: SwiGLU runs in the epilogue
-  RC(gemm(st, at(L.n2), h, 0, s->P(chunk, li, L_Wgu), 2 * f, 1, at(L.gu), 2 * f, T, 2 * f, h,
+  RC(gemm(s, st, at(L.n2), h, 0, s->P(chunk, li, L_Wgu), 2 * f, 1, at(L.gu), 2 * f, T, 2 * f, h,
           JPP_EPI_SWIGLU, nullptr, nullptr, 0, nullptr, 0, at(L.s), f));
-  RC(gemm(st, at(L.s), f, 0, s->P(chunk, li, L_Wd), h, 1, y, h, T, h, f, JPP_EPI_BF16, nullptr,
+  RC(gemm(s, st, at(L.s), f, 0, s->P(chunk, li, L_Wd), h, 1, y, h, T, h, f, JPP_EPI_BF16, nullptr,
           at(L.h1), h));
   return JPP_OK;
 }
@@ -332,48 +351,48 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     RC(norm_b(s, st, dy, at(L.c), (float*)at(L.mean2), (float*)at(L.rstd2),
               s->P(chunk, li, B_ln2g), nullptr, wt(W.dc), s->G(chunk, li, B_ln2g),
               s->G(chunk, li, B_ln2b)));
-    RC(gemm(st, wt(W.dc), h, 0, s->P(chunk, li, B_W2), h, 0, wt(W.du), f, T, f, h, JPP_EPI_DGELU,
+    RC(gemm(s, st, wt(W.dc), h, 0, s->P(chunk, li, B_W2), h, 0, wt(W.du), f, T, f, h, JPP_EPI_DGELU,
             nullptr, nullptr, 0, at(L.u), f, nullptr, 0, s->d.gelu_tanh));
-    RC(gemm(st, wt(W.du), f, 0, s->P(chunk, li, B_W1), f, 0, dx1, h, T, h, f, JPP_EPI_BF16, nullptr,
+    RC(gemm(s, st, wt(W.du), f, 0, s->P(chunk, li, B_W1), f, 0, dx1, h, T, h, f, JPP_EPI_BF16, nullptr,
             wt(W.dc), h));
     RC(norm_b(s, st, dx1, at(L.a), (float*)at(L.mean1), (float*)at(L.rstd1),
               s->P(chunk, li, B_ln1g), nullptr, wt(W.da), s->G(chunk, li, B_ln1g),
               s->G(chunk, li, B_ln1b)));
-    RC(gemm(st, wt(W.da), h, 0, s->P(chunk, li, B_Wo), h, 0, dctx, h, T, h, h, JPP_EPI_BF16));
+    RC(gemm(s, st, wt(W.da), h, 0, s->P(chunk, li, B_Wo), h, 0, dctx, h, T, h, h, JPP_EPI_BF16));
     attn_args(s, aa, slot, L);
-    bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
+    uint8_t* dqkv = (uint8_t*)wt(W.dqkv);
     aa.d_o = dctx; aa.lddo = h;
-    aa.dq = dqkv; aa.dk = dqkv + h; aa.dv = dqkv + 2 * h;
+    aa.dq = dqkv; aa.dk = dqkv + h * s->es; aa.dv = dqkv + 2 * h * s->es;
     aa.lddq = aa.lddk = aa.lddv = 3 * h;
     aa.delta = s->S<float>(s->s_delta);
-    RC(jpp_attn_bwd(st, &aa));
-    RC(gemm(st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dx, h, T, h, 3 * h,
+    RC(attn_b(s, st, &aa));
+    RC(gemm(s, st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dx, h, T, h, 3 * h,
             JPP_EPI_BF16, nullptr, wt(W.da), h));
     const jpp_colsum_item bias_grads[4] = {{wt(W.dc), h, h, s->G(chunk, li, B_b2)},
                                            {wt(W.du), f, f, s->G(chunk, li, B_b1)},
                                            {wt(W.da), h, h, s->G(chunk, li, B_bo)},
                                            {dqkv, 3 * h, 3 * h, s->G(chunk, li, B_bqkv)}};
-    RC(jpp_colsum_accum_multi(st, 4, bias_grads, T, partial));
+    RC(bias_grads4(s, st, bias_grads, partial));
     return JPP_OK;
   }
   void* dn = s->S<>(s->s_t2);   // dn2, later dn1
   void* dctx = s->S<>(s->s_t3);
   if (s->d.family == JPP_FAMILY_DECODER) {
-    RC(gemm(st, dy, h, 0, s->P(chunk, li, B_W2), h, 0, wt(W.du), f, T, f, h, JPP_EPI_DGELU,
+    RC(gemm(s, st, dy, h, 0, s->P(chunk, li, B_W2), h, 0, wt(W.du), f, T, f, h, JPP_EPI_DGELU,
             nullptr, nullptr, 0, at(L.u), f, nullptr, 0, s->d.gelu_tanh));
-    RC(gemm(st, wt(W.du), f, 0, s->P(chunk, li, B_W1), f, 0, dn, h, T, h, f, JPP_EPI_BF16));
+    RC(gemm(s, st, wt(W.du), f, 0, s->P(chunk, li, B_W1), f, 0, dn, h, T, h, f, JPP_EPI_BF16));
     RC(norm_b(s, st, dn, at(L.h1), (float*)at(L.mean2), (float*)at(L.rstd2),
               s->P(chunk, li, B_ln2g), dy, wt(W.dh1), s->G(chunk, li, B_ln2g),
               s->G(chunk, li, B_ln2b)));
-    RC(gemm(st, wt(W.dh1), h, 0, s->P(chunk, li, B_Wo), h, 0, dctx, h, T, h, h, JPP_EPI_BF16));
+    RC(gemm(s, st, wt(W.dh1), h, 0, s->P(chunk, li, B_Wo), h, 0, dctx, h, T, h, h, JPP_EPI_BF16));
     attn_args(s, aa, slot, L);
-    bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
+    uint8_t* dqkv = (uint8_t*)wt(W.dqkv);
     aa.d_o = dctx; aa.lddo = h;
-    aa.dq = dqkv; aa.dk = dqkv + h; aa.dv = dqkv + 2 * h;
+    aa.dq = dqkv; aa.dk = dqkv + h * s->es; aa.dv = dqkv + 2 * h * s->es;
     aa.lddq = aa.lddk = aa.lddv = 3 * h;
     aa.delta = s->S<float>(s->s_delta);
-    RC(jpp_attn_bwd(st, &aa));
-    RC(gemm(st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dn, h, T, h, 3 * h,
+    RC(attn_b(s, st, &aa));
+    RC(gemm(s, st, dqkv, 3 * h, 0, s->P(chunk, li, B_Wqkv), 3 * h, 0, dn, h, T, h, 3 * h,
             JPP_EPI_BF16));
     RC(norm_b(s, st, dn, at(L.x), (float*)at(L.mean1), (float*)at(L.rstd1),
               s->P(chunk, li, B_ln1g), wt(W.dh1), dx, s->G(chunk, li, B_ln1g),
@@ -382,7 +401,7 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
                                            {wt(W.du), f, f, s->G(chunk, li, B_b1)},
                                            {wt(W.dh1), h, h, s->G(chunk, li, B_bo)},
                                            {dqkv, 3 * h, 3 * h, s->G(chunk, li, B_bqkv)}};
-    RC(jpp_colsum_accum_multi(st, 4, bias_grads, T, partial));
+    RC(bias_grads4(s, st, bias_grads, partial));
     return JPP_OK;
   }
   // llama
@@ -398,14 +417,14 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
              h * 2 * f, dxp, h, 0, s->cap, h, 2 * f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_bwd(st, &ma, dxp, (const float*)wt(W.dlogits), dn));
   } else {
-    RC(gemm(st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, wt(W.dgu), 2 * f, T, f, h, JPP_EPI_DSWIGLU,
+    RC(gemm(s, st, dy, h, 0, s->P(chunk, li, L_Wd), h, 0, wt(W.dgu), 2 * f, T, f, h, JPP_EPI_DSWIGLU,
             nullptr, nullptr, 0, at(L.gu), 2 * f));
-    RC(gemm(st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
+    RC(gemm(s, st, wt(W.dgu), 2 * f, 0, s->P(chunk, li, L_Wgu), 2 * f, 0, dn, h, T, h, 2 * f,
             JPP_EPI_BF16));
   }
   RC(norm_b(s, st, dn, at(L.h1), nullptr, (float*)at(L.rstd2), s->P(chunk, li, L_rms2), dy,
             wt(W.dh1), s->G(chunk, li, L_rms2), nullptr));
-  RC(gemm(st, wt(W.dh1), h, 0, s->P(chunk, li, L_Wo), h, 0, dctx, s->ctxw, T, s->ctxw, h,
+  RC(gemm(s, st, wt(W.dh1), h, 0, s->P(chunk, li, L_Wo), h, 0, dctx, s->ctxw, T, s->ctxw, h,
           JPP_EPI_BF16));
   attn_args(s, aa, slot, L);
   bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
@@ -415,10 +434,10 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
   aa.dv = dqkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd;
   aa.lddq = aa.lddk = aa.lddv = s->qkvw;
   aa.delta = s->S<float>(s->s_delta);
-  RC(jpp_attn_bwd(st, &aa));
+  RC(attn_b(s, st, &aa));
   RC(jpp_rope(st, dqkv, s->qkvw, s->S<float>(s->s_cos), s->S<float>(s->s_sin), s->d.batch,
               s->d.seq, s->d.n_heads + s->d.n_kv_heads, (int)s->hd, 1));
-  RC(gemm(st, dqkv, s->qkvw, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 0, dn, h, T, h, s->qkvw,
+  RC(gemm(s, st, dqkv, s->qkvw, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 0, dn, h, T, h, s->qkvw,
           JPP_EPI_BF16));
   RC(norm_b(s, st, dn, at(L.x), nullptr, (float*)at(L.rstd1), s->P(chunk, li, L_rms1), wt(W.dh1),
             dx, s->G(chunk, li, L_rms1), nullptr));
@@ -470,7 +489,7 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
 }
 
 void carve_layer(jpp_stage* s, Carver& c, LayerStash& L, bool with_w) {
-  const size_t T = s->T, h = s->h, f = s->f, e = 2;
+  const size_t T = s->T, h = s->h, f = s->f, e = s->es;
   const size_t stat = (size_t)s->d.batch * s->d.n_heads * s->d.seq * 4;
   L.x = c.take(T * h * e);
   L.qkv = c.take(T * s->qkvw * e);
@@ -516,7 +535,7 @@ void carve_layer(jpp_stage* s, Carver& c, LayerStash& L, bool with_w) {
 }
 
 void carve_w(jpp_stage* s, Carver& c, LayerStash& L) {
-  const size_t T = s->T, h = s->h, f = s->f, e = 2;
+  const size_t T = s->T, h = s->h, f = s->f, e = s->es;
   L.dqkv = c.take(T * s->qkvw * e);
   if (s->d.family == JPP_FAMILY_BERT) {
     L.dc = c.take(T * h * e);
@@ -576,8 +595,17 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
     JPP_REQUIRE(kvh == d->n_heads && d->n_heads * hd == d->hidden,
                 "stage_create: the decoder block needs n_heads*head_dim == hidden and no GQA");
 
+  JPP_REQUIRE(d->dtype == JPP_DTYPE_BF16 || d->dtype == JPP_DTYPE_F32, "stage_create: unknown dtype %d",
+              d->dtype);
+  if (d->dtype == JPP_DTYPE_F32)
+    JPP_REQUIRE((d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_DECODER) &&
+                    d->fused_wgrad_accum,
+                "stage_create: f32 stages exist for the BERT and decoder-block families, with "
+                "the accumulation in the weight-gradient GEMM");
+
   jpp_stage* s = new jpp_stage();
   s->d = *d;
+  s->es = d->dtype == JPP_DTYPE_F32 ? 4 : 2;
   s->d.n_kv_heads = kvh;
   s->d.head_dim = hd;
   s->T = T; s->h = d->hidden; s->f = d->ffn; s->hd = hd;
@@ -616,7 +644,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   Carver sc;
   if (!d->split_backward)
     for (int i = 0; i < (d->two_streams ? 3 : 1); ++i) carve_w(s, sc, s->wsets[i]);
-  const size_t e = 2;
+  const size_t e = s->es;
   s->s_dx[0] = sc.take(T * h * e);
   s->s_dx[1] = sc.take(T * h * e);
   const size_t rows_t = d->family == JPP_FAMILY_MIXTRAL ? (size_t)s->cap : (size_t)T;
@@ -644,7 +672,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   s->scratch_bytes = sc.total;
 
   const size_t n_layers = (size_t)d->n_chunks * d->layers_per_chunk;
-  hipError_t e1 = hipMalloc((void**)&s->params, n_layers * s->layer_elems * 2);
+  hipError_t e1 = hipMalloc((void**)&s->params, n_layers * s->layer_elems * s->es);
   hipError_t e2 = e1 == hipSuccess ? hipMalloc((void**)&s->grads, n_layers * s->layer_elems * 4)
                                    : e1;
   hipError_t e3 = e2 == hipSuccess ? hipMalloc((void**)&s->scratch, s->scratch_bytes) : e2;
@@ -663,8 +691,9 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
     return jpp_set_error(JPP_ERR_HIP, "stage_create: allocation failed: %s",
                          hipGetErrorString(e4));
   }
-  s->total_bytes = n_layers * s->layer_elems * 6 + s->scratch_bytes + s->slot_bytes * d->max_live;
-  hipMemset(s->params, 0, n_layers * s->layer_elems * 2);
+  s->total_bytes = n_layers * s->layer_elems * (4 + s->es) + s->scratch_bytes +
+                   s->slot_bytes * d->max_live;
+  hipMemset(s->params, 0, n_layers * s->layer_elems * s->es);
   hipMemset(s->grads, 0, n_layers * s->layer_elems * 4);
 
   {
@@ -789,7 +818,7 @@ int jpp_stage_optimizer_init(jpp_stage* s, void* stream) {
   JPP_REQUIRE(s, "stage: null");
   const size_t n = (size_t)s->d.n_chunks * s->d.layers_per_chunk * s->layer_elems;
   for (auto& p : s->opt)
-    if (!p) {
+    if (!p && !(s->f32() && &p == &s->opt[0])) {   // f32 parameters are their own f32 weights
       if (hipMalloc((void**)&p, n * 4) != hipSuccess) {
         p = nullptr;
         (void)hipGetLastError();
@@ -797,7 +826,7 @@ int jpp_stage_optimizer_init(jpp_stage* s, void* stream) {
       }
       s->total_bytes += n * 4;
     }
-  RC(jpp_cast_bf16_to_f32(stream, s->params, s->opt[0], (int64_t)n));
+  if (!s->f32()) RC(jpp_cast_bf16_to_f32(stream, s->params, s->opt[0], (int64_t)n));
   RC(jpp_fill_u32(s->opt[1], 0u, n, stream));
   return jpp_fill_u32(s->opt[2], 0u, n, stream);
 }
@@ -806,22 +835,24 @@ int jpp_stage_opt_ptr(jpp_stage* s, int which, int chunk, int layer, int i, floa
   RC(check_pli(s, chunk, layer, i));
   JPP_REQUIRE(which >= 0 && which < 3, "opt_ptr: which = %d, expected 0 (weights), 1 (m) or 2 (v)",
               which);
-  JPP_REQUIRE(s->opt[which], "opt_ptr: jpp_stage_optimizer_init has not run");
-  *ptr = s->opt[which] + (s->G(chunk, layer, i) - s->grads);
+  JPP_REQUIRE(s->opt[which == 0 && s->f32() ? 1 : which],
+              "opt_ptr: jpp_stage_optimizer_init has not run");
+  float* base = which == 0 && s->f32() ? (float*)s->params : s->opt[which];
+  *ptr = base + (s->G(chunk, layer, i) - s->grads);
   return JPP_OK;
 }
 
 int jpp_stage_adam_step(jpp_stage* s, void* stream, int64_t step, double lr, double beta1,
                         double beta2, double eps, double grad_scale) {
   JPP_REQUIRE(s, "stage: null");
-  JPP_REQUIRE(s->opt[0] && s->opt[1] && s->opt[2],
+  JPP_REQUIRE((s->opt[0] || s->f32()) && s->opt[1] && s->opt[2],
               "adam_step: jpp_stage_optimizer_init has not run");
   RC(jpp_stage_join(s, stream));  // weight gradients may still be running on the second stream
   jpp_adam_args a;
   a.count = (int64_t)s->d.n_chunks * s->d.layers_per_chunk * (int64_t)s->layer_elems;
   a.grad = s->grads;
-  a.master = s->opt[0];
-  a.param = s->params;
+  a.master = s->f32() ? (float*)s->params : s->opt[0];
+  a.param = s->f32() ? nullptr : s->params;
   a.m = s->opt[1];
   a.v = s->opt[2];
   a.step = step;
@@ -840,7 +871,7 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
   JPP_REQUIRE(chunk >= 0 && chunk < s->d.n_chunks, "run_task: chunk %d out of range", chunk);
   hipStream_t st = (hipStream_t)stream;
   const int nl = s->d.layers_per_chunk;
-  const size_t act = (size_t)s->T * s->h * 2;
+  const size_t act = (size_t)s->T * s->h * s->es;
   const auto key = std::make_pair(chunk, mb);
 
   if (kind == JPP_FWD) {

@@ -85,12 +85,13 @@ class StageDesc(C.Structure):
                 ("n_experts", C.c_int), ("top_k", C.c_int), ("n_chunks", C.c_int),
                 ("layers_per_chunk", C.c_int), ("max_live", C.c_int),
                 ("split_backward", C.c_int), ("fused_wgrad_accum", C.c_int),
-                ("two_streams", C.c_int)]
+                ("two_streams", C.c_int), ("dtype", C.c_int)]
 
 
 EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32, EPI_SWIGLU, EPI_DSWIGLU = range(7)
 NORM_PARTIALS = 256
 FAMILY = {"bert": 0, "llama": 1, "mixtral": 2, "decoder": 3}
+DTYPE = {"bf16": 0, "f32": 1}
 
 # every symbol include/jaxpp_amd.h declares
 EXPORTS = [
@@ -464,12 +465,13 @@ class StageExecutor:
                  two_streams: bool = False):
         require_gpu()
         self.spec = spec
+        self.dtype = getattr(spec, "dtype", "bf16")
         self.n_chunks, self.layers_per_chunk = n_chunks, layers_per_chunk
         d = StageDesc(FAMILY[spec.family], spec.hidden, spec.n_heads, spec.kvh, spec.d, spec.ffn,
                       spec.seq, spec.batch, int(spec.causal), spec.rope_theta, spec.eps,
                       int(spec.gelu_tanh), spec.n_experts, spec.top_k, n_chunks,
                       layers_per_chunk, max_live, int(split_backward), int(fused_wgrad_accum),
-                      int(two_streams))
+                      int(two_streams), DTYPE[self.dtype])
         h = C.c_void_p()
         check(load().jpp_stage_create(C.byref(d), C.byref(h)))
         self.handle = h.value
@@ -503,7 +505,7 @@ class StageExecutor:
         return np.where(w < 32, 32 * q + w, f + 32 * q + w - 32)
 
     def set_params(self, chunk: int, layer: int, params: dict):
-        """Upload float32 host arrays as bf16 device parameters."""
+        """Upload float32 host arrays as device parameters (bf16, or f32 for an f32 stage)."""
         for name, rows, cols in self.params:
             a = np.asarray(params[name], dtype=np.float32)
             assert a.size == rows * cols, (name, a.shape, rows, cols)
@@ -511,17 +513,19 @@ class StageExecutor:
             if order is not None:
                 a = np.ascontiguousarray(a.reshape(rows, cols)[:, order])
             upload_ptr(self._ptr(load().jpp_stage_param_ptr, chunk, layer, name),
-                       to_bf16_bits(a))
+                       a if self.dtype == "f32" else to_bf16_bits(a))
 
     def get_params(self, chunk: int, layer: int) -> dict:
-        """The bf16 device parameters as float32 host arrays."""
+        """The device parameters as float32 host arrays."""
         self.join()
         out = {}
         for name, rows, cols in self.params:
             shape = (cols,) if rows == 1 and not name.startswith("W") else (rows, cols)
-            bits = download_ptr(self._ptr(load().jpp_stage_param_ptr, chunk, layer, name),
-                                np.uint16, shape)
-            a = from_bf16_bits(bits)
+            ptr = self._ptr(load().jpp_stage_param_ptr, chunk, layer, name)
+            if self.dtype == "f32":
+                a = download_ptr(ptr, np.float32, shape)
+            else:
+                a = from_bf16_bits(download_ptr(ptr, np.uint16, shape))
             order = self._device_columns(name, cols)
             if order is not None:
                 host = np.empty_like(a)
@@ -544,6 +548,19 @@ class StageExecutor:
                 g = host
             out[name] = g
         return out
+
+    def upload_activation(self, a: np.ndarray) -> "DeviceBuffer":
+        """A float32 host array as a device tensor of the stage's element type."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        return DeviceBuffer.from_numpy(a if self.dtype == "f32" else to_bf16_bits(a))
+
+    def new_activation(self) -> "DeviceBuffer":
+        return DeviceBuffer(self.spec.tokens * self.spec.hidden * (4 if self.dtype == "f32" else 2))
+
+    def download_activation(self, buf: "DeviceBuffer", shape) -> np.ndarray:
+        if self.dtype == "f32":
+            return buf.download(np.float32, shape)
+        return buf.download_bf16(shape)
 
     def zero_grads(self, stream=None):
         check(load().jpp_stage_zero_grads(self.handle, stream))

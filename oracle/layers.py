@@ -92,6 +92,7 @@ class LayerCfg:
     gelu_tanh: bool = False
     n_experts: int = 0
     top_k: int = 0
+    dtype: str = "bf16"              # element type of parameters and activations: "bf16" | "f32"
 
     @property
     def kvh(self) -> int:

@@ -187,3 +187,59 @@ def test_colsum_and_mse_f32():
     d = out.astype(np.float64) - tgt
     close(loss.download(np.float32, (1,)), np.array([0.125 * (d * d).mean()]), 1e-5, "loss")
     close(dout.download(np.float32, (n,)), 0.125 * 2 * d / n, 1e-5, "dout")
+
+
+# ---------------------------------------------------------------------------
+# whole stages in f32 against the oracle's f32 numerics
+# ---------------------------------------------------------------------------
+from jaxpp_amd import schedules as S                      # noqa: E402
+from jaxpp_amd.model import LayerSpec, init_layer_params  # noqa: E402
+from jaxpp_amd.plan import make_rank_plan                 # noqa: E402
+
+from test_gpu_stage import run_on_gpu, run_on_oracle      # noqa: E402
+
+# the CPU-runnable configuration: post-LN encoder layers of hidden 256, 4 heads, FFN 1024,
+# 128-token sequences in microbatches of 4, two stages of two layers, Std1F1B, 8 microbatches
+CFG1 = LayerSpec("bert", 256, 4, 1024, 128, 4, eps=1e-12, dtype="f32")
+DECODER_F32 = LayerSpec("decoder", 256, 2, 512, 128, 2, causal=True, eps=1e-6, gelu_tanh=True,
+                        dtype="f32")
+BERT_D64_F32 = LayerSpec("bert", 128, 2, 256, 256, 1, eps=1e-5, dtype="f32")
+
+STAGES_F32 = [
+    ("cfg1-rank0", CFG1, S.Std1F1B(2), 8, 0, 2),
+    ("cfg1-rank1", CFG1, S.Std1F1B(2), 8, 1, 2),
+    ("bert-zb", BERT_D64_F32, S.ZeroBubble(2), 3, 1, 2),
+    ("bert-zb-first-stage", BERT_D64_F32, S.ZeroBubble(2), 2, 0, 1),
+    ("decoder-1f1b", DECODER_F32, S.Std1F1B(2), 3, 1, 2),
+    ("decoder-zb", DECODER_F32, S.ZeroBubble(2), 3, 1, 1),
+    ("decoder-interleaved", DECODER_F32, S.Interleaved1F1B(4, 2), 4, 0, 1),
+]
+
+
+@pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
+@pytest.mark.parametrize("name,spec,sched,n,rank,lpc", STAGES_F32, ids=[c[0] for c in STAGES_F32])
+def test_f32_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
+    print(f"f32 stage case {name} two_streams={two_streams}", flush=True)
+    plan = make_rank_plan(sched, n, rank)
+    params = {s: [init_layer_params(spec, 3, s * lpc + li, perturb=True) for li in range(lpc)]
+              for s in plan.stages}
+    row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
+    ys_w, dxs_w, acc_w = run_on_oracle(spec, plan, params, row)
+    ys, dxs, grads = run_on_gpu(spec, plan, lpc, params, two_streams=two_streams)
+    assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
+    for k in ys_w:
+        close(ys[k], ys_w[k].astype(np.float64), 1e-4, f"y{k}")
+    for k in dxs_w:
+        close(dxs[k], dxs_w[k].astype(np.float64), 1e-4, f"dx{k}")
+    for s in plan.stages:
+        for li in range(lpc):
+            for pname, want in acc_w[s][li].items():
+                got = grads[s][li][pname]
+                close(got, want.reshape(got.shape).astype(np.float64), 1e-4, f"grad {s}/{li}/{pname}")
+
+
+def test_f32_stage_needs_a_family_with_f32_operators():
+    spec = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
+                     dtype="f32")
+    with pytest.raises(rt.JppError, match="f32 stages exist for"):
+        rt.StageExecutor(spec, 1, 1, 1)

@@ -59,9 +59,8 @@ def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_str
         t = pt.task
         kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
         key = (kind, t.stage_id, t.mubatch_idx)
-        ins[key] = rt.DeviceBuffer.from_f32_as_bf16(
-            boundary_tensor(kind, t.stage_id, t.mubatch_idx, shape, seed))
-        outs[key] = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+        ins[key] = ex.upload_activation(boundary_tensor(kind, t.stage_id, t.mubatch_idx, shape, seed))
+        outs[key] = ex.new_activation()
 
     def io(pt, lane=0):
         kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
@@ -81,8 +80,8 @@ def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_str
     ex.join()
     rt.sync()
     assert ex.live_slots() == 0
-    ys = {k[1:]: b.download_bf16(shape) for k, b in outs.items() if k[0] == "x"}
-    dxs = {k[1:]: b.download_bf16(shape) for k, b in outs.items() if k[0] == "dy"}
+    ys = {k[1:]: ex.download_activation(b, shape) for k, b in outs.items() if k[0] == "x"}
+    dxs = {k[1:]: ex.download_activation(b, shape) for k, b in outs.items() if k[0] == "dy"}
     grads = {stage: [ex.get_grads(c, li) for li in range(layers_per_chunk)]
              for c, stage in enumerate(plan.stages)}
     ex.close()
@@ -92,10 +91,13 @@ def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_str
 def run_on_oracle(spec, plan, params, row, seed=0):
     cfg = L.LayerCfg(**spec.as_dict())
     shape = (spec.tokens, spec.hidden)
-    ro = O.RankOracle(cfg, {s: params[s] for s in plan.stages}, L.Numerics.bf16())
+    f32 = spec.dtype == "f32"
+    rnd = (lambda a: a) if f32 else L.bf16_round
+    ro = O.RankOracle(cfg, {s: params[s] for s in plan.stages},
+                      L.Numerics.f32() if f32 else L.Numerics.bf16())
     ys, dxs = ro.run_row(row,
-                         lambda s, m: L.bf16_round(boundary_tensor("x", s, m, shape, seed)),
-                         lambda s, m: L.bf16_round(boundary_tensor("dy", s, m, shape, seed)))
+                         lambda s, m: rnd(boundary_tensor("x", s, m, shape, seed)),
+                         lambda s, m: rnd(boundary_tensor("dy", s, m, shape, seed)))
     return ys, dxs, ro.acc
 
 
