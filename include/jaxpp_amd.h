@@ -330,7 +330,7 @@ int jpp_moe_router_wgrad(void* stream, const jpp_moe_args* args, const void* x,
 
 /* ---- stage executor: stands in for `task_impl` on one pipeline rank ----------
  * A stage object holds this rank's chunks (the stages the schedule places on
- * it), their bf16 parameters, the f32 gradient accumulators (the loop carry of
+ * it), their parameters (bf16, or f32: `dtype`), the f32 gradient accumulators (the loop carry of
  * `treduce`), and a ring of residual slots sized for the schedule's peak
  * number of live microbatches (src/jaxpp/core.py:1732-1890 decides the same
  * lifetimes by donation and explicit deletes). */

@@ -322,12 +322,13 @@ def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSche
     act_elems = spec.tokens * spec.hidden
     if x.shape[1:] != (spec.tokens, spec.hidden):
         x = x.reshape(n, spec.tokens, spec.hidden)
-    xs_dev = [rt.DeviceBuffer.from_f32_as_bf16(x[m]) for m in range(n)]
+    f32 = spec.dtype == "f32"           # an f32 model runs through the f32 operators
+    xs_dev = [execs[0].upload_activation(x[m]) for m in range(n)]
     act, cot = {}, {}                   # (stage, mb) -> DeviceBuffer
     free = []
 
     def take():
-        return free.pop() if free else rt.DeviceBuffer(act_elems * 2)
+        return free.pop() if free else execs[0].new_activation()
 
     loss_dev = rt.DeviceBuffer(4 * n)
     partial = rt.DeviceBuffer(4 * rt.NORM_PARTIALS)
@@ -362,12 +363,17 @@ def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSche
                     if body.loss_scale is None:
                         raise AssertionError("the last stage has no loss to differentiate")
                     d = take()
-                    rt.check(lib.jpp_mse_loss(None, dst.ptr, xs_dev[m].ptr, act_elems,
-                                              float(loss_scale), loss_dev.ptr + 4 * m, d.ptr,
-                                              partial.ptr))
+                    if f32:
+                        rt.check(lib.jpp_mse_loss_f32(None, dst.ptr, xs_dev[m].ptr, act_elems,
+                                                      float(loss_scale), loss_dev.ptr + 4 * m,
+                                                      d.ptr))
+                    else:
+                        rt.check(lib.jpp_mse_loss(None, dst.ptr, xs_dev[m].ptr, act_elems,
+                                                  float(loss_scale), loss_dev.ptr + 4 * m, d.ptr,
+                                                  partial.ptr))
                     cot[s, m] = d
                     if want_pred:
-                        preds[m] = dst.download_bf16((spec.tokens, spec.hidden))
+                        preds[m] = execs[r].download_activation(dst, (spec.tokens, spec.hidden))
                     free.append(dst)
             elif kind is TaskType.BWD_W:
                 execs[r].run_task(kind, c, m)

@@ -243,3 +243,95 @@ def test_f32_stage_needs_a_family_with_f32_operators():
                      dtype="f32")
     with pytest.raises(rt.JppError, match="f32 stages exist for"):
         rt.StageExecutor(spec, 1, 1, 1)
+
+
+def test_cfg1_train_step_through_the_public_api():
+    """The CPU-runnable configuration end to end in float32: 4 post-LN encoder layers of hidden
+    256 in 2 stages, 8 microbatches of 4 x 128 tokens, Std1F1B, loss mean((out - in)^2) / 8 -
+    losses and accumulated gradients against the sequential loop in the oracle's f32 numerics,
+    to the 1e-4 stated for fp32 results."""
+    from functools import partial
+
+    import jaxpp_amd as jaxpp
+    from oracle import stage as O
+
+    n_mb, pp, n_layers = 8, 2, 4
+    model = jaxpp.nn.TransformerStack(CFG1, n_layers=n_layers, layers_per_stage=n_layers // pp)
+    params = model.init(seed=0, perturb=True)
+    batch = np.random.default_rng(1).standard_normal((n_mb, CFG1.tokens, CFG1.hidden),
+                                                     dtype=np.float32)
+    mesh = jaxpp.MpmdMesh(jaxpp.DeviceMesh(np.arange(pp).reshape(pp, 1), ("mpmd", "data")), "mpmd")
+    schedule = jaxpp.Std1F1B(pp)
+
+    def loss_fn(pars, mb):
+        res = model.apply(pars, mb)
+        return jaxpp.nn.mse_loss(res, mb) / n_mb, (res, 4)
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=mesh)
+    def train_step(pars, batch):
+        mubatch_grad = partial(jaxpp.value_and_grad(loss_fn, has_aux=True), pars)
+        (losses, (pred, _)), grad = jaxpp.treduce(mubatch_grad, batch, schedule=schedule)
+        return losses, pred, grad
+
+    losses, pred, grad = train_step(params, batch)
+    cfg = L.LayerCfg(**CFG1.as_dict())
+    per = n_layers // pp
+    stages = [params["layers"][s * per:(s + 1) * per] for s in range(pp)]
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.f32())
+    close(losses, want_loss.astype(np.float64), 1e-4, "losses")
+    assert pred.shape == batch.shape and np.isfinite(pred).all()
+    for s in range(pp):
+        for li in range(per):
+            for k, v in want_acc[s][li].items():
+                got = grad["layers"][s * per + li][k]
+                close(got, v.reshape(got.shape).astype(np.float64), 1e-4, f"grad {s}/{li}/{k}")
+    train_step.close()
+
+
+def test_f32_stage_adam_after_loop():
+    """Two train steps of an f32 rank: the parameters are their own f32 weights (no second
+    copy), Adam rewrites them in place and clears the accumulators."""
+    from jaxpp_amd.model import boundary_tensor
+    from jaxpp_amd.rank_loop import RankLoop
+    from jaxpp_amd.types import TaskType
+    from oracle import stage as O
+
+    spec, schedule, n_mb, rank, lpc = CFG1, S.Std1F1B(2), 4, 1, 2
+    plan = make_rank_plan(schedule, n_mb, rank)
+    shape = (spec.tokens, spec.hidden)
+    ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True, False)
+    host = [init_layer_params(spec, 3, li, perturb=True) for li in range(lpc)]
+    for li in range(lpc):
+        ex.set_params(0, li, host[li])
+    ex.optimizer_init()
+    bufs = {}
+
+    def io(pt, lane=0):
+        kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
+        key = (kind, pt.task.stage_id, pt.task.mubatch_idx)
+        if key not in bufs:
+            bufs[key] = (ex.upload_activation(boundary_tensor(kind, *key[1:], shape, 0)),
+                         ex.new_activation())
+        return bufs[key][0].ptr, bufs[key][1].ptr
+
+    m = [{k: np.zeros_like(v) for k, v in p.items()} for p in host]
+    v = [{k: np.zeros_like(v_) for k, v_ in p.items()} for p in host]
+    w = [dict(p) for p in host]
+    for step in (1, 2):
+        RankLoop(ex, plan).run(io)
+        grads = [ex.get_grads(0, li) for li in range(lpc)]
+        ex.adam_step(step, lr=1e-3, grad_scale=1.0 / n_mb)
+        rt.sync()
+        for li in range(lpc):
+            g = {k: a.reshape(host[li][k].shape) * np.float32(1.0 / n_mb) for k, a in grads[li].items()}
+            w[li] = O.adam_step(w[li], g, m[li], v[li], step, 1e-3)
+            state, new_p = ex.get_opt_state(0, li), ex.get_params(0, li)
+            for k in host[li]:
+                gw, gm, gv = (a.reshape(host[li][k].shape) for a in state[k])
+                close(gm, m[li][k].astype(np.float64), 2e-6, f"step {step} m[{k}]")
+                close(gv, v[li][k].astype(np.float64), 2e-6, f"step {step} v[{k}]")
+                close(gw, w[li][k].astype(np.float64), 2e-6, f"step {step} weights[{k}]")
+                assert np.array_equal(new_p[k].reshape(gw.shape), gw), k
+                assert np.abs(gw - host[li][k]).max() > 0, f"{k} did not move"
+            assert all(not a.any() for a in ex.get_grads(0, li).values())
+    ex.close()
