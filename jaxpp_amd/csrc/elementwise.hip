@@ -183,6 +183,130 @@ __global__ __launch_bounds__(kNormBwdWaves * 64) void norm_bwd_kernel(
   }
 }
 
+// Rows of 4096 or 8192 columns: a row is spread over the 8 waves of a workgroup (a lane owns
+// NCHB pieces of 8 columns), R rows at a time.  The wave-per-row kernel above needs the row,
+// its gradient and 8 partial sums per piece in registers - 200 to 256 registers and, at 8192
+// columns, spills - so few waves fit a CU and each waits out its own loads.  Here a lane holds
+// 12 registers per row, the loads of R rows are in flight together, and the price is one
+// barrier per R rows for the row sums (wave sums meet in LDS and are added in wave order).
+// Every column belongs to one lane of the workgroup, so its partial sums of the scale / shift
+// gradients leave without a reduction across waves; summation orders are fixed throughout.
+__device__ __forceinline__ void keep_packed(uint4& v) {
+  asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+}
+
+template <bool LN, int NCHB, int R>
+__global__ __launch_bounds__(512) void norm_bwd_wide_kernel(
+    const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x, const float* __restrict__ mean_in,
+    const float* __restrict__ rstd_in, const bf16_t* __restrict__ gamma,
+    const bf16_t* __restrict__ resid, bf16_t* __restrict__ dx, float* __restrict__ partial,
+    long rows, int cols) {
+  __shared__ float red[2][R][8][2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float g[NCHB][8], pg[NCHB][8], pb[LN ? NCHB : 1][8];
+#pragma unroll
+  for (int i = 0; i < NCHB; ++i) {
+    unpack8(((const uint4*)gamma)[tid + 512 * i], g[i]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pg[i][e] = 0.f;
+      if (LN) pb[i][e] = 0.f;
+    }
+  }
+  int par = 0;
+  for (long r0 = (long)blockIdx.x * R; r0 < rows; r0 += (long)gridDim.x * R, par ^= 1) {
+    uint4 vx[R][NCHB], vd[R][NCHB], vr[R][NCHB];
+    float rstd[R], mean[R];
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+      const long row = min(r0 + q, rows - 1);   // rows past the end repeat the last one, unused
+      rstd[q] = rstd_in[row];
+      mean[q] = LN ? mean_in[row] : 0.f;
+#pragma unroll
+      for (int i = 0; i < NCHB; ++i) {
+        const long at = row * (cols / 8) + tid + 512 * i;
+        vx[q][i] = ((const uint4*)x)[at];
+        vd[q][i] = ((const uint4*)dy)[at];
+        if (resid) vr[q][i] = ((const uint4*)resid)[at];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+      float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+      for (int i = 0; i < NCHB; ++i) {
+        float fx[8], fd[8];
+        unpack8(vx[q][i], fx);
+        unpack8(vd[q][i], fd);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float dg = fd[e] * g[i][e];
+          s1 += dg;
+          s2 += dg * ((fx[e] - mean[q]) * rstd[q]);
+        }
+      }
+      s2 = wave_sum(s2);
+      if (LN) s1 = wave_sum(s1);
+      if (lane == 0) {
+        red[par][q][wave][0] = s1;
+        red[par][q][wave][1] = s2;
+      }
+    }
+    __syncthreads();
+    // the rows stay packed across the barrier: without this the compiler keeps the unpacked
+    // f32 values of all R rows alive instead (three times the registers)
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int i = 0; i < NCHB; ++i) {
+        keep_packed(vx[q][i]);
+        keep_packed(vd[q][i]);
+        if (resid) keep_packed(vr[q][i]);
+      }
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+      if (r0 + q >= rows) break;
+      float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        s1 += red[par][q][w][0];
+        s2 += red[par][q][w][1];
+      }
+      s2 /= cols;
+      s1 = LN ? s1 / cols : 0.f;
+#pragma unroll
+      for (int i = 0; i < NCHB; ++i) {
+        float fx[8], fd[8], r[8];
+        unpack8(vx[q][i], fx);
+        unpack8(vd[q][i], fd);
+        if (resid) unpack8(vr[q][i], r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xh = (fx[e] - mean[q]) * rstd[q];
+          pg[i][e] += fd[e] * xh;
+          if (LN) pb[i][e] += fd[e];
+          float o = (fd[e] * g[i][e] - s1 - xh * s2) * rstd[q];
+          if (resid) o += r[e];
+          fx[e] = o;
+        }
+        ((uint4*)dx)[(r0 + q) * (cols / 8) + tid + 512 * i] = pack8(fx);
+      }
+    }
+  }
+  float* pgam = partial + (long)blockIdx.x * cols;
+  float* pbet = partial + ((long)gridDim.x + blockIdx.x) * cols;
+#pragma unroll
+  for (int i = 0; i < NCHB; ++i) {
+    const int c = (tid + 512 * i) * 8;
+    *(float4*)(pgam + c) = make_float4(pg[i][0], pg[i][1], pg[i][2], pg[i][3]);
+    *(float4*)(pgam + c + 4) = make_float4(pg[i][4], pg[i][5], pg[i][6], pg[i][7]);
+    if (LN) {
+      *(float4*)(pbet + c) = make_float4(pb[i][0], pb[i][1], pb[i][2], pb[i][3]);
+      *(float4*)(pbet + c + 4) = make_float4(pb[i][4], pb[i][5], pb[i][6], pb[i][7]);
+    }
+  }
+}
+
 // acc[j] += sum_b partial[b][j]: a block owns 32 columns; 32 thread groups sum interleaved
 // subsets of the partials (8 independent loads each for 256 partials), then one combines them
 // in a fixed order.  blockIdx.y picks one of two reductions (gamma and beta of a LayerNorm
@@ -503,12 +627,20 @@ int launch_norm_bwd(hipStream_t st, const jpp_norm_args* a) {
                      (const bf16_t*)a->dy, (const bf16_t*)a->x, a->mean, a->rstd,             \
                      (const bf16_t*)a->gamma, (const bf16_t*)a->resid, (bf16_t*)a->dx,        \
                      a->partial, (long)a->rows, (int)a->cols)
-  if (nch <= 1) JPP_NB(1);
+#define JPP_NBW(N)                                                                            \
+  hipLaunchKernelGGL((norm_bwd_wide_kernel<LN, N, 4>), dim3(blocks), dim3(512), 0, st,         \
+                     (const bf16_t*)a->dy, (const bf16_t*)a->x, a->mean, a->rstd,             \
+                     (const bf16_t*)a->gamma, (const bf16_t*)a->resid, (bf16_t*)a->dx,        \
+                     a->partial, (long)a->rows, (int)a->cols)
+  if (a->cols == 4096) JPP_NBW(1);
+  else if (a->cols == 8192) JPP_NBW(2);
+  else if (nch <= 1) JPP_NB(1);
   else if (nch <= 2) JPP_NB(2);
   else if (nch <= 4) JPP_NB(4);
   else if (nch <= 8) JPP_NB(8);
   else JPP_NB(16);
 #undef JPP_NB
+#undef JPP_NBW
   JPP_LAUNCH_CHECK();
   const int cb = (int)((a->cols + 31) / 32);
   hipLaunchKernelGGL(partial_reduce_kernel, dim3(cb, LN ? 2 : 1), dim3(1024), 0, st, a->partial,
