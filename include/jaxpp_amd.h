@@ -253,14 +253,16 @@ int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t coun
  * hidden 256; tests/test_transformations.py:44-118 also builds its model in float32).
  * Same argument structs, every bf16 tensor replaced by an f32 one; plain fp32 arithmetic
  * in a fixed summation order, sized for small problems (not for the matrix cores).
- * jpp_gemm_f32: M, N multiples of 64, K of 16; epilogues JPP_EPI_BF16 (= store, with bias
- * and residual), JPP_EPI_F32, JPP_EPI_GELU, JPP_EPI_DGELU, JPP_EPI_ACC_F32; no groups.
+ * jpp_gemm_f32: M, N multiples of 64, K of 16; every epilogue of jpp_gemm_bf16
+ * (JPP_EPI_BF16 = store in the element type, with bias and residual); no groups.
  * jpp_attn_*_f32: seq a multiple of 64.  jpp_norm_bwd_f32 does not use `partial`. */
 int jpp_gemm_f32(void* stream, const jpp_gemm_args* args);
 int jpp_attn_fwd_f32(void* stream, const jpp_attn_args* args);
 int jpp_attn_bwd_f32(void* stream, const jpp_attn_args* args);
 int jpp_norm_fwd_f32(void* stream, const jpp_norm_args* args);
 int jpp_norm_bwd_f32(void* stream, const jpp_norm_args* args);
+int jpp_rope_f32(void* stream, float* x, int64_t ld, const float* cos_tab, const float* sin_tab,
+                 int batch, int seq, int n_rot_heads, int head_dim, int inverse);
 int jpp_colsum_accum_f32(void* stream, const float* x, int64_t ld, int64_t rows, int64_t cols,
                          float* acc);
 int jpp_mse_loss_f32(void* stream, const float* out, const float* target, int64_t count,
@@ -356,8 +358,8 @@ typedef struct {
                             still be running when jpp_stage_run_task returns control of the
                             caller's stream - see jpp_stage_join */
   int dtype;             /* jpp_dtype of parameters, activations and boundary tensors.
-                            JPP_DTYPE_F32: BERT and decoder-block families, through the *_f32
-                            operators; gradient accumulators are f32 either way */
+                            JPP_DTYPE_F32: the dense families (not the expert layer), through
+                            the *_f32 operators; gradient accumulators are f32 either way */
 } jpp_stage_desc;
 
 enum jpp_dtype { JPP_DTYPE_BF16 = 0, JPP_DTYPE_F32 = 1 };

@@ -36,6 +36,13 @@ __device__ __forceinline__ float gelu_grad32(float u, int tanh_form) {
          u * expf(-0.5f * u * u) * 0.3989422804014327f;
 }
 
+__device__ __forceinline__ float swiglu32(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+__device__ __forceinline__ void swiglu_grad32(float g, float u, float d, float& dg, float& du) {
+  const float sg = 1.0f / (1.0f + expf(-g));
+  dg = d * u * sg * (1.0f + g * (1.0f - sg));
+  du = d * g * sg;
+}
+
 // ---------------------------------------------------------------------------
 // C[m,n] = epilogue(sum_k Aop[m,k] Bop[n,k]); operand orientations as jpp_gemm_bf16
 // ---------------------------------------------------------------------------
@@ -104,6 +111,26 @@ __global__ __launch_bounds__(256) void sgemm_kernel(SgemmParams p) {
       float v = acc[i][j];
       if (p.epi == JPP_EPI_ACC_F32) {
         p.c[row * p.ldc + col] += v;
+        continue;
+      }
+      if (p.epi == JPP_EPI_SWIGLU) {
+        // a 64-column tile is one block of the interleaved layout: gate features in its first
+        // 32 columns (threads tx < 8), the matching up features 32 columns on (thread tx + 8,
+        // lane + 8 of the same wave)
+        p.c[row * p.ldc + col] = v;
+        const float other = __shfl_xor(v, 8);
+        if (tx < 8) p.c2[row * p.ldc2 + n0 / 2 + tx * 4 + j] = swiglu32(v, other);
+        continue;
+      }
+      if (p.epi == JPP_EPI_DSWIGLU) {
+        // v = d s of feature `col`; gate / up of that feature sit at 64 q + w and 64 q + 32 + w
+        const long q = col >> 5, w = col & 31;
+        const float* arow = p.aux + row * p.ldaux + 64 * q + w;
+        float dg, du;
+        swiglu_grad32(arow[0], arow[32], v, dg, du);
+        float* crow = p.c + row * p.ldc + 64 * q + w;
+        crow[0] = dg;
+        crow[32] = du;
         continue;
       }
       if (p.bias) v += p.bias[col];
@@ -234,6 +261,28 @@ __global__ __launch_bounds__(256) void mse32_kernel(const float* __restrict__ ou
     __syncthreads();
   }
   if (threadIdx.x == 0) loss[0] = scale * red[0] / (float)count;
+}
+
+// half-split rotary embedding in place on the first `heads` heads of each row
+__global__ __launch_bounds__(256) void rope32_kernel(float* __restrict__ x, long ld,
+                                                     const float* __restrict__ cos_tab,
+                                                     const float* __restrict__ sin_tab, long rows,
+                                                     int seq, int heads, int d, int inverse) {
+  const int half = d / 2;
+  const long total = rows * heads * half;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const int j = (int)(i % half);
+    const long th = i / half;
+    const int hh = (int)(th % heads);
+    const long t = th / heads;
+    const int pos = (int)(t % seq);
+    float* p = x + t * ld + hh * d + j;
+    const float cs = cos_tab[(long)pos * half + j];
+    const float sn = inverse ? -sin_tab[(long)pos * half + j] : sin_tab[(long)pos * half + j];
+    const float a = p[0], b = p[half];
+    p[0] = a * cs - b * sn;
+    p[half] = b * cs + a * sn;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -448,14 +497,18 @@ int jpp_gemm_f32(void* stream, const jpp_gemm_args* a) {
               (long)a->n, (long)a->k);
   JPP_REQUIRE(a->group_mode == JPP_GROUP_NONE, "gemm_f32: grouped problems are bf16 only");
   const int e = a->epilogue;
-  JPP_REQUIRE(e == JPP_EPI_BF16 || e == JPP_EPI_F32 || e == JPP_EPI_GELU || e == JPP_EPI_DGELU ||
-                  e == JPP_EPI_ACC_F32,
-              "gemm_f32: unsupported epilogue %d", e);
+  JPP_REQUIRE(e >= JPP_EPI_BF16 && e <= JPP_EPI_DSWIGLU, "gemm_f32: unsupported epilogue %d", e);
   JPP_REQUIRE(a->lda >= (a->trans_a ? a->m : a->k) && a->ldb >= (a->trans_b ? a->n : a->k) &&
                   a->ldc >= a->n,
               "gemm_f32: leading dimension too small");
   if (e == JPP_EPI_GELU) JPP_REQUIRE(a->c2 && a->ldc2 >= a->n, "gemm_f32: GELU epilogue needs c2");
   if (e == JPP_EPI_DGELU) JPP_REQUIRE(a->aux && a->ldaux >= a->n, "gemm_f32: dGELU epilogue needs aux");
+  if (e == JPP_EPI_SWIGLU)
+    JPP_REQUIRE(a->c2 && a->ldc2 >= a->n / 2 && !a->bias && !a->resid,
+                "gemm_f32: SwiGLU epilogue needs c2 [M, N/2] and takes no bias / residual");
+  if (e == JPP_EPI_DSWIGLU)
+    JPP_REQUIRE(a->aux && a->ldaux >= 2 * a->n && a->ldc >= 2 * a->n && !a->bias && !a->resid,
+                "gemm_f32: dSwiGLU epilogue needs aux and C of width 2N and takes no bias / residual");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n, "gemm_f32: bad ldresid");
   SgemmParams p;
   p.a = (const float*)a->a; p.b = (const float*)a->b; p.c = (float*)a->c; p.c2 = (float*)a->c2;
@@ -466,6 +519,20 @@ int jpp_gemm_f32(void* stream, const jpp_gemm_args* a) {
   p.ta = a->trans_a != 0; p.tb = a->trans_b != 0; p.epi = e; p.gelu_tanh = a->gelu_tanh;
   hipLaunchKernelGGL(sgemm_kernel, dim3((unsigned)(a->n / 64), (unsigned)(a->m / 64)), dim3(256), 0,
                      (hipStream_t)stream, p);
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+int jpp_rope_f32(void* stream, float* x, int64_t ld, const float* cos_tab, const float* sin_tab,
+                 int batch, int seq, int n_rot_heads, int head_dim, int inverse) {
+  JPP_REQUIRE(x && cos_tab && sin_tab, "rope_f32: null operand");
+  JPP_REQUIRE(batch > 0 && seq > 0 && n_rot_heads > 0 && head_dim > 0 && head_dim % 2 == 0 &&
+                  ld >= (int64_t)n_rot_heads * head_dim,
+              "rope_f32: bad shape");
+  const long rows = (long)batch * seq, total = rows * n_rot_heads * (head_dim / 2);
+  const unsigned grid = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+  hipLaunchKernelGGL(rope32_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, x, (long)ld,
+                     cos_tab, sin_tab, rows, seq, n_rot_heads, head_dim, inverse);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }

@@ -170,6 +170,14 @@ int gemm(jpp_stage* s, hipStream_t st, const void* a, int64_t lda, int ta, const
   return s->f32() ? jpp_gemm_f32(st, &g) : jpp_gemm_bf16(st, &g);
 }
 
+int rope(jpp_stage* s, hipStream_t st, void* x, int inverse) {
+  const int heads = s->d.n_heads + s->d.n_kv_heads;
+  float* c = s->S<float>(s->s_cos);
+  float* sn = s->S<float>(s->s_sin);
+  return s->f32() ? jpp_rope_f32(st, (float*)x, s->qkvw, c, sn, s->d.batch, s->d.seq, heads,
+                                 (int)s->hd, inverse)
+                  : jpp_rope(st, x, s->qkvw, c, sn, s->d.batch, s->d.seq, heads, (int)s->hd, inverse);
+}
 int attn_f(jpp_stage* s, hipStream_t st, const jpp_attn_args* a) {
   return s->f32() ? jpp_attn_fwd_f32(st, a) : jpp_attn_fwd(st, a);
 }
@@ -301,8 +309,7 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
             (float*)at(L.rstd1)));
   RC(gemm(s, st, at(L.n1), h, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 1, at(L.qkv), s->qkvw, T, s->qkvw,
           h, JPP_EPI_BF16));
-  RC(jpp_rope(st, at(L.qkv), s->qkvw, s->S<float>(s->s_cos), s->S<float>(s->s_sin), s->d.batch,
-              s->d.seq, s->d.n_heads + s->d.n_kv_heads, (int)s->hd, 0));
+  RC(rope(s, st, at(L.qkv), 0));
   attn_args(s, aa, slot, L);
   RC(attn_f(s, st, &aa));
   RC(gemm(s, st, at(L.ctx), s->ctxw, 0, s->P(chunk, li, L_Wo), h, 1, at(L.h1), h, T, h, s->ctxw,
@@ -427,16 +434,15 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
   RC(gemm(s, st, wt(W.dh1), h, 0, s->P(chunk, li, L_Wo), h, 0, dctx, s->ctxw, T, s->ctxw, h,
           JPP_EPI_BF16));
   attn_args(s, aa, slot, L);
-  bf16_t* dqkv = (bf16_t*)wt(W.dqkv);
+  uint8_t* dqkv = (uint8_t*)wt(W.dqkv);
   aa.d_o = dctx; aa.lddo = s->ctxw;
   aa.dq = dqkv;
-  aa.dk = dqkv + (int64_t)s->d.n_heads * s->hd;
-  aa.dv = dqkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd;
+  aa.dk = dqkv + (int64_t)s->d.n_heads * s->hd * s->es;
+  aa.dv = dqkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd * s->es;
   aa.lddq = aa.lddk = aa.lddv = s->qkvw;
   aa.delta = s->S<float>(s->s_delta);
   RC(attn_b(s, st, &aa));
-  RC(jpp_rope(st, dqkv, s->qkvw, s->S<float>(s->s_cos), s->S<float>(s->s_sin), s->d.batch,
-              s->d.seq, s->d.n_heads + s->d.n_kv_heads, (int)s->hd, 1));
+  RC(rope(s, st, dqkv, 1));
   RC(gemm(s, st, dqkv, s->qkvw, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 0, dn, h, T, h, s->qkvw,
           JPP_EPI_BF16));
   RC(norm_b(s, st, dn, at(L.x), nullptr, (float*)at(L.rstd1), s->P(chunk, li, L_rms1), wt(W.dh1),
@@ -598,10 +604,9 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   JPP_REQUIRE(d->dtype == JPP_DTYPE_BF16 || d->dtype == JPP_DTYPE_F32, "stage_create: unknown dtype %d",
               d->dtype);
   if (d->dtype == JPP_DTYPE_F32)
-    JPP_REQUIRE((d->family == JPP_FAMILY_BERT || d->family == JPP_FAMILY_DECODER) &&
-                    d->fused_wgrad_accum,
-                "stage_create: f32 stages exist for the BERT and decoder-block families, with "
-                "the accumulation in the weight-gradient GEMM");
+    JPP_REQUIRE(d->family != JPP_FAMILY_MIXTRAL && d->fused_wgrad_accum,
+                "stage_create: f32 stages exist for the dense families, with the accumulation "
+                "in the weight-gradient GEMM");
 
   jpp_stage* s = new jpp_stage();
   s->d = *d;

@@ -104,7 +104,7 @@ EXPORTS = [
     "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_gemm_f32", "jpp_attn_fwd_f32", "jpp_attn_bwd_f32", "jpp_norm_fwd_f32", "jpp_norm_bwd_f32",
-    "jpp_colsum_accum_f32", "jpp_mse_loss_f32",
+    "jpp_colsum_accum_f32", "jpp_mse_loss_f32", "jpp_rope_f32",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_sum_accum_f32", "jpp_colsum_accum", "jpp_colsum_accum_multi", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
@@ -170,6 +170,8 @@ def load():
     lib.jpp_norm_bwd_f32.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
     lib.jpp_colsum_accum_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
                                          C.c_void_p]
+    lib.jpp_rope_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int,
+                                 C.c_int, C.c_int, C.c_int, C.c_int]
     lib.jpp_mse_loss_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float,
                                      C.c_void_p, C.c_void_p]
     lib.jpp_swiglu_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,

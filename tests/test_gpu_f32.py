@@ -83,12 +83,66 @@ def test_gemm_f32_epilogues(lay, m, n, k):
         close(run(rt.EPI_DGELU, aux=daux.ptr, ldaux=n, gelu_tanh=tanh_form), prod * gp, 1e-5, "dgelu")
 
 
+def test_gemm_f32_swiglu_epilogues_and_rope():
+    rng = np.random.default_rng(21)
+    m, f, k = 128, 192, 64                 # gate/up interleaved in blocks of 32 columns
+    A = rng.standard_normal((m, k), dtype=np.float32)
+    W = rng.standard_normal((k, 2 * f), dtype=np.float32) * np.float32(0.2)   # [gate | up]
+    c = np.arange(2 * f)
+    q, w = c // 64, c % 64
+    order = np.where(w < 32, 32 * q + w, f + 32 * q + w - 32)                 # device column -> host column
+    da, dw = dev(A), dev(W[:, order])
+    gu, s_out = rt.DeviceBuffer(m * 2 * f * 4), rt.DeviceBuffer(m * f * 4)
+    rt.gemm(da.ptr, dw.ptr, gu.ptr, m, 2 * f, k, k, 2 * f, 2 * f, 0, 1, rt.EPI_SWIGLU, c2=s_out.ptr,
+            ldc2=f, f32=True)
+    rt.sync()
+    prod = A.astype(np.float64) @ W.astype(np.float64)
+    g64, u64 = prod[:, :f], prod[:, f:]
+    close(gu.download(np.float32, (m, 2 * f)), prod[:, order], 1e-5, "gate/up")
+    close(s_out.download(np.float32, (m, f)), g64 / (1 + np.exp(-g64)) * u64, 1e-5, "swiglu")
+    # gradient: d(gate/up) from ds = dy Wd^T, C of width 2f in the interleaved layout
+    h = 64
+    dy = rng.standard_normal((m, h), dtype=np.float32)
+    Wd = rng.standard_normal((f, h), dtype=np.float32) * np.float32(0.2)
+    ddy, dwd, dgu = dev(dy), dev(Wd), rt.DeviceBuffer(m * 2 * f * 4)
+    rt.gemm(ddy.ptr, dwd.ptr, dgu.ptr, m, f, h, h, h, 2 * f, 0, 0, rt.EPI_DSWIGLU, aux=gu.ptr,
+            ldaux=2 * f, f32=True)
+    rt.sync()
+    ds = dy.astype(np.float64) @ Wd.astype(np.float64).T
+    sg = 1 / (1 + np.exp(-g64))
+    want = np.concatenate([ds * u64 * sg * (1 + g64 * (1 - sg)), ds * g64 * sg], 1)
+    close(dgu.download(np.float32, (m, 2 * f)), want[:, order], 1e-5, "d gate/up")
+    # rotary embedding and its inverse
+    B, S, heads, d = 2, 64, 3, 128
+    ld = (heads + 1) * d
+    x = rng.standard_normal((B * S, ld), dtype=np.float32)
+    ang = np.arange(S)[:, None] * (5e5 ** (-2.0 * np.arange(d // 2) / d))[None, :]
+    cs, sn = np.cos(ang), np.sin(ang)
+    bx, bc, bs = dev(x), dev(cs), dev(sn)
+    lib = rt.load()
+    rt.check(lib.jpp_rope_f32(None, bx.ptr, ld, bc.ptr, bs.ptr, B, S, heads, d, 0))
+    rt.sync()
+    want = x.astype(np.float64).copy()
+    xr = want[:, :heads * d].reshape(B, S, heads, d)
+    a, b = xr[..., :d // 2].copy(), xr[..., d // 2:].copy()
+    xr[..., :d // 2] = a * cs[None, :, None, :] - b * sn[None, :, None, :]
+    xr[..., d // 2:] = b * cs[None, :, None, :] + a * sn[None, :, None, :]
+    want[:, :heads * d] = xr.reshape(B * S, heads * d)
+    close(bx.download(np.float32, (B * S, ld)), want, 1e-5, "rope (last head untouched)")
+    rt.check(lib.jpp_rope_f32(None, bx.ptr, ld, bc.ptr, bs.ptr, B, S, heads, d, 1))
+    rt.sync()
+    close(bx.download(np.float32, (B * S, ld)), x.astype(np.float64), 1e-5, "rope then inverse")
+
+
 def test_gemm_f32_rejects_what_it_does_not_do():
     d = rt.DeviceBuffer(64 * 64 * 4)
     with pytest.raises(rt.JppError, match="multiples of 64"):
         rt.gemm(d.ptr, d.ptr, d.ptr, 32, 64, 16, 16, 64, 64, 0, 1, f32=True)
-    with pytest.raises(rt.JppError, match="unsupported epilogue"):
+    with pytest.raises(rt.JppError, match="SwiGLU epilogue needs c2"):
         rt.gemm(d.ptr, d.ptr, d.ptr, 64, 64, 16, 16, 64, 64, 0, 1, rt.EPI_SWIGLU, f32=True)
+    with pytest.raises(rt.JppError, match="grouped problems are bf16 only"):
+        rt.gemm(d.ptr, d.ptr, d.ptr, 64, 64, 16, 16, 64, 64, 0, 1, f32=True, seg=d.ptr, n_seg=1,
+                group_mode=1)
 
 
 @pytest.mark.parametrize("ln", [True, False], ids=["layernorm", "rmsnorm"])
@@ -205,7 +259,15 @@ DECODER_F32 = LayerSpec("decoder", 256, 2, 512, 128, 2, causal=True, eps=1e-6, g
                         dtype="f32")
 BERT_D64_F32 = LayerSpec("bert", 128, 2, 256, 256, 1, eps=1e-5, dtype="f32")
 
+LLAMA_F32 = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
+                      rope_theta=5e5, eps=1e-5, dtype="f32")
+LLAMA_D64_F32 = LayerSpec("llama", 256, 4, 256, 256, 1, n_kv_heads=2, head_dim=64, causal=True,
+                          rope_theta=1e4, eps=1e-5, dtype="f32")
+
 STAGES_F32 = [
+    ("llama-interleaved", LLAMA_F32, S.Interleaved1F1B(4, 2), 4, 0, 2),
+    ("llama-zb", LLAMA_D64_F32, S.ZeroBubble(3), 3, 1, 2),
+    ("llama-dualpipev", LLAMA_F32, S.DualPipeV(4, 2), 4, 1, 1),
     ("cfg1-rank0", CFG1, S.Std1F1B(2), 8, 0, 2),
     ("cfg1-rank1", CFG1, S.Std1F1B(2), 8, 1, 2),
     ("bert-zb", BERT_D64_F32, S.ZeroBubble(2), 3, 1, 2),
@@ -239,9 +301,9 @@ def test_f32_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
 
 
 def test_f32_stage_needs_a_family_with_f32_operators():
-    spec = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
-                     dtype="f32")
-    with pytest.raises(rt.JppError, match="f32 stages exist for"):
+    spec = LayerSpec("mixtral", 256, 2, 256, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
+                     n_experts=8, top_k=2, dtype="f32")
+    with pytest.raises(rt.JppError, match="f32 stages exist for the dense families"):
         rt.StageExecutor(spec, 1, 1, 1)
 
 
