@@ -165,7 +165,7 @@ def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
 
 @pytest.mark.parametrize("ln,rows,cols", [(True, 300, 256), (True, 1024, 1024), (False, 512, 4096),
                                           (False, 130, 8192), (False, 64, 128), (True, 261, 4096),
-                                          (True, 1030, 8192)])
+                                          (True, 1030, 8192), (True, 140, 6144), (False, 140, 5120)])
 def test_norm_fwd_bwd(ln, rows, cols):
     print(f"norm ln={ln} {rows}x{cols}", flush=True)
     rng = np.random.default_rng(rows + cols)
