@@ -250,7 +250,7 @@ int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t coun
 /* ---- the same operators on f32 tensors -----------------------------------------
  * The full-precision flavour of a stage (jpp_stage_desc.dtype = JPP_DTYPE_F32): the
  * reference's CPU-runnable configuration is float32 end to end (BERT-style stack of
- * hidden 256; tests/test_transformations.py:44-118 also builds its model in float32).
+ * hidden 256; tests/test_transformations.py:42-93 also builds its model in float32).
  * Same argument structs, every bf16 tensor replaced by an f32 one; plain fp32 arithmetic
  * in a fixed summation order, sized for small problems (not for the matrix cores).
  * jpp_gemm_f32: M, N multiples of 64, K of 16; every epilogue of jpp_gemm_bf16

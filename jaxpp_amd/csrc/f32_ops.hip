@@ -1,6 +1,6 @@
 // The layer's operators on fp32 tensors: the full-precision flavour of a stage, as the
 // reference's own CPU-runnable configuration uses it (BERT-style stack of hidden 256 in
-// float32, tests/test_transformations.py:44-118 builds its model in float32 too).  Same
+// float32, tests/test_transformations.py:42-93 builds its model in float32 too).  Same
 // argument structs as the bf16 entry points with every bf16 tensor replaced by an f32 one.
 //
 // These kernels serve small problems whose results must hold 1e-4 against an fp32 CPU run;
