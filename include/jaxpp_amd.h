@@ -254,7 +254,8 @@ int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t coun
  * Same argument structs, every bf16 tensor replaced by an f32 one; plain fp32 arithmetic
  * in a fixed summation order, sized for small problems (not for the matrix cores).
  * jpp_gemm_f32: M, N multiples of 64, K of 16; every epilogue of jpp_gemm_bf16
- * (JPP_EPI_BF16 = store in the element type, with bias and residual); no groups.
+ * (JPP_EPI_BF16 = store in the element type, with bias and residual) and both grouped modes
+ * (group offsets multiples of 64; a grouped contraction runs over the padded extent).
  * jpp_attn_*_f32: seq a multiple of 64.  jpp_norm_bwd_f32 does not use `partial`. */
 int jpp_gemm_f32(void* stream, const jpp_gemm_args* args);
 int jpp_attn_fwd_f32(void* stream, const jpp_attn_args* args);
@@ -298,6 +299,8 @@ int jpp_adam_step(void* stream, const jpp_adam_args* args);
  * Tokens are assigned to rows of "permuted" buffers, grouped by expert in token
  * order, each group padded to a multiple of 256 rows (padding rows are zero);
  * jpp_moe_capacity() rows always suffice.  seg[e] is the first row of expert e. */
+enum jpp_dtype { JPP_DTYPE_BF16 = 0, JPP_DTYPE_F32 = 1 };
+
 typedef struct {
   const void* x;     /* bf16 [tokens, hidden]: router input (jpp_moe_route only) */
   const void* wr;    /* bf16 [hidden, n_experts] */
@@ -311,6 +314,8 @@ typedef struct {
   void* work;        /* int32 [2 * ceil(tokens / 256) * n_experts] scratch */
   int64_t tokens, hidden;
   int n_experts, top_k; /* 8, 2 */
+  int dtype;            /* jpp_dtype of x, wr and of every activation tensor passed beside the
+                           struct (bf16 in the comments here and below: f32 when JPP_DTYPE_F32) */
 } jpp_moe_args;
 
 int64_t jpp_moe_capacity(int64_t tokens, int n_experts, int top_k);
@@ -358,11 +363,10 @@ typedef struct {
                             still be running when jpp_stage_run_task returns control of the
                             caller's stream - see jpp_stage_join */
   int dtype;             /* jpp_dtype of parameters, activations and boundary tensors.
-                            JPP_DTYPE_F32: the dense families (not the expert layer), through
-                            the *_f32 operators; gradient accumulators are f32 either way */
+                            JPP_DTYPE_F32: every family, through the *_f32 operators and the
+                            routing kernels' f32 form; gradient accumulators are f32 either way */
 } jpp_stage_desc;
 
-enum jpp_dtype { JPP_DTYPE_BF16 = 0, JPP_DTYPE_F32 = 1 };
 
 int jpp_stage_create(const jpp_stage_desc* desc, jpp_stage** out);
 int jpp_stage_destroy(jpp_stage* stage);

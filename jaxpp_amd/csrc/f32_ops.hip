@@ -57,6 +57,10 @@ struct SgemmParams {
   int m, n, k;
   long lda, ldb, ldc, ldc2, ldresid, ldaux;
   int ta, tb, epi, gelu_tanh;
+  // grouped problems, as for the bf16 GEMM: seg[0..n_seg] are row offsets (multiples of 64)
+  const int* seg;
+  int n_seg, group_mode;
+  long stride_b, stride_c;
 };
 
 // 64x64 output tile, 16x16 threads of 4x4 outputs each, K in steps of 16 through LDS
@@ -64,6 +68,21 @@ __global__ __launch_bounds__(256) void sgemm_kernel(SgemmParams p) {
   __shared__ float As[16][68], Bs[16][68];
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
   const long m0 = (long)blockIdx.y * 64, n0 = (long)blockIdx.x * 64;
+  if (p.group_mode == JPP_GROUP_M) {
+    // rows of A and C are grouped by expert; each group multiplies its own B
+    if (m0 >= p.seg[p.n_seg]) return;
+    int e = 0;
+    while (p.seg[e + 1] <= m0) ++e;
+    p.b += (long)e * p.stride_b;
+  } else if (p.group_mode == JPP_GROUP_K) {
+    // one output per expert (blockIdx.z); the contraction runs over the expert's rows
+    const int e = blockIdx.z;
+    const long r0 = p.seg[e];
+    p.k = p.seg[e + 1] - p.seg[e];
+    p.a += r0 * p.lda;
+    p.b += r0 * p.ldb;
+    p.c += (long)e * p.stride_c;
+  }
   float acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -492,14 +511,23 @@ extern "C" {
 
 int jpp_gemm_f32(void* stream, const jpp_gemm_args* a) {
   JPP_REQUIRE(a && a->a && a->b && a->c, "gemm_f32: null operand");
-  JPP_REQUIRE(a->m > 0 && a->n > 0 && a->k > 0 && a->m % 64 == 0 && a->n % 64 == 0 && a->k % 16 == 0,
+  const bool group_k = a->group_mode == JPP_GROUP_K;
+  JPP_REQUIRE(a->m > 0 && a->n > 0 && (a->k > 0 || group_k) && a->m % 64 == 0 && a->n % 64 == 0 &&
+                  (a->k % 16 == 0 || group_k),
               "gemm_f32: M, N must be multiples of 64 and K of 16, got %ldx%ldx%ld", (long)a->m,
               (long)a->n, (long)a->k);
-  JPP_REQUIRE(a->group_mode == JPP_GROUP_NONE, "gemm_f32: grouped problems are bf16 only");
+  if (a->group_mode != JPP_GROUP_NONE) {
+    JPP_REQUIRE(a->group_mode == JPP_GROUP_M || group_k, "gemm_f32: unknown group_mode %d",
+                a->group_mode);
+    JPP_REQUIRE(a->seg && a->n_seg > 0 && a->n_seg <= 256, "gemm_f32: grouped problem needs seg[n_seg+1]");
+    JPP_REQUIRE(!a->bias && !a->resid, "gemm_f32: grouped problems take no bias / residual");
+    JPP_REQUIRE(!group_k || (a->trans_a && a->trans_b),
+                "gemm_f32: a grouped contraction takes both operands with the rows as the slow index");
+  }
   const int e = a->epilogue;
   JPP_REQUIRE(e >= JPP_EPI_BF16 && e <= JPP_EPI_DSWIGLU, "gemm_f32: unsupported epilogue %d", e);
-  JPP_REQUIRE(a->lda >= (a->trans_a ? a->m : a->k) && a->ldb >= (a->trans_b ? a->n : a->k) &&
-                  a->ldc >= a->n,
+  JPP_REQUIRE(a->lda >= (a->trans_a ? a->m : (group_k ? 0 : a->k)) &&
+                  a->ldb >= (a->trans_b ? a->n : (group_k ? 0 : a->k)) && a->ldc >= a->n,
               "gemm_f32: leading dimension too small");
   if (e == JPP_EPI_GELU) JPP_REQUIRE(a->c2 && a->ldc2 >= a->n, "gemm_f32: GELU epilogue needs c2");
   if (e == JPP_EPI_DGELU) JPP_REQUIRE(a->aux && a->ldaux >= a->n, "gemm_f32: dGELU epilogue needs aux");
@@ -517,8 +545,11 @@ int jpp_gemm_f32(void* stream, const jpp_gemm_args* a) {
   p.lda = a->lda; p.ldb = a->ldb; p.ldc = a->ldc; p.ldc2 = a->ldc2; p.ldresid = a->ldresid;
   p.ldaux = a->ldaux;
   p.ta = a->trans_a != 0; p.tb = a->trans_b != 0; p.epi = e; p.gelu_tanh = a->gelu_tanh;
-  hipLaunchKernelGGL(sgemm_kernel, dim3((unsigned)(a->n / 64), (unsigned)(a->m / 64)), dim3(256), 0,
-                     (hipStream_t)stream, p);
+  p.seg = a->seg; p.n_seg = a->n_seg; p.group_mode = a->group_mode;
+  p.stride_b = a->stride_b; p.stride_c = a->stride_c;
+  hipLaunchKernelGGL(sgemm_kernel,
+                     dim3((unsigned)(a->n / 64), (unsigned)(a->m / 64), group_k ? (unsigned)a->n_seg : 1u),
+                     dim3(256), 0, (hipStream_t)stream, p);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }

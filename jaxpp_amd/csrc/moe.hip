@@ -11,6 +11,28 @@ namespace {
 constexpr int kE = 8;        // experts
 constexpr int kPad = 256;    // expert groups start at multiples of the GEMM tile height
 
+// 8 consecutive elements of a bf16 or an f32 tensor
+__device__ __forceinline__ void load8(const bf16_t* p, float (&f)[8]) {
+  unpack8(*(const uint4*)p, f);
+}
+__device__ __forceinline__ void load8(const float* p, float (&f)[8]) {
+  const float4 a = ((const float4*)p)[0], b = ((const float4*)p)[1];
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w;
+  f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float (&f)[8]) { *(uint4*)p = pack8(f); }
+__device__ __forceinline__ void store8(float* p, const float (&f)[8]) {
+  ((float4*)p)[0] = make_float4(f[0], f[1], f[2], f[3]);
+  ((float4*)p)[1] = make_float4(f[4], f[5], f[6], f[7]);
+}
+__device__ __forceinline__ void copy8(const bf16_t* src, bf16_t* dst) { *(uint4*)dst = *(const uint4*)src; }
+__device__ __forceinline__ void copy8(const float* src, float* dst) {
+  ((float4*)dst)[0] = ((const float4*)src)[0];
+  ((float4*)dst)[1] = ((const float4*)src)[1];
+}
+__device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+__device__ __forceinline__ float to_f32(float v) { return v; }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -19,8 +41,9 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // logits = x Wr (fp32), top-2 by value (ties -> lower index), gates = softmax
 // over the two selected logits.  One wave per token.
-__global__ __launch_bounds__(256) void router_kernel(const bf16_t* __restrict__ x,
-                                                     const bf16_t* __restrict__ wr, long T, int h,
+template <typename El>
+__global__ __launch_bounds__(256) void router_kernel(const El* __restrict__ x,
+                                                     const El* __restrict__ wr, long T, int h,
                                                      int* __restrict__ ids,
                                                      float* __restrict__ gates) {
   const int lane = threadIdx.x & 63;
@@ -31,11 +54,11 @@ __global__ __launch_bounds__(256) void router_kernel(const bf16_t* __restrict__ 
   for (int e = 0; e < kE; ++e) acc[e] = 0.f;
   for (int c = lane; c < h / 8; c += 64) {
     float xv[8];
-    unpack8(*(const uint4*)(x + t * h + c * 8), xv);
+    load8(x + t * h + c * 8, xv);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float w[8];
-      unpack8(*(const uint4*)(wr + (long)(c * 8 + j) * kE), w);
+      load8(wr + (long)(c * 8 + j) * kE, w);
 #pragma unroll
       for (int e = 0; e < kE; ++e) acc[e] += xv[j] * w[e];
     }
@@ -135,45 +158,52 @@ __global__ __launch_bounds__(256) void assign_kernel(const int* __restrict__ ids
 }
 
 // xp[row] = x[tok_of[row]] (zero for padding rows)
-__global__ __launch_bounds__(256) void gather_kernel(const bf16_t* __restrict__ x,
+template <typename El>
+__global__ __launch_bounds__(256) void gather_kernel(const El* __restrict__ x,
                                                      const int* __restrict__ tok_of,
                                                      const int* __restrict__ seg, int h,
-                                                     bf16_t* __restrict__ xp) {
+                                                     El* __restrict__ xp) {
   const int hc = h / 8;
   const long rows = seg[kE];
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < rows * hc; i += (long)gridDim.x * 256) {
     const long row = i / hc;
     const int c = (int)(i - row * hc);
     const int t = tok_of[row];
-    ((uint4*)(xp + row * h))[c] =
-        t >= 0 ? ((const uint4*)(x + (long)t * h))[c] : make_uint4(0, 0, 0, 0);
+    if (t >= 0) {
+      copy8(x + (long)t * h + c * 8, xp + row * h + c * 8);
+    } else {
+      const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      store8(xp + row * h + c * 8, z);
+    }
   }
 }
 
 // y[t] = resid[t] + sum_k gate[t,k] * eo[row_of[t,k]]
-__global__ __launch_bounds__(256) void combine_fwd_kernel(const bf16_t* __restrict__ eo,
+template <typename El>
+__global__ __launch_bounds__(256) void combine_fwd_kernel(const El* __restrict__ eo,
                                                           const int* __restrict__ row_of,
                                                           const float* __restrict__ gates,
-                                                          const bf16_t* __restrict__ resid, long T,
-                                                          int h, bf16_t* __restrict__ y) {
+                                                          const El* __restrict__ resid, long T,
+                                                          int h, El* __restrict__ y) {
   const int hc = h / 8;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < T * hc; i += (long)gridDim.x * 256) {
     const long t = i / hc;
     const int c = (int)(i - t * hc);
     float r[8], a[8], b[8];
-    unpack8(((const uint4*)(resid + t * h))[c], r);
-    unpack8(((const uint4*)(eo + (long)row_of[t * 2] * h))[c], a);
-    unpack8(((const uint4*)(eo + (long)row_of[t * 2 + 1] * h))[c], b);
+    load8(resid + t * h + c * 8, r);
+    load8(eo + (long)row_of[t * 2] * h + c * 8, a);
+    load8(eo + (long)row_of[t * 2 + 1] * h + c * 8, b);
     const float g0 = gates[t * 2], g1 = gates[t * 2 + 1];
 #pragma unroll
     for (int e = 0; e < 8; ++e) r[e] = (r[e] + g0 * a[e]) + g1 * b[e];
-    ((uint4*)(y + t * h))[c] = pack8(r);
+    store8(y + t * h + c * 8, r);
   }
 }
 
 // d(gate) and d(logits): one wave per token
-__global__ __launch_bounds__(256) void gate_bwd_kernel(const bf16_t* __restrict__ dy,
-                                                       const bf16_t* __restrict__ eo,
+template <typename El>
+__global__ __launch_bounds__(256) void gate_bwd_kernel(const El* __restrict__ dy,
+                                                       const El* __restrict__ eo,
                                                        const int* __restrict__ row_of,
                                                        const int* __restrict__ ids,
                                                        const float* __restrict__ gates, long T,
@@ -181,14 +211,14 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const bf16_t* __restrict_
   const int lane = threadIdx.x & 63;
   const long t = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
-  const bf16_t* e0 = eo + (long)row_of[t * 2] * h;
-  const bf16_t* e1 = eo + (long)row_of[t * 2 + 1] * h;
+  const El* e0 = eo + (long)row_of[t * 2] * h;
+  const El* e1 = eo + (long)row_of[t * 2 + 1] * h;
   float d0 = 0.f, d1 = 0.f;
   for (int c = lane; c < h / 8; c += 64) {
     float g[8], a[8], b[8];
-    unpack8(((const uint4*)(dy + t * h))[c], g);
-    unpack8(((const uint4*)e0)[c], a);
-    unpack8(((const uint4*)e1)[c], b);
+    load8(dy + t * h + c * 8, g);
+    load8(e0 + c * 8, a);
+    load8(e1 + c * 8, b);
 #pragma unroll
     for (int e = 0; e < 8; ++e) { d0 += g[e] * a[e]; d1 += g[e] * b[e]; }
   }
@@ -205,11 +235,12 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const bf16_t* __restrict_
 }
 
 // deo[row] = gate_of[row] * dy[tok_of[row]] (zero for padding rows)
-__global__ __launch_bounds__(256) void scatter_dy_kernel(const bf16_t* __restrict__ dy,
+template <typename El>
+__global__ __launch_bounds__(256) void scatter_dy_kernel(const El* __restrict__ dy,
                                                          const int* __restrict__ tok_of,
                                                          const float* __restrict__ gate_of,
                                                          const int* __restrict__ seg, int h,
-                                                         bf16_t* __restrict__ deo) {
+                                                         El* __restrict__ deo) {
   const int hc = h / 8;
   const long rows = seg[kE];
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < rows * hc; i += (long)gridDim.x * 256) {
@@ -218,46 +249,48 @@ __global__ __launch_bounds__(256) void scatter_dy_kernel(const bf16_t* __restric
     const int t = tok_of[row];
     float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (t >= 0) {
-      unpack8(((const uint4*)(dy + (long)t * h))[c], f);
+      load8(dy + (long)t * h + c * 8, f);
       const float g = gate_of[row];
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] *= g;
     }
-    ((uint4*)(deo + row * h))[c] = pack8(f);
+    store8(deo + row * h + c * 8, f);
   }
 }
 
 // dx[t] = dxp[row_of[t,0]] + dxp[row_of[t,1]] + dlogits[t] Wr^T
-__global__ __launch_bounds__(256) void combine_bwd_kernel(const bf16_t* __restrict__ dxp,
+template <typename El>
+__global__ __launch_bounds__(256) void combine_bwd_kernel(const El* __restrict__ dxp,
                                                           const int* __restrict__ row_of,
                                                           const float* __restrict__ dlogits,
-                                                          const bf16_t* __restrict__ wr, long T,
-                                                          int h, bf16_t* __restrict__ dx) {
+                                                          const El* __restrict__ wr, long T,
+                                                          int h, El* __restrict__ dx) {
   const int hc = h / 8;
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < T * hc; i += (long)gridDim.x * 256) {
     const long t = i / hc;
     const int c = (int)(i - t * hc);
     float a[8], b[8], dl[kE];
-    unpack8(((const uint4*)(dxp + (long)row_of[t * 2] * h))[c], a);
-    unpack8(((const uint4*)(dxp + (long)row_of[t * 2 + 1] * h))[c], b);
+    load8(dxp + (long)row_of[t * 2] * h + c * 8, a);
+    load8(dxp + (long)row_of[t * 2 + 1] * h + c * 8, b);
 #pragma unroll
     for (int e = 0; e < kE; ++e) dl[e] = dlogits[t * kE + e];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float w[8];
-      unpack8(*(const uint4*)(wr + (long)(c * 8 + j) * kE), w);
+      load8(wr + (long)(c * 8 + j) * kE, w);
       float r = 0.f;
 #pragma unroll
       for (int e = 0; e < kE; ++e) r += dl[e] * w[e];
       a[j] = (a[j] + b[j]) + r;
     }
-    ((uint4*)(dx + t * h))[c] = pack8(a);
+    store8(dx + t * h + c * 8, a);
   }
 }
 
 // dWr[j, e] += sum_t x[t, j] * dlogits[t, e]: block (row panel b, column panel)
 // writes partial[b][j][e]; wr_reduce sums the panels in order
-__global__ __launch_bounds__(256) void wr_partial_kernel(const bf16_t* __restrict__ x,
+template <typename El>
+__global__ __launch_bounds__(256) void wr_partial_kernel(const El* __restrict__ x,
                                                          const float* __restrict__ dlogits, long T,
                                                          int h, float* __restrict__ partial) {
   const int j = blockIdx.y * 256 + threadIdx.x;
@@ -266,7 +299,7 @@ __global__ __launch_bounds__(256) void wr_partial_kernel(const bf16_t* __restric
 #pragma unroll
   for (int e = 0; e < kE; ++e) acc[e] = 0.f;
   for (long t = blockIdx.x; t < T; t += gridDim.x) {
-    const float xv = bf16_to_f32(x[t * h + j]);
+    const float xv = to_f32(x[t * h + j]);
 #pragma unroll
     for (int e = 0; e < kE; ++e) acc[e] += xv * dlogits[t * kE + e];
   }
@@ -307,14 +340,21 @@ int jpp_moe_route(void* stream, const jpp_moe_args* a) {
               "moe_route: null operand");
   JPP_REQUIRE(a->n_experts == kE && a->top_k == 2, "moe_route: built for 8 experts, top-2");
   JPP_REQUIRE(a->tokens > 0 && a->hidden % 8 == 0, "moe_route: bad shape");
+  JPP_REQUIRE(a->dtype == JPP_DTYPE_BF16 || a->dtype == JPP_DTYPE_F32, "moe_route: unknown dtype %d",
+              a->dtype);
   hipStream_t st = (hipStream_t)stream;
   const long T = a->tokens;
   const int nblk = (int)((T + 255) / 256);
   int* cnt = (int*)a->work;
   int* base = cnt + (long)nblk * kE;
   const long cap = jpp_moe_capacity(T, kE, 2);
-  hipLaunchKernelGGL(router_kernel, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st,
-                     (const bf16_t*)a->x, (const bf16_t*)a->wr, T, (int)a->hidden, a->ids, a->gates);
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(router_kernel<float>, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st,
+                       (const float*)a->x, (const float*)a->wr, T, (int)a->hidden, a->ids, a->gates);
+  } else {
+    hipLaunchKernelGGL(router_kernel<bf16_t>, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st,
+                       (const bf16_t*)a->x, (const bf16_t*)a->wr, T, (int)a->hidden, a->ids, a->gates);
+  }
   hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(cap)), dim3(256), 0, st, a->tok_of, -1, cap);
   hipLaunchKernelGGL(count_kernel, dim3(nblk), dim3(256), 0, st, a->ids, T, cnt);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, st, cnt, nblk, a->seg, base);
@@ -327,9 +367,15 @@ int jpp_moe_route(void* stream, const jpp_moe_args* a) {
 int jpp_moe_gather(void* stream, const jpp_moe_args* a, const void* x, void* xp) {
   JPP_REQUIRE(a && x && xp, "moe_gather: null operand");
   const long cap = jpp_moe_capacity(a->tokens, kE, 2);
-  hipLaunchKernelGGL(gather_kernel, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0,
-                     (hipStream_t)stream, (const bf16_t*)x, a->tok_of, a->seg, (int)a->hidden,
-                     (bf16_t*)xp);
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(gather_kernel<float>, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)x, a->tok_of, a->seg, (int)a->hidden,
+                       (float*)xp);
+  } else {
+    hipLaunchKernelGGL(gather_kernel<bf16_t>, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)x, a->tok_of, a->seg, (int)a->hidden,
+                       (bf16_t*)xp);
+  }
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -337,9 +383,15 @@ int jpp_moe_gather(void* stream, const jpp_moe_args* a, const void* x, void* xp)
 int jpp_moe_combine_fwd(void* stream, const jpp_moe_args* a, const void* eo, const void* resid,
                         void* y) {
   JPP_REQUIRE(a && eo && resid && y, "moe_combine_fwd: null operand");
-  hipLaunchKernelGGL(combine_fwd_kernel, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
-                     (hipStream_t)stream, (const bf16_t*)eo, a->row_of, a->gates,
-                     (const bf16_t*)resid, (long)a->tokens, (int)a->hidden, (bf16_t*)y);
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(combine_fwd_kernel<float>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)eo, a->row_of, a->gates,
+                       (const float*)resid, (long)a->tokens, (int)a->hidden, (float*)y);
+  } else {
+    hipLaunchKernelGGL(combine_fwd_kernel<bf16_t>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)eo, a->row_of, a->gates,
+                       (const bf16_t*)resid, (long)a->tokens, (int)a->hidden, (bf16_t*)y);
+  }
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -349,12 +401,24 @@ int jpp_moe_bwd_prepare(void* stream, const jpp_moe_args* a, const void* dy, con
   JPP_REQUIRE(a && dy && eo && dlogits && deo, "moe_bwd_prepare: null operand");
   hipStream_t st = (hipStream_t)stream;
   const long cap = jpp_moe_capacity(a->tokens, kE, 2);
-  hipLaunchKernelGGL(gate_bwd_kernel, dim3((unsigned)((a->tokens + 3) / 4)), dim3(256), 0, st,
-                     (const bf16_t*)dy, (const bf16_t*)eo, a->row_of, a->ids, a->gates,
-                     (long)a->tokens, (int)a->hidden, dlogits);
-  hipLaunchKernelGGL(scatter_dy_kernel, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0, st,
-                     (const bf16_t*)dy, a->tok_of, a->gate_of, a->seg, (int)a->hidden,
-                     (bf16_t*)deo);
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(gate_bwd_kernel<float>, dim3((unsigned)((a->tokens + 3) / 4)), dim3(256), 0, st,
+                       (const float*)dy, (const float*)eo, a->row_of, a->ids, a->gates,
+                       (long)a->tokens, (int)a->hidden, dlogits);
+  } else {
+    hipLaunchKernelGGL(gate_bwd_kernel<bf16_t>, dim3((unsigned)((a->tokens + 3) / 4)), dim3(256), 0, st,
+                       (const bf16_t*)dy, (const bf16_t*)eo, a->row_of, a->ids, a->gates,
+                       (long)a->tokens, (int)a->hidden, dlogits);
+  }
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(scatter_dy_kernel<float>, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0, st,
+                       (const float*)dy, a->tok_of, a->gate_of, a->seg, (int)a->hidden,
+                       (float*)deo);
+  } else {
+    hipLaunchKernelGGL(scatter_dy_kernel<bf16_t>, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0, st,
+                       (const bf16_t*)dy, a->tok_of, a->gate_of, a->seg, (int)a->hidden,
+                       (bf16_t*)deo);
+  }
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -362,9 +426,15 @@ int jpp_moe_bwd_prepare(void* stream, const jpp_moe_args* a, const void* dy, con
 int jpp_moe_combine_bwd(void* stream, const jpp_moe_args* a, const void* dxp,
                         const float* dlogits, void* dx) {
   JPP_REQUIRE(a && dxp && dlogits && dx, "moe_combine_bwd: null operand");
-  hipLaunchKernelGGL(combine_bwd_kernel, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
-                     (hipStream_t)stream, (const bf16_t*)dxp, a->row_of, dlogits,
-                     (const bf16_t*)a->wr, (long)a->tokens, (int)a->hidden, (bf16_t*)dx);
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(combine_bwd_kernel<float>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)dxp, a->row_of, dlogits,
+                       (const float*)a->wr, (long)a->tokens, (int)a->hidden, (float*)dx);
+  } else {
+    hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
+                       (hipStream_t)stream, (const bf16_t*)dxp, a->row_of, dlogits,
+                       (const bf16_t*)a->wr, (long)a->tokens, (int)a->hidden, (bf16_t*)dx);
+  }
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -374,8 +444,13 @@ int jpp_moe_router_wgrad(void* stream, const jpp_moe_args* a, const void* x, con
   JPP_REQUIRE(a && x && dlogits && acc && partial, "moe_router_wgrad: null operand");
   hipStream_t st = (hipStream_t)stream;
   const int nb = 64;
-  hipLaunchKernelGGL(wr_partial_kernel, dim3(nb, (unsigned)((a->hidden + 255) / 256)), dim3(256), 0,
-                     st, (const bf16_t*)x, dlogits, (long)a->tokens, (int)a->hidden, partial);
+  if (a->dtype == JPP_DTYPE_F32) {
+    hipLaunchKernelGGL(wr_partial_kernel<float>, dim3(nb, (unsigned)((a->hidden + 255) / 256)), dim3(256), 0,
+                       st, (const float*)x, dlogits, (long)a->tokens, (int)a->hidden, partial);
+  } else {
+    hipLaunchKernelGGL(wr_partial_kernel<bf16_t>, dim3(nb, (unsigned)((a->hidden + 255) / 256)), dim3(256), 0,
+                       st, (const bf16_t*)x, dlogits, (long)a->tokens, (int)a->hidden, partial);
+  }
   const long n = (long)a->hidden * kE;
   hipLaunchKernelGGL(wr_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, partial,
                      nb, n, acc);

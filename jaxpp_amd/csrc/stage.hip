@@ -127,7 +127,7 @@ enum MixtralP { X_rms1, X_Wqkv, X_Wo, X_rms2, X_Wr, X_Wgu, X_Wd };
     if (rc_) return rc_;    \
   } while (0)
 
-int ggemm(hipStream_t st, int mode, const int* seg, int n_seg, const void* a, int64_t lda, int ta,
+int ggemm(jpp_stage* s, hipStream_t st, int mode, const int* seg, int n_seg, const void* a, int64_t lda, int ta,
           const void* b, int64_t ldb, int tb, int64_t stride_b, void* c, int64_t ldc,
           int64_t stride_c, int64_t m, int64_t n, int64_t k, int epi, int64_t rows,
           const void* aux = nullptr, int64_t ldaux = 0, void* c2 = nullptr, int64_t ldc2 = 0) {
@@ -139,7 +139,7 @@ int ggemm(hipStream_t st, int mode, const int* seg, int n_seg, const void* a, in
   g.group_rows = rows;
   g.seg_rows = seg + n_seg + 1;   // the routing kernels leave the token counts behind the offsets
   g.aux = aux; g.ldaux = ldaux; g.c2 = c2; g.ldc2 = ldc2;
-  return jpp_gemm_bf16(st, &g);
+  return s->d.dtype == JPP_DTYPE_F32 ? jpp_gemm_f32(st, &g) : jpp_gemm_bf16(st, &g);
 }
 
 void moe_args(jpp_stage* s, jpp_moe_args& m, uint8_t* slot, const LayerStash& L, int chunk,
@@ -155,6 +155,7 @@ void moe_args(jpp_stage* s, jpp_moe_args& m, uint8_t* slot, const LayerStash& L,
   m.seg = (int32_t*)(slot + L.seg.off);
   m.work = s->S<>(s->s_moework);
   m.tokens = s->T; m.hidden = s->h; m.n_experts = s->d.n_experts; m.top_k = s->d.top_k;
+  m.dtype = s->d.dtype;
 }
 
 int gemm(jpp_stage* s, hipStream_t st, const void* a, int64_t lda, int ta, const void* b, int64_t ldb, int tb,
@@ -325,10 +326,10 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
     RC(jpp_moe_gather(st, &ma, at(L.n2), at(L.xp)));
     // gate and up columns of each expert's Wgu are interleaved in blocks of 32, as in the
     // dense layer: SwiGLU runs in the epilogue
-    RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.xp), h, 0, s->P(chunk, li, X_Wgu), 2 * f, 1, h * 2 * f,
+    RC(ggemm(s, st, JPP_GROUP_M, seg, E, at(L.xp), h, 0, s->P(chunk, li, X_Wgu), 2 * f, 1, h * 2 * f,
              at(L.gu), 2 * f, 0, s->cap, 2 * f, h, JPP_EPI_SWIGLU, s->T * s->d.top_k, nullptr, 0,
              at(L.s), f));
-    RC(ggemm(st, JPP_GROUP_M, seg, E, at(L.s), f, 0, s->P(chunk, li, X_Wd), h, 1, f * h, at(L.eo), h,
+    RC(ggemm(s, st, JPP_GROUP_M, seg, E, at(L.s), f, 0, s->P(chunk, li, X_Wd), h, 1, f * h, at(L.eo), h,
              0, s->cap, h, f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_fwd(st, &ma, at(L.eo), at(L.h1), y));
     return JPP_OK;
@@ -418,9 +419,9 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     const int E = s->d.n_experts;
     void* dxp = s->S<>(s->s_t4);
     RC(jpp_moe_bwd_prepare(st, &ma, dy, at(L.eo), (float*)wt(W.dlogits), wt(W.deo)));
-    RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.deo), h, 0, s->P(chunk, li, X_Wd), h, 0, f * h,
+    RC(ggemm(s, st, JPP_GROUP_M, ma.seg, E, wt(W.deo), h, 0, s->P(chunk, li, X_Wd), h, 0, f * h,
              wt(W.dgu), 2 * f, 0, s->cap, f, h, JPP_EPI_DSWIGLU, s->T * s->d.top_k, at(L.gu), 2 * f));
-    RC(ggemm(st, JPP_GROUP_M, ma.seg, E, wt(W.dgu), 2 * f, 0, s->P(chunk, li, X_Wgu), 2 * f, 0,
+    RC(ggemm(s, st, JPP_GROUP_M, ma.seg, E, wt(W.dgu), 2 * f, 0, s->P(chunk, li, X_Wgu), 2 * f, 0,
              h * 2 * f, dxp, h, 0, s->cap, h, 2 * f, JPP_EPI_BF16, s->T * s->d.top_k));
     RC(jpp_moe_combine_bwd(st, &ma, dxp, (const float*)wt(W.dlogits), dn));
   } else {
@@ -477,9 +478,9 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
     jpp_moe_args ma;
     moe_args(s, ma, slot, L, chunk, li);
     const int E = s->d.n_experts;
-    RC(ggemm(st, JPP_GROUP_K, ma.seg, E, at(L.s), f, 1, wt(W.deo), h, 1, 0, s->G(chunk, li, X_Wd), h,
+    RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.s), f, 1, wt(W.deo), h, 1, 0, s->G(chunk, li, X_Wd), h,
              f * h, f, h, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
-    RC(ggemm(st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, wt(W.dgu), 2 * f, 1, 0,
+    RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, wt(W.dgu), 2 * f, 1, 0,
              s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
     RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)wt(W.dlogits), s->G(chunk, li, X_Wr),
                             partial));
@@ -604,9 +605,8 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   JPP_REQUIRE(d->dtype == JPP_DTYPE_BF16 || d->dtype == JPP_DTYPE_F32, "stage_create: unknown dtype %d",
               d->dtype);
   if (d->dtype == JPP_DTYPE_F32)
-    JPP_REQUIRE(d->family != JPP_FAMILY_MIXTRAL && d->fused_wgrad_accum,
-                "stage_create: f32 stages exist for the dense families, with the accumulation "
-                "in the weight-gradient GEMM");
+    JPP_REQUIRE(d->fused_wgrad_accum,
+                "stage_create: f32 stages accumulate in the weight-gradient GEMM");
 
   jpp_stage* s = new jpp_stage();
   s->d = *d;

@@ -63,7 +63,8 @@ class MoeArgs(C.Structure):
     _fields_ = [("x", C.c_void_p), ("wr", C.c_void_p), ("ids", C.c_void_p), ("gates", C.c_void_p),
                 ("row_of", C.c_void_p), ("tok_of", C.c_void_p), ("gate_of", C.c_void_p),
                 ("seg", C.c_void_p), ("work", C.c_void_p), ("tokens", C.c_int64),
-                ("hidden", C.c_int64), ("n_experts", C.c_int), ("top_k", C.c_int)]
+                ("hidden", C.c_int64), ("n_experts", C.c_int), ("top_k", C.c_int),
+                ("dtype", C.c_int)]
 
 
 class AdamArgs(C.Structure):

@@ -140,9 +140,8 @@ def test_gemm_f32_rejects_what_it_does_not_do():
         rt.gemm(d.ptr, d.ptr, d.ptr, 32, 64, 16, 16, 64, 64, 0, 1, f32=True)
     with pytest.raises(rt.JppError, match="SwiGLU epilogue needs c2"):
         rt.gemm(d.ptr, d.ptr, d.ptr, 64, 64, 16, 16, 64, 64, 0, 1, rt.EPI_SWIGLU, f32=True)
-    with pytest.raises(rt.JppError, match="grouped problems are bf16 only"):
-        rt.gemm(d.ptr, d.ptr, d.ptr, 64, 64, 16, 16, 64, 64, 0, 1, f32=True, seg=d.ptr, n_seg=1,
-                group_mode=1)
+    with pytest.raises(rt.JppError, match="grouped problem needs seg"):
+        rt.gemm(d.ptr, d.ptr, d.ptr, 64, 64, 16, 16, 64, 64, 0, 1, f32=True, group_mode=1)
 
 
 @pytest.mark.parametrize("ln", [True, False], ids=["layernorm", "rmsnorm"])
@@ -264,7 +263,13 @@ LLAMA_F32 = LayerSpec("llama", 256, 2, 384, 128, 2, n_kv_heads=1, head_dim=128, 
 LLAMA_D64_F32 = LayerSpec("llama", 256, 4, 256, 256, 1, n_kv_heads=2, head_dim=64, causal=True,
                           rope_theta=1e4, eps=1e-5, dtype="f32")
 
+MIXTRAL_F32 = LayerSpec("mixtral", 256, 2, 256, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
+                        rope_theta=5e5, eps=1e-5, n_experts=8, top_k=2, dtype="f32")
+
 STAGES_F32 = [
+    ("mixtral-1f1b", MIXTRAL_F32, S.Std1F1B(2), 3, 1, 2),
+    ("mixtral-dualpipev", MIXTRAL_F32, S.DualPipeV(4, 2), 4, 0, 1),
+    ("mixtral-zb", MIXTRAL_F32, S.ZeroBubble(2), 3, 1, 1),
     ("llama-interleaved", LLAMA_F32, S.Interleaved1F1B(4, 2), 4, 0, 2),
     ("llama-zb", LLAMA_D64_F32, S.ZeroBubble(3), 3, 1, 2),
     ("llama-dualpipev", LLAMA_F32, S.DualPipeV(4, 2), 4, 1, 1),
@@ -300,11 +305,9 @@ def test_f32_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
                 close(got, want.reshape(got.shape).astype(np.float64), 1e-4, f"grad {s}/{li}/{pname}")
 
 
-def test_f32_stage_needs_a_family_with_f32_operators():
-    spec = LayerSpec("mixtral", 256, 2, 256, 128, 2, n_kv_heads=1, head_dim=128, causal=True,
-                     n_experts=8, top_k=2, dtype="f32")
-    with pytest.raises(rt.JppError, match="f32 stages exist for the dense families"):
-        rt.StageExecutor(spec, 1, 1, 1)
+def test_f32_stage_accumulates_in_the_gemm():
+    with pytest.raises(rt.JppError, match="f32 stages accumulate in the weight-gradient GEMM"):
+        rt.StageExecutor(CFG1, 1, 1, 1, fused_wgrad_accum=False)
 
 
 def test_cfg1_train_step_through_the_public_api():
