@@ -400,3 +400,46 @@ def test_f32_stage_adam_after_loop():
                 assert np.abs(gw - host[li][k]).max() > 0, f"{k} did not move"
             assert all(not a.any() for a in ex.get_grads(0, li).values())
     ex.close()
+
+
+def test_example_model_train_step_in_float32():
+    """The reference's example at its default dtype (examples/basic.py:36, :72, :100: float32): a
+    stack of pre-LN causal decoder blocks, a stage marker after every `num_layers // pp`
+    layers, uniform inputs (:238), loss mean((res - batch)**2) / num_ubatches, Std1F1B over two
+    stages; losses and gradients against the sequential loop at 1e-4."""
+    from functools import partial
+
+    import jaxpp_amd as jaxpp
+    from oracle import stage as O
+
+    spec = LayerSpec("decoder", 256, 2, 512, 128, 1, causal=True, eps=1e-6, gelu_tanh=True,
+                     dtype="f32")
+    n_mb, pp, n_layers = 4, 2, 4
+    schedule = jaxpp.Std1F1B(pp)
+    model = jaxpp.nn.TransformerStack(spec, n_layers=n_layers, layers_per_stage=n_layers // pp)
+    params = model.init(seed=0, perturb=True)
+    batch = np.random.default_rng(2).uniform(size=(n_mb, spec.tokens, spec.hidden)).astype(np.float32)
+    mesh = jaxpp.MpmdMesh(jaxpp.DeviceMesh(np.arange(pp).reshape(pp, 1), ("mpmd", "data")), "mpmd")
+
+    def loss_fn(pars, mb):
+        res = model.apply(pars, mb)
+        return jaxpp.nn.mse_loss(res, mb) / n_mb, (res, 4)
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=mesh)
+    def train_step(pars, batch):
+        mubatch_grad = partial(jaxpp.value_and_grad(loss_fn, has_aux=True), pars)
+        (losses, (pred, _)), grad = jaxpp.treduce(mubatch_grad, batch, schedule=schedule)
+        return losses, pred, grad
+
+    losses, pred, grad = train_step(params, batch)
+    per = n_layers // pp
+    stages = [params["layers"][s * per:(s + 1) * per] for s in range(pp)]
+    want_loss, want_acc = O.treduce_sequential(L.LayerCfg(**spec.as_dict()), stages, list(batch),
+                                               L.Numerics.f32())
+    close(losses, want_loss.astype(np.float64), 1e-4, "losses")
+    for s in range(pp):
+        for li in range(per):
+            for k, v in want_acc[s][li].items():
+                got = grad["layers"][s * per + li][k]
+                close(got, v.reshape(got.shape).astype(np.float64), 1e-4, f"grad {s}/{li}/{k}")
+    train_step.close()
