@@ -46,4 +46,5 @@ def test_struct_layouts_match_header_sizes():
     assert ctypes.sizeof(rt.AttnArgs) == 10 * 8 + 8 * 8 + 6 * 4
     assert ctypes.sizeof(rt.NormArgs) == 12 * 8 + 2 * 8 + 8
     assert ctypes.sizeof(rt.StageDesc) == 21 * 4
+    assert ctypes.sizeof(rt.MoeArgs) == 9 * 8 + 2 * 8 + 3 * 4 + 4      # 3 ints, padded to 8
     assert ctypes.sizeof(rt.AdamArgs) == 8 + 5 * 8 + 8 + 5 * 8 + 8
