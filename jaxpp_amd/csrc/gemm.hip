@@ -75,14 +75,21 @@ __device__ __forceinline__ void swiglu_grad_f(float g, float u, float d, float& 
 // XCDs (8 of them, each with its own L2); give every XCD a contiguous range of
 // tiles, and inside a range walk GROUP tile-rows at a time so the B panels in
 // flight stay L2 resident.
+#ifndef JPP_COLUMN_SPLIT_ROWS
+#define JPP_COLUMN_SPLIT_ROWS 64
+#endif
+constexpr int kColumnSplitRows = JPP_COLUMN_SPLIT_ROWS;  // tile rows from which XCDs split by columns
+
 __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int nwg = tiles_m * tiles_n;
-  if ((tiles_n & 7) == 0 && tiles_m >= 64) {
+  if ((tiles_n & 7) == 0 && tiles_m >= kColumnSplitRows) {
     // Very tall outputs (the experts' row-grouped products: 16 384 token copies and more):
     // every XCD owns an eighth of the tile columns and walks them 8 tile-rows at a time, so a
     // B panel - which changes from expert to expert - is fetched by one XCD only.  The split
     // below would hand whole row groups to single XCDs and have each of them stream every
-    // column of B (+1.3 % on the Mixtral-shaped stage; at 16 tile-rows it costs 2.5 %).
+    // column of B (+1.3 % on the Mixtral-shaped stage and, through the 112-tile-row weight
+    // gradient of its down projection, +0.8 % on the 70B-shaped one; at 16 tile-rows it costs
+    // 2.5 %, at 56 it changes nothing).
     const int x = pid & 7, l = pid >> 3, cols_per = tiles_n >> 3;
     const int group = l / (8 * cols_per), within = l - group * 8 * cols_per;
     const int gsize = min(tiles_m - group * 8, 8);
