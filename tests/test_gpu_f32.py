@@ -134,6 +134,43 @@ def test_gemm_f32_swiglu_epilogues_and_rope():
     close(bx.download(np.float32, (B * S, ld)), x.astype(np.float64), 1e-5, "rope then inverse")
 
 
+def test_gemm_f32_grouped_modes():
+    rng = np.random.default_rng(12)
+    E, h, f = 8, 128, 192
+    counts = [300, 0, 256, 17, 700, 1, 255, 512]
+    seg = np.zeros(E + 1, np.int32)
+    for e, c in enumerate(counts):
+        seg[e + 1] = seg[e] + (c + 255) // 256 * 256
+    cap = int(seg[E]) + 256
+    xp = np.zeros((cap, h), np.float32)
+    dy = np.zeros((cap, f), np.float32)
+    for e, c in enumerate(counts):
+        xp[seg[e]:seg[e] + c] = rng.standard_normal((c, h), dtype=np.float32)
+        dy[seg[e]:seg[e] + c] = rng.standard_normal((c, f), dtype=np.float32)
+    w = rng.standard_normal((E, h, f), dtype=np.float32) * np.float32(0.1)
+    b_seg = rt.DeviceBuffer.from_numpy(seg)
+    b_xp, b_w, b_dy = dev(xp), dev(w), dev(dy)
+    out = dev(np.zeros((cap, f), np.float32))
+    rt.gemm(b_xp.ptr, b_w.ptr, out.ptr, cap, f, h, h, f, f, 0, 1, rt.EPI_BF16, seg=b_seg.ptr, n_seg=E,
+            group_mode=1, stride_b=h * f, f32=True)
+    rt.sync()
+    got = out.download(np.float32, (cap, f))
+    for e in range(E):
+        if counts[e]:
+            close(got[seg[e]:seg[e + 1]], xp[seg[e]:seg[e + 1]].astype(np.float64) @ w[e], 1e-5, f"group {e}")
+    assert not got[seg[E]:].any(), "tiles past the last group must not be written"
+    acc0 = rng.standard_normal((E, h, f), dtype=np.float32)
+    b_acc = dev(acc0)
+    rt.gemm(b_xp.ptr, b_dy.ptr, b_acc.ptr, h, f, 0, h, f, f, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
+            n_seg=E, group_mode=2, stride_c=h * f, f32=True)
+    rt.sync()
+    gw = b_acc.download(np.float32, (E, h, f))
+    for e in range(E):
+        want = acc0[e] + xp[seg[e]:seg[e + 1]].astype(np.float64).T @ dy[seg[e]:seg[e + 1]]
+        close(gw[e], want, 1e-5, f"dW group {e}")
+    np.testing.assert_array_equal(gw[1], acc0[1])       # empty group: untouched
+
+
 def test_gemm_f32_rejects_what_it_does_not_do():
     d = rt.DeviceBuffer(64 * 64 * 4)
     with pytest.raises(rt.JppError, match="multiples of 64"):
