@@ -48,3 +48,35 @@ def test_struct_layouts_match_header_sizes():
     assert ctypes.sizeof(rt.StageDesc) == 21 * 4
     assert ctypes.sizeof(rt.MoeArgs) == 9 * 8 + 2 * 8 + 3 * 4 + 4      # 3 ints, padded to 8
     assert ctypes.sizeof(rt.AdamArgs) == 8 + 5 * 8 + 8 + 5 * 8 + 8
+
+
+def test_struct_fields_match_the_header_as_a_c_compiler_sees_it(tmp_path):
+    """Every ctypes mirror against the header itself: a C program prints sizeof and the offset of
+    every field (a field missing from the header fails to compile, a reordered or retyped one
+    changes an offset)."""
+    import shutil
+    import subprocess
+    import pytest
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    pairs = {"jpp_gemm_args": rt.GemmArgs, "jpp_attn_args": rt.AttnArgs, "jpp_norm_args": rt.NormArgs,
+             "jpp_moe_args": rt.MoeArgs, "jpp_stage_desc": rt.StageDesc, "jpp_adam_args": rt.AdamArgs,
+             "jpp_colsum_item": rt.ColsumItem}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "jaxpp_amd.h"', 'int main(void) {']
+    for cname, cls in pairs.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, _ in cls._fields_:
+            lines.append(f'  printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines += ['  return 0;', '}']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run([cc, "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                   check=True, capture_output=True)
+    got = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True,
+                                                 text=True).stdout.splitlines())
+    for cname, cls in pairs.items():
+        assert int(got[cname]) == ctypes.sizeof(cls), cname
+        for fname, _ in cls._fields_:
+            assert int(got[f"{cname}.{fname}"]) == getattr(cls, fname).offset, f"{cname}.{fname}"
