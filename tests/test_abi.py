@@ -80,3 +80,30 @@ def test_struct_fields_match_the_header_as_a_c_compiler_sees_it(tmp_path):
         assert int(got[cname]) == ctypes.sizeof(cls), cname
         for fname, _ in cls._fields_:
             assert int(got[f"{cname}.{fname}"]) == getattr(cls, fname).offset, f"{cname}.{fname}"
+
+
+def test_enum_values_match_the_header(tmp_path):
+    import shutil
+    import subprocess
+    import pytest
+    from jaxpp_amd.types import TaskType
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    want = {"JPP_EPI_BF16": rt.EPI_BF16, "JPP_EPI_GELU": rt.EPI_GELU, "JPP_EPI_DGELU": rt.EPI_DGELU,
+            "JPP_EPI_ACC_F32": rt.EPI_ACC_F32, "JPP_EPI_F32": rt.EPI_F32, "JPP_EPI_SWIGLU": rt.EPI_SWIGLU,
+            "JPP_EPI_DSWIGLU": rt.EPI_DSWIGLU, "JPP_FAMILY_BERT": rt.FAMILY["bert"],
+            "JPP_FAMILY_LLAMA": rt.FAMILY["llama"], "JPP_FAMILY_MIXTRAL": rt.FAMILY["mixtral"],
+            "JPP_FAMILY_DECODER": rt.FAMILY["decoder"], "JPP_DTYPE_BF16": rt.DTYPE["bf16"],
+            "JPP_DTYPE_F32": rt.DTYPE["f32"], "JPP_FWD": TaskType.FWD.value, "JPP_BWD": TaskType.BWD.value,
+            "JPP_BWD_I": TaskType.BWD_I.value, "JPP_BWD_W": TaskType.BWD_W.value,
+            "JPP_NORM_PARTIALS": rt.NORM_PARTIALS, "JPP_GROUP_M": 1, "JPP_GROUP_K": 2}
+    body = "\n".join(f'  printf("{k} %d\\n", (int){k});' for k in want)
+    src = tmp_path / "enums.c"
+    src.write_text('#include <stdio.h>\n#include "jaxpp_amd.h"\nint main(void) {\n' + body + "\n  return 0;\n}\n")
+    exe = tmp_path / "enums"
+    subprocess.run([cc, "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                   check=True, capture_output=True)
+    got = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True,
+                                                 text=True).stdout.splitlines())
+    assert {k: int(v) for k, v in got.items()} == want
