@@ -3,8 +3,11 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <algorithm>
+
 #include "common.h"
 
+#include <mutex>
 #include <string>
 #include <utility>
 #include <vector>
@@ -12,30 +15,106 @@
 namespace {
 thread_local char g_err[1024] = "";
 
+// The launch probe.  One probe at a time, shared by every host thread: all of its state sits
+// behind `mu`, which a probed launch holds from the event in front of the kernel to the event
+// behind it, so launches from several threads cannot interleave their brackets.  Events come
+// from a pool of at most kProbeRing pairs: when every pair is in use the oldest one is waited
+// for, read and reused, so the number of live events is bounded however long the probe stays
+// open.  The first HIP error is kept and reported by jpp_probe_end; after it the probe stops
+// recording (launches go on unbracketed).
+constexpr size_t kProbeRing = 4096;
+
 struct Probe {
+  std::mutex mu;                 // guards every field below
+  std::mutex launch_mu;          // held across one bracketed launch
   bool active = false;
   std::string cls;
-  std::vector<std::pair<hipEvent_t, hipEvent_t>> events;
-  hipEvent_t open_ev = nullptr;
-  double flops = 0, bytes = 0;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> ring;  // created on demand, reused
+  size_t head = 0, live = 0;     // oldest pair in flight, number in flight
+  bool open = false;             // ring[(head + live) % size].first has been recorded
+  int64_t launches = 0;
+  double ms = 0, flops = 0, bytes = 0;
+  hipError_t err = hipSuccess;
+  char err_what[96] = "";
+
+  void fail(hipError_t e, const char* what) {
+    if (err == hipSuccess) {
+      err = e;
+      snprintf(err_what, sizeof(err_what), "%s", what);
+    }
+  }
+  // waits for the oldest pair in flight and folds its duration into the total
+  void retire_oldest() {
+    auto& ev = ring[head];
+    float t = 0;
+    hipError_t e = hipEventSynchronize(ev.second);
+    if (e == hipSuccess) e = hipEventElapsedTime(&t, ev.first, ev.second);
+    if (e != hipSuccess) fail(e, "reading a launch's events");
+    else ms += t;
+    head = (head + 1) % ring.size();
+    --live;
+  }
 } g_probe;
 }  // namespace
 
 bool jpp_probe_wants(const char* kernel_class) {
-  return g_probe.active && g_probe.cls == kernel_class;
+  std::lock_guard<std::mutex> lock(g_probe.mu);
+  return g_probe.active && g_probe.err == hipSuccess && g_probe.cls == kernel_class;
 }
+
 void jpp_probe_open(hipStream_t stream) {
-  hipEventCreate(&g_probe.open_ev);
-  hipEventRecord(g_probe.open_ev, stream);
+  g_probe.launch_mu.lock();      // released by jpp_probe_close
+  std::lock_guard<std::mutex> lock(g_probe.mu);
+  Probe& p = g_probe;
+  if (!p.active || p.err != hipSuccess) return;
+  if (p.live == p.ring.size()) {
+    if (p.ring.size() < kProbeRing) {
+      // grow: only while the ring has not wrapped (head == 0), so order is kept
+      hipEvent_t a = nullptr, b = nullptr;
+      hipError_t e = hipEventCreate(&a);
+      if (e == hipSuccess) e = hipEventCreate(&b);
+      if (e != hipSuccess) {
+        if (a) hipEventDestroy(a);
+        p.fail(e, "hipEventCreate");
+        return;
+      }
+      if (p.head != 0) {         // rotate so that the oldest pair is first again
+        std::rotate(p.ring.begin(), p.ring.begin() + p.head, p.ring.end());
+        p.head = 0;
+      }
+      p.ring.emplace_back(a, b);
+    } else {
+      p.retire_oldest();
+    }
+  }
+  auto& ev = p.ring[(p.head + p.live) % p.ring.size()];
+  const hipError_t e = hipEventRecord(ev.first, stream);
+  if (e != hipSuccess) {
+    p.fail(e, "hipEventRecord in front of a launch");
+    return;
+  }
+  p.open = true;
 }
+
 void jpp_probe_close(hipStream_t stream, double flops, double bytes) {
-  hipEvent_t stop;
-  hipEventCreate(&stop);
-  hipEventRecord(stop, stream);
-  g_probe.events.emplace_back(g_probe.open_ev, stop);
-  g_probe.open_ev = nullptr;
-  g_probe.flops += flops;
-  g_probe.bytes += bytes;
+  {
+    std::lock_guard<std::mutex> lock(g_probe.mu);
+    Probe& p = g_probe;
+    if (p.open) {
+      p.open = false;
+      auto& ev = p.ring[(p.head + p.live) % p.ring.size()];
+      const hipError_t e = hipEventRecord(ev.second, stream);
+      if (e != hipSuccess) {
+        p.fail(e, "hipEventRecord behind a launch");
+      } else {
+        ++p.live;
+        ++p.launches;
+        p.flops += flops;
+        p.bytes += bytes;
+      }
+    }
+  }
+  g_probe.launch_mu.unlock();
 }
 
 int jpp_set_error(int code, const char* fmt, ...) {
@@ -165,33 +244,32 @@ int jpp_event_elapsed_ms(void* start, void* stop, float* ms) {
 }
 int jpp_probe_begin(const char* kernel_class) {
   JPP_REQUIRE(kernel_class && *kernel_class, "probe_begin: empty class name");
+  std::lock_guard<std::mutex> lock(g_probe.mu);
   JPP_REQUIRE(!g_probe.active, "probe_begin: a probe is already active");
   g_probe.active = true;
   g_probe.cls = kernel_class;
-  g_probe.flops = g_probe.bytes = 0;
+  g_probe.head = g_probe.live = 0;
+  g_probe.open = false;
+  g_probe.launches = 0;
+  g_probe.ms = g_probe.flops = g_probe.bytes = 0;
+  g_probe.err = hipSuccess;
+  g_probe.err_what[0] = 0;
   return JPP_OK;
 }
 int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, double* total_bytes) {
-  JPP_REQUIRE(g_probe.active, "probe_end: no active probe");
-  g_probe.active = false;
-  double ms = 0;
-  hipError_t err = hipSuccess;
-  for (auto& ev : g_probe.events) {
-    float t = 0;
-    hipError_t e = hipEventSynchronize(ev.second);
-    if (e == hipSuccess) e = hipEventElapsedTime(&t, ev.first, ev.second);
-    if (e != hipSuccess) err = e;
-    ms += t;
-    hipEventDestroy(ev.first);
-    hipEventDestroy(ev.second);
-  }
-  if (launches) *launches = (int64_t)g_probe.events.size();
-  if (total_ms) *total_ms = ms;
-  if (total_flops) *total_flops = g_probe.flops;
-  if (total_bytes) *total_bytes = g_probe.bytes;
-  g_probe.events.clear();
-  if (err != hipSuccess)
-    return jpp_set_error(JPP_ERR_HIP, "probe_end: %s", hipGetErrorString(err));
+  std::lock_guard<std::mutex> launch_lock(g_probe.launch_mu);  // no bracket half open
+  std::lock_guard<std::mutex> lock(g_probe.mu);
+  Probe& p = g_probe;
+  JPP_REQUIRE(p.active, "probe_end: no active probe");
+  p.active = false;
+  while (p.live) p.retire_oldest();
+  if (launches) *launches = p.launches;
+  if (total_ms) *total_ms = p.ms;
+  if (total_flops) *total_flops = p.flops;
+  if (total_bytes) *total_bytes = p.bytes;
+  if (p.err != hipSuccess)
+    return jpp_set_error(JPP_ERR_HIP, "probe: %s failed: %s (timings are incomplete)", p.err_what,
+                         hipGetErrorString(p.err));
   return JPP_OK;
 }
 int jpp_mem_info(size_t* free_bytes, size_t* total_bytes) {

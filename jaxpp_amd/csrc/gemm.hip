@@ -22,6 +22,9 @@
 #include <math.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <string>
+
 #include "common.h"
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -483,16 +486,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 
 template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS>
 const char* class_name() {
-  static char name[64] = "";
-  if (!name[0]) {
+  // built once per instantiation; the initialisation of a function-local static is
+  // thread-safe
+  static const std::string name = [] {
+    char buf[64];
     const char* lay = TA ? "tn" : (TB ? "nn" : "nt");
     const char* epi = EPI == JPP_EPI_BF16 ? "bf16" : EPI == JPP_EPI_GELU ? "gelu"
                     : EPI == JPP_EPI_DGELU ? "dgelu" : EPI == JPP_EPI_ACC_F32 ? "accf32"
                     : EPI == JPP_EPI_SWIGLU ? "swiglu" : EPI == JPP_EPI_DSWIGLU ? "dswiglu" : "f32";
-    snprintf(name, sizeof(name), "gemm_%s_%s_%dx%d%s%s", lay, epi, BM, BN, NW == 8 ? "w8" : "",
+    snprintf(buf, sizeof(buf), "gemm_%s_%s_%dx%d%s%s", lay, epi, BM, BN, NW == 8 ? "w8" : "",
              NS == 2 ? "" : NS == 3 ? "s3" : "s4");
-  }
-  return name;
+    return std::string(buf);
+  }();
+  return name.c_str();
 }
 
 template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4, int NS = 2>
@@ -513,12 +519,15 @@ int launch(hipStream_t stream, GemmParams& p) {
                    2.0 * am * ak + b_bytes + copies * am * p.n * cb);
   auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW, NS>;
   static_assert(SMEM <= 160 * 1024, "LDS of one CU");
-  static bool configured = false;  // per instantiation; attribute is sticky
-  if (!configured) {
-    JPP_CHECK_HIP(hipFuncSetAttribute((const void*)kern,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, SMEM));
-    configured = true;
-  }
+  // the LDS limit of a kernel is sticky: set once per instantiation, by whichever host
+  // thread launches it first (the others wait for that call and see its result)
+  static std::once_flag configured;
+  static hipError_t configure_rc = hipSuccess;
+  std::call_once(configured, [&] {
+    configure_rc = hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+  });
+  JPP_CHECK_HIP(configure_rc);
   p.tiles_m = p.m / BM;
   p.tiles_n = p.n / BN;
   const int blocks = p.tiles_m * p.tiles_n * (p.group_mode == JPP_GROUP_K ? p.n_seg : 1);
@@ -584,6 +593,7 @@ int dispatch(hipStream_t stream, const jpp_gemm_args* a, GemmParams& p, int tile
   JPP_GEMM_CASE(0, 1, JPP_EPI_GELU);     // forward + GELU
   JPP_GEMM_CASE(0, 1, JPP_EPI_F32);      // forward, f32 out (router logits)
   JPP_GEMM_CASE(0, 1, JPP_EPI_SWIGLU);   // gate/up projection + SwiGLU
+  JPP_GEMM_CASE(0, 1, JPP_EPI_ACC_F32);  // weight gradient from a transposed activation
   JPP_GEMM_CASE(0, 0, JPP_EPI_BF16);     // input gradient
   JPP_GEMM_CASE(0, 0, JPP_EPI_DGELU);    // input gradient through GELU
   JPP_GEMM_CASE(0, 0, JPP_EPI_DSWIGLU);  // input gradient through SwiGLU
