@@ -405,6 +405,14 @@ size_t jpp_stage_bytes(const jpp_stage* stage);
 int jpp_stage_run_task(jpp_stage* stage, int kind, int chunk, int mubatch, const void* in,
                        void* out, void* stream);
 int jpp_stage_live_slots(const jpp_stage* stage);
+/* Mixture-of-experts stages: the routing a forward task chose for one layer of a live
+ * (chunk, microbatch) - between its FWD and the task that releases its residuals - copied on
+ * `stream` into caller-owned device buffers: ids int32 [tokens, top_k] (experts by descending
+ * logit) and gates f32 [tokens, top_k]; either may be NULL.  The reference leaves routing to
+ * the user's model; a host needs it for load statistics and auxiliary losses, and the parity
+ * tests to hold the oracle to the device's choice where router logits tie within rounding. */
+int jpp_stage_routing(jpp_stage* stage, int chunk, int mubatch, int layer, int32_t* ids,
+                      float* gates, void* stream);
 
 #ifdef __cplusplus
 }

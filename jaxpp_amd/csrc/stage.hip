@@ -867,6 +867,28 @@ int jpp_stage_adam_step(jpp_stage* s, void* stream, int64_t step, double lr, dou
   return jpp_adam_step(stream, &a);
 }
 
+int jpp_stage_routing(jpp_stage* s, int chunk, int mb, int layer, int32_t* ids, float* gates,
+                      void* stream) {
+  JPP_REQUIRE(s, "stage_routing: null stage");
+  JPP_REQUIRE(s->d.family == JPP_FAMILY_MIXTRAL, "stage_routing: not a mixture-of-experts stage");
+  JPP_REQUIRE(chunk >= 0 && chunk < s->d.n_chunks && layer >= 0 && layer < s->d.layers_per_chunk,
+              "stage_routing: (chunk %d, layer %d) out of range", chunk, layer);
+  JPP_REQUIRE(ids || gates, "stage_routing: nothing to copy");
+  auto it = s->live.find(std::make_pair(chunk, mb));
+  if (it == s->live.end())
+    return jpp_set_error(JPP_ERR_STATE, "stage_routing: (chunk %d, mubatch %d) holds no residuals",
+                         chunk, mb);
+  const uint8_t* slot = s->slots[it->second];
+  const LayerStash& L = s->lay[layer];
+  const size_t n = (size_t)s->T * s->d.top_k * 4;
+  if (ids)
+    JPP_CHECK_HIP(hipMemcpyAsync(ids, slot + L.ids.off, n, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+  if (gates)
+    JPP_CHECK_HIP(hipMemcpyAsync(gates, slot + L.gates.off, n, hipMemcpyDeviceToDevice,
+                                 (hipStream_t)stream));
+  return JPP_OK;
+}
+
 size_t jpp_stage_bytes(const jpp_stage* s) { return s ? s->total_bytes : 0; }
 int jpp_stage_live_slots(const jpp_stage* s) { return s ? (int)s->live.size() : 0; }
 

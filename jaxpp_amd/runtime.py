@@ -115,7 +115,7 @@ EXPORTS = [
     "jpp_stage_param_ptr", "jpp_stage_grad_ptr", "jpp_stage_zero_grads", "jpp_stage_join",
     "jpp_stage_quiesce",
     "jpp_stage_bytes",
-    "jpp_stage_run_task", "jpp_stage_live_slots",
+    "jpp_stage_run_task", "jpp_stage_live_slots", "jpp_stage_routing",
 ]
 
 
@@ -218,6 +218,8 @@ def load():
     lib.jpp_stage_run_task.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                        C.c_void_p, C.c_void_p]
     lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
+    lib.jpp_stage_routing.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                      C.c_void_p]
     lib.jpp_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int64, C.POINTER(C.c_double)]
     lib.jpp_adam_step.argtypes = [C.c_void_p, C.POINTER(AdamArgs)]
     lib.jpp_stage_optimizer_init.argtypes = [C.c_void_p, C.c_void_p]
@@ -616,6 +618,16 @@ class StageExecutor:
 
     def live_slots(self) -> int:
         return load().jpp_stage_live_slots(self.handle)
+
+    def routing(self, chunk: int, mubatch: int, layer: int):
+        """(expert ids [tokens, top_k] int32, gates [tokens, top_k] f32) a forward task of a
+        mixture-of-experts stage chose, while that microbatch's residuals are live."""
+        n = self.spec.tokens * self.spec.top_k
+        ids, gates = DeviceBuffer(4 * n), DeviceBuffer(4 * n)
+        check(load().jpp_stage_routing(self.handle, chunk, mubatch, layer, ids.ptr, gates.ptr, None))
+        sync()
+        shape = (self.spec.tokens, self.spec.top_k)
+        return ids.download(np.int32, shape), gates.download(np.float32, shape)
 
     def close(self):
         if getattr(self, "handle", None):

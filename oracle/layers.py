@@ -217,9 +217,11 @@ def rope_apply(x, cos, sin, inverse=False):
     return np.concatenate([x1 * c - x2 * s, x2 * c + x1 * s], -1)
 
 
-def attention_fwd(q, k, v, causal, acc=np.float32):
+def attention_fwd(q, k, v, causal, acc=np.float32, rt=identity):
     """q: [B,S,Hq,d]; k,v: [B,S,Hkv,d].  Returns o [B,S,Hq,d] and the row
-    log-sum-exp of the scaled scores [B,Hq,S]."""
+    log-sum-exp of the scaled scores [B,Hq,S].  ``rt`` rounds the probabilities
+    where they become an operand of the second product (a bf16 path multiplies
+    bf16 probabilities; the row sum is taken before rounding)."""
     B, S, Hq, d = q.shape
     Hkv = k.shape[2]
     grp = Hq // Hkv
@@ -233,12 +235,14 @@ def attention_fwd(q, k, v, causal, acc=np.float32):
     m = s.max(-1, keepdims=True)
     p = np.exp(s - m)
     l = p.sum(-1, keepdims=True)
-    o = np.matmul(p / l, va)
+    o = np.matmul(p / l, va) if rt is identity else np.matmul(rt(p).astype(acc), va) / l
     lse = (m + np.log(l))[..., 0]
     return o.transpose(0, 2, 1, 3), lse
 
 
-def attention_bwd(q, k, v, o, do, lse, causal, acc=np.float32):
+def attention_bwd(q, k, v, o, do, lse, causal, acc=np.float32, rt=identity):
+    """``rt`` rounds the recomputed probabilities and the score cotangents where
+    they become operands of the three gradient products."""
     B, S, Hq, d = q.shape
     Hkv = k.shape[2]
     grp = Hq // Hkv
@@ -252,10 +256,10 @@ def attention_bwd(q, k, v, o, do, lse, causal, acc=np.float32):
     if causal:
         s = np.where(np.tril(np.ones((S, S), bool)), s, -np.inf)
     p = np.exp(s - lse.astype(acc)[..., None])
-    dv = np.matmul(p.transpose(0, 1, 3, 2), doa)
+    dv = np.matmul(rt(p).astype(acc).transpose(0, 1, 3, 2), doa)
     dp = np.matmul(doa, va.transpose(0, 1, 3, 2))
     delta = (doa * oa).sum(-1, keepdims=True)
-    ds = p * (dp - delta) * scale
+    ds = rt(p * (dp - delta) * scale).astype(acc)
     dq = np.matmul(ds, ka)
     dk = np.matmul(ds.transpose(0, 1, 3, 2), qa)
     dk = dk.reshape(B, Hkv, grp, S, d).sum(2)
@@ -303,9 +307,13 @@ def _join_qkv(cfg: LayerCfg, q, k, v):
     return np.concatenate([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], -1)
 
 
-def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics):
+def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics, forced_ids=None):
     """Forward of one layer.  Returns (y, stash); the stash is what the
-    forward task hands to the backward task(s) of the same microbatch."""
+    forward task hands to the backward task(s) of the same microbatch.
+    ``forced_ids`` ([T, top_k] expert ids, mixture layers only) replaces the
+    layer's own top-k selection; the gates are the softmax over the logits of
+    the forced experts.  Tests use it to hold the oracle to the routing the
+    device chose where a token's logits tie within rounding."""
     rt, acc = nm.rt, nm.acc
     T, h = cfg.tokens, cfg.hidden
     assert x.shape == (T, h)
@@ -313,7 +321,7 @@ def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics):
     if cfg.family == "bert":
         qkv = rt(mm(x, p["Wqkv"], acc) + p["bqkv"].astype(acc))
         q, k, v = _split_qkv(cfg, qkv)
-        o, lse = attention_fwd(q, k, v, cfg.causal, acc)
+        o, lse = attention_fwd(q, k, v, cfg.causal, acc, rt)
         ctx = rt(o.reshape(T, -1))
         a = rt(mm(ctx, p["Wo"], acc) + p["bo"].astype(acc) + x.astype(acc))
         y1, mean1, rstd1 = layernorm_fwd(a, p["ln1_g"], p["ln1_b"], cfg.eps, acc)
@@ -335,7 +343,7 @@ def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics):
         n1 = rt(y1)
         qkv = rt(mm(n1, p["Wqkv"], acc) + p["bqkv"].astype(acc))
         q, k, v = _split_qkv(cfg, qkv)
-        o, lse = attention_fwd(q, k, v, cfg.causal, acc)
+        o, lse = attention_fwd(q, k, v, cfg.causal, acc, rt)
         ctx = rt(o.reshape(T, -1))
         h1 = rt(mm(ctx, p["Wo"], acc) + p["bo"].astype(acc) + x.astype(acc))
         y2, mean2, rstd2 = layernorm_fwd(h1, p["ln2_g"], p["ln2_b"], cfg.eps, acc)
@@ -356,7 +364,7 @@ def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics):
         q = rt(rope_apply(q.astype(acc), cos, sin))
         k = rt(rope_apply(k.astype(acc), cos, sin))
         qkv = _join_qkv(cfg, q, k, v)
-        o, lse = attention_fwd(q, k, v, cfg.causal, acc)
+        o, lse = attention_fwd(q, k, v, cfg.causal, acc, rt)
         ctx = rt(o.reshape(T, -1))
         h1 = rt(mm(ctx, p["Wo"], acc) + x.astype(acc))
         y2, rstd2 = rmsnorm_fwd(h1, p["rms2_g"], cfg.eps, acc)
@@ -368,7 +376,7 @@ def layer_fwd(cfg: LayerCfg, p: dict, x, nm: Numerics):
             y = rt(mm(s, p["Wd"], acc) + h1.astype(acc))
             st.update(gu=gu, s=s)
             return y, st
-        return _moe_fwd(cfg, p, n2, h1, st, nm)
+        return _moe_fwd(cfg, p, n2, h1, st, nm, forced_ids)
     raise ValueError(cfg.family)
 
 
@@ -393,7 +401,7 @@ def layer_bwd_i(cfg: LayerCfg, p: dict, st: dict, dy, nm: Numerics):
         B, S, d = cfg.batch, cfg.seq, cfg.d
         dq, dk, dv = attention_bwd(q, k, v, st["ctx"].reshape(B, S, cfg.n_heads, d),
                                    dctx.reshape(B, S, cfg.n_heads, d), st["lse"],
-                                   cfg.causal, acc)
+                                   cfg.causal, acc, rt)
         dqkv = rt(_join_qkv(cfg, dq, dk, dv))
         dx = rt(mm(dqkv, p["Wqkv"].T, acc) + da.astype(acc))
         small["b2"] = dc.astype(acc).sum(0)
@@ -413,7 +421,7 @@ def layer_bwd_i(cfg: LayerCfg, p: dict, st: dict, dy, nm: Numerics):
         B, S, d = cfg.batch, cfg.seq, cfg.d
         dq, dk, dv = attention_bwd(q, k, v, st["ctx"].reshape(B, S, cfg.n_heads, d),
                                    dctx.reshape(B, S, cfg.n_heads, d), st["lse"],
-                                   cfg.causal, acc)
+                                   cfg.causal, acc, rt)
         dqkv = rt(_join_qkv(cfg, dq, dk, dv))
         dn1 = rt(mm(dqkv, p["Wqkv"].T, acc))
         dx_, small["ln1_g"], small["ln1_b"] = layernorm_bwd(
@@ -440,7 +448,7 @@ def layer_bwd_i(cfg: LayerCfg, p: dict, st: dict, dy, nm: Numerics):
         B, S, d = cfg.batch, cfg.seq, cfg.d
         dq, dk, dv = attention_bwd(q, k, v, st["ctx"].reshape(B, S, cfg.n_heads, d),
                                    dctx.reshape(B, S, cfg.n_heads, d), st["lse"],
-                                   cfg.causal, acc)
+                                   cfg.causal, acc, rt)
         cos, sin = rope_tables(cfg.seq, cfg.d, cfg.rope_theta, acc)
         dq = rope_apply(rt(dq).astype(acc), cos, sin, inverse=True)
         dk = rope_apply(rt(dk).astype(acc), cos, sin, inverse=True)
@@ -486,11 +494,17 @@ def moe_route(logits, top_k):
     return order, e / e.sum(-1, keepdims=True)
 
 
-def _moe_fwd(cfg, p, n2, h1, st, nm):
+def _moe_fwd(cfg, p, n2, h1, st, nm, forced_ids=None):
     rt, acc = nm.rt, nm.acc
     T, f, E = cfg.tokens, cfg.ffn, cfg.n_experts
     logits = mm(n2, p["Wr"], acc).astype(acc)
     ids, gates = moe_route(logits, cfg.top_k)
+    st["own_ids"] = ids
+    if forced_ids is not None:
+        ids = np.asarray(forced_ids).reshape(T, cfg.top_k).astype(ids.dtype)
+        sel = np.take_along_axis(logits, ids, -1)
+        e = np.exp(sel - sel.max(-1, keepdims=True))
+        gates = e / e.sum(-1, keepdims=True)
     y = h1.astype(acc).copy()
     gu_all = np.zeros((T, cfg.top_k, 2 * f), acc)
     s_all = np.zeros((T, cfg.top_k, f), acc)

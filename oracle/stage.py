@@ -41,20 +41,43 @@ class RankOracle:
     """One rank holding one or more stages ("chunks"), each a list of layers."""
 
     def __init__(self, cfg: L.LayerCfg, chunks: dict, nm: L.Numerics,
-                 round_wgrad: bool = False):
+                 round_wgrad: bool = False, layer_cfgs: dict | None = None):
+        """``layer_cfgs``: stage_id -> [LayerCfg per layer] for stages whose layers differ
+        in shape or family; every other layer is a ``cfg`` layer."""
         self.cfg, self.nm, self.round_wgrad = cfg, nm, round_wgrad
+        self.layer_cfgs = layer_cfgs or {}
         self.chunks = chunks                       # stage_id -> [param dict per layer]
         self.acc = {s: [{k: np.zeros(v.shape, np.float32) for k, v in p.items()}
                         for p in ps] for s, ps in chunks.items()}
         self.stash, self.wstash = {}, {}
         self.live = self.peak_live = 0
+        # mixture layers: per (stage, microbatch) and layer, every token's gap between its
+        # last selected router logit and the best one left out (a small gap = a near tie,
+        # where top-k selection is discontinuous)
+        self.router_margin = {}
+        # (stage, microbatch) -> [expert ids [T, top_k] per layer] to impose on mixture layers
+        # (see layers.layer_fwd), and how many tokens that changed per layer
+        self.forced_ids = {}
+        self.forced_changes = {}
 
     # -- tasks -----------------------------------------------------------
+    def cfg_of(self, stage, li):
+        return self.layer_cfgs[stage][li] if stage in self.layer_cfgs else self.cfg
+
     def fwd(self, stage, mb, x):
         sts = []
-        for p in self.chunks[stage]:
-            x, st = L.layer_fwd(self.cfg, p, x, self.nm)
+        for li, p in enumerate(self.chunks[stage]):
+            forced = self.forced_ids.get((stage, mb))
+            x, st = L.layer_fwd(self.cfg_of(stage, li), p, x, self.nm,
+                                forced[li] if forced is not None else None)
             sts.append(st)
+            if forced is not None and "own_ids" in st:
+                changed = (np.sort(st["own_ids"], -1) != np.sort(st["ids"], -1)).any(-1)
+                self.forced_changes.setdefault((stage, mb), []).append(changed)
+            if "logits" in st:
+                k = self.cfg_of(stage, li).top_k
+                srt = np.sort(st["logits"].astype(np.float64), axis=-1)
+                self.router_margin.setdefault((stage, mb), []).append(srt[:, -k] - srt[:, -k - 1])
         self.stash[stage, mb] = sts
         self.live += 1
         self.peak_live = max(self.peak_live, self.live)
@@ -68,7 +91,8 @@ class RankOracle:
         sts = self.stash[stage, mb]
         wsts = [None] * len(sts)
         for li in reversed(range(len(sts))):
-            dy, wst, small = L.layer_bwd_i(self.cfg, self.chunks[stage][li], sts[li], dy, self.nm)
+            dy, wst, small = L.layer_bwd_i(self.cfg_of(stage, li), self.chunks[stage][li], sts[li], dy,
+                                           self.nm)
             wsts[li] = wst
             for name, g in small.items():
                 self._add(stage, li, name, g)
@@ -78,7 +102,7 @@ class RankOracle:
     def bwd_w(self, stage, mb):
         sts, wsts = self.stash.pop((stage, mb)), self.wstash.pop((stage, mb))
         for li in reversed(range(len(sts))):
-            for name, g in L.layer_bwd_w(self.cfg, sts[li], wsts[li], self.nm).items():
+            for name, g in L.layer_bwd_w(self.cfg_of(stage, li), sts[li], wsts[li], self.nm).items():
                 if self.round_wgrad:
                     g = self.nm.rt(g.astype(np.float32))
                 self._add(stage, li, name, g)
@@ -115,18 +139,22 @@ class RankOracle:
 # ---------------------------------------------------------------------------
 # whole model: sequential loop and scheduled pipeline (cfg "CPU plumbing")
 # ---------------------------------------------------------------------------
-def treduce_sequential(cfg, stage_layers, xs, nm, round_wgrad=False):
+def treduce_sequential(cfg, stage_layers, xs, nm, round_wgrad=False, targets=None,
+                       layer_cfgs=None):
     """The loop as ``treduce`` defines it: microbatches in order, every stage
-    forward then backward; losses concatenated, gradients summed."""
+    forward then backward; losses concatenated, gradients summed.  The loss
+    compares the last stage's output with ``targets[m]`` (default: the
+    microbatch itself, as in the reference's examples)."""
     n = len(xs)
-    ro = RankOracle(cfg, dict(enumerate(stage_layers)), nm, round_wgrad)
+    targets = xs if targets is None else targets
+    ro = RankOracle(cfg, dict(enumerate(stage_layers)), nm, round_wgrad, layer_cfgs)
     losses = np.zeros(n, np.float32)
     S = len(stage_layers)
     for m in range(n):
         a = xs[m]
         for s in range(S):
             a = ro.fwd(s, m, a)
-        losses[m], d = L.mse_loss(a, xs[m], n, nm.acc)
+        losses[m], d = L.mse_loss(a, targets[m], n, nm.acc)
         d = nm.rt(d.astype(np.float32))
         for s in reversed(range(S)):
             d = ro.bwd(s, m, d)

@@ -7,6 +7,8 @@ two schedules of the same work)."""
 import numpy as np
 import pytest
 
+import parity
+
 from jaxpp_amd import runtime as rt
 from jaxpp_amd import schedules as S
 from jaxpp_amd.model import LayerSpec, boundary_tensor, init_layer_params
@@ -35,11 +37,7 @@ def _gpu():
     rt.require_gpu()
 
 
-def close(got, want, rtol, what):
-    scale = float(np.abs(want).max()) + 1e-30
-    err = float(np.abs(got - want).max())
-    assert np.isfinite(got).all(), f"{what}: non-finite"
-    assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+close = parity.close
 
 
 def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_streams=True):
@@ -133,9 +131,9 @@ def test_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
     ys, dxs, grads = run_on_gpu(spec, plan, lpc, params, two_streams=two_streams)
     assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
     for k in ys_w:
-        close(ys[k], ys_w[k], 2e-2, f"y{k}")
+        parity.close_stage(ys[k], ys_w[k], 2e-2, f"y{k}")
     for k in dxs_w:
-        close(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
+        parity.close_stage(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
     bad = []
     for s in plan.stages:
         for li in range(lpc):
@@ -151,9 +149,13 @@ def test_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
                 # expert's gradient, so router and expert weights are held to 2e-2 in the
                 # Frobenius norm and 1e-1 in the max norm; all else to 2e-2 in the max norm.
                 routed = spec.family == "mixtral" and pname in ("Wr", "Wgu", "Wd")
-                ok = (fro <= 2e-2 and err <= 1e-1) if routed else err <= 2e-2
+                n_bad, n_el, worst = parity.violations(got, want, 2e-2)
+                ok = (fro <= 2e-2 and err <= 1e-1) if routed else (
+                    err <= 2e-2 and n_bad <= parity.STAGE_BAD_FRAC * n_el and worst <= parity.MAX_EXCESS)
                 if not (np.isfinite(got).all() and ok):
-                    bad.append(f"grad {s}/{li}/{pname}: max err {err:.4g}, frobenius {fro:.4g}")
+                    bad.append(f"grad {s}/{li}/{pname}: max err {err:.4g}, frobenius {fro:.4g}, "
+                               f"{n_bad} of {n_el} elements outside the elementwise bound "
+                               f"(worst {worst:.3g} x)")
     assert not bad, "\n".join(bad)
 
 
@@ -180,8 +182,9 @@ def test_unfused_accumulate_path_is_close():
     plan = make_rank_plan(S.Std1F1B(1), n, 0)
     a = run_on_gpu(spec, plan, 1, params, fused=True)
     b = run_on_gpu(spec, plan, 1, params, fused=False)
+    # the unfused path rounds each microbatch's weight gradient to bf16 before adding it
     for k, v in a[2][0][0].items():
-        close(b[2][0][0][k], v, 1e-2, k)
+        close(b[2][0][0][k], v, 2e-2, k)
 
 
 def test_lifetime_errors():

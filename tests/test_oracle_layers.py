@@ -4,6 +4,8 @@ differences, brute-force attention rows, scipy/torch special functions and
 algebraic invariants."""
 import math
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -258,3 +260,37 @@ def test_bf16_mode_stays_close_to_f32():
     y16, dx16, g16 = oracle_grads(spec, pb, x, dy, L.Numerics.bf16())
     for a, b in [(y16, y32), (dx16, dx32)] + [(g16[k], g32[k]) for k in g32]:
         assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max() + 1e-6
+
+
+@pytest.mark.skipif(not os.environ.get("JPP_SLOW_TESTS"),
+                    reason="about three minutes and 40 GB of host memory; set JPP_SLOW_TESTS=1")
+def test_bf16_sensitivity_of_a_70b_shaped_layer():
+    """How far two faithful bf16 evaluations of one Llama-70B-shaped layer (hidden 8192, 64 / 8
+    heads, SwiGLU 28672, 2048 tokens) may differ: the oracle accumulating in f32 against the
+    oracle accumulating in f64, same bf16 storage rounding.  Measured: no element of the
+    output, 2e-4 of the input cotangent (first tokens ahead) and 1.0e-3 of the QKV weight
+    gradient (all in the key columns) outside 2e-2 * (|want| + rms), worst 2.9 x.  This is the
+    yardstick for the fraction the full-size GPU test of the same layer grants."""
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import parity
+    from jaxpp_amd.model import LayerSpec, boundary_tensor
+    from test_gpu_full_size import big_params
+    spec = LayerSpec("llama", 8192, 64, 28672, 2048, 1, n_kv_heads=8, head_dim=128, causal=True,
+                     rope_theta=5e5, eps=1e-5)
+    cfg = L.LayerCfg(**spec.as_dict())
+    params = big_params(spec, [1], 1)[1][0]
+    shape = (spec.tokens, spec.hidden)
+    x = L.bf16_round(boundary_tensor("x", 1, 0, shape, 0))
+    dy = L.bf16_round(boundary_tensor("dy", 1, 0, shape, 0))
+    res = []
+    for nm in (L.Numerics.bf16(), L.Numerics(L.bf16_round, np.float64)):
+        y, st = L.layer_fwd(cfg, params, x, nm)
+        dx, wst, _ = L.layer_bwd_i(cfg, params, st, dy, nm)
+        res.append((y, dx, L.layer_bwd_w(cfg, st, wst, nm)["Wqkv"].astype(np.float32)))
+    fracs = []
+    for a, b in zip(*res):
+        n_bad, n, worst = parity.violations(a, b, 2e-2)
+        fracs.append(n_bad / n)
+        assert worst <= parity.MAX_EXCESS
+    assert fracs[0] <= 1e-5 and 5e-5 <= fracs[1] <= 1e-3 and 3e-4 <= fracs[2] <= 4e-3, fracs
