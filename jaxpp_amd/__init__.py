@@ -5,7 +5,7 @@
 reference's names (see jaxpp_amd/api.py)."""
 __version__ = "0.1.0"
 
-_API = ("nn", "collect_task_times_ms", "mpmd_jit_with_loop", "order_tasks", "validate_schedule",
+_API = ("nn", "optim", "take", "collect_task_times_ms", "mpmd_jit_with_loop", "order_tasks", "validate_schedule",
         "value_and_grad", "DeviceMesh", "MpmdMesh", "mark_stage_end", "pipeline_enter_stage",
         "BaseSchedule", "DualPipeV", "Eager1F1B", "Interleaved1F1B", "KimiK2", "Std1F1B",
         "ZeroBubble", "Add", "Concat", "Max", "treduce", "treduce_i")

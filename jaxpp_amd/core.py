@@ -25,7 +25,6 @@ import numpy as np
 
 from jaxpp_amd import tracing
 from jaxpp_amd.mesh import MpmdMesh
-from jaxpp_amd.plan import make_rank_plan
 from jaxpp_amd.schedules import (BaseSchedule, FusedTask, Task, mk_task_name,
                                  preprocess_schedule_tasks)
 from jaxpp_amd.types import TaskType
@@ -65,6 +64,12 @@ def value_and_grad(fun: Callable, has_aux: bool = False) -> Callable:
         if tracing.current() is None:
             raise RuntimeError("value_and_grad(...) evaluates inside jaxpp_amd.treduce")
         out = fun(params, *args)
+        value = out[0] if has_aux else out
+        if not (isinstance(value, tracing.Traced) and value.shape == () and
+                value.producer[0] == "mse"):
+            raise TypeError("value_and_grad differentiates a scalar loss (the first element of "
+                            "the function's result with has_aux)")
+        tracing.current().differentiated = value
         grads = tracing.tree_map(lambda a: tracing.GradOf(id(a), tuple(np.shape(a))), params)
         return out, grads
 
@@ -77,22 +82,51 @@ def value_and_grad(fun: Callable, has_aux: bool = False) -> Callable:
 @dataclass
 class StagedBody:
     stage_layers: list          # per stage: [(spec, params dict), ...]
-    loss_scale: float | None    # scale of the mse loss of the last stage, if any
+    has_loss: bool              # the last stage ends in an mse loss
     leaf_owner: dict            # id(param array) -> (stage, layer index, name)
+    input_index: int            # which microbatched input feeds the first layer
+    target: tuple | None        # ("input", k) | ("const", array): what the loss compares with
+    final_uid: int = 0          # the value the last stage hands out (the prediction)
 
 
 def cluster_ops(tr: tracing.Trace, target_num_stages: int) -> StagedBody:
-    stages, cur, has_mse = [], [], False
+    """Cuts the traced body at its markers (reference: ``cluster_by_yield_eqns`` /
+    ``clusters_to_tasks``, src/jaxpp/core.py:958-1118: a task is whatever lies between two
+    markers).  The body must be one chain: a microbatched input through layers and markers to
+    the prediction the loss reads."""
+    stages, cur, mse = [], [], None
+    producer_of = {sym.uid: ("input", k) for k, (_, sym) in enumerate(tr.inputs)}
+    head = None                    # uid of the value the chain has reached
+    input_index = None
     for op in tr.ops:
         if op[0] == "layer":
-            if has_mse:
+            if mse is not None:
                 raise AssertionError("layers after the loss are not part of any stage")
-            cur.append((op[1], op[2]))
+            _, spec, params, in_uid, out_uid = op
+            if head is None:
+                src = producer_of.get(in_uid)
+                if src is None:
+                    raise NotImplementedError("the first layer must read a microbatched input "
+                                              "of the loop")
+                input_index = src[1]
+            elif in_uid != head:
+                raise NotImplementedError("the loop body must be a single chain of layers: a "
+                                          "layer reads the value the previous layer or marker "
+                                          "produced")
+            head = out_uid
+            cur.append((spec, params))
         elif op[0] == "yield":
+            ins, outs = op[3], op[4]
+            if head is None or head not in ins:
+                raise NotImplementedError("mark_stage_end must be applied to the value the "
+                                          "chain of layers has reached")
+            head = outs[ins.index(head)]
             stages.append(cur)
             cur = []
         elif op[0] == "mse":
-            has_mse = True
+            if mse is not None:
+                raise NotImplementedError("one loss per loop body")
+            mse = op
     if cur and stages:            # trailing layers join the last stage, like trailing eqns
         stages[-1] = stages[-1] + cur
     found = len(stages)
@@ -100,13 +134,24 @@ def cluster_ops(tr: tracing.Trace, target_num_stages: int) -> StagedBody:
         raise AssertionError(f"Unexpected number of pipeline markers: found {found} "
                              f"expected {target_num_stages}.\n")
     owner = {}
-    for s, layers in enumerate(stages):
+    for s_, layers in enumerate(stages):
         if not layers:
-            raise AssertionError(f"Empty stage {(s, TaskType.FWD)}")
+            raise AssertionError(f"Empty stage {(s_, TaskType.FWD)}")
         for li, (_, params) in enumerate(layers):
             for name, arr in params.items():
-                owner[id(arr)] = (s, li, name)
-    return StagedBody(stages, 1.0 if has_mse else None, owner)
+                owner[id(arr)] = (s_, li, name)
+    target = None
+    if mse is not None:
+        _, pred_uid, target = mse
+        # trailing layers (after the last marker) move `head` past the marker's output
+        if pred_uid != head:
+            raise NotImplementedError("the loss must read the output of the last layer of the "
+                                      "last stage")
+    shapes = {(sp.tokens, sp.hidden, sp.dtype) for layers in stages for sp, _ in layers}
+    if len(shapes) != 1:
+        raise NotImplementedError("every layer of the body must keep the activation's shape "
+                                  f"(tokens, hidden) and element type; found {sorted(shapes)}")
+    return StagedBody(stages, mse is not None, owner, input_index, target, head)
 
 
 # ---------------------------------------------------------------------------
@@ -224,7 +269,7 @@ _active_function = None
 class TraceableFunction:
     def __init__(self, fun: Callable, mpmd_mesh: MpmdMesh, options: dict):
         self.fun, self.mpmd_mesh, self.options = fun, mpmd_mesh, options
-        self._executors = {}        # key -> {rank: StageExecutor}
+        self._executors = {}        # key -> {(stage, segment): StageExecutor}
         self.last_order = None      # TimedEntry list of the last loop
         self.__wrapped__ = fun
 
@@ -280,7 +325,45 @@ def mpmd_jit_with_loop(fun: Callable | None = None, mpmd_mesh: MpmdMesh | None =
 # ---------------------------------------------------------------------------
 # running the loop
 # ---------------------------------------------------------------------------
-def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSchedule):
+@dataclass
+class _Segment:
+    """Consecutive layers of one stage that share a layer shape: one stage executor."""
+    spec: Any
+    layers: list                # parameter dicts
+    first: int                  # index of its first layer inside the stage
+    ex: Any = None
+
+
+def _segments(layers: list) -> list:
+    segs = []
+    for li, (spec, params) in enumerate(layers):
+        if segs and segs[-1].spec == spec:
+            segs[-1].layers.append(params)
+        else:
+            segs.append(_Segment(spec, [params], li))
+    return segs
+
+
+def _stage_lifetimes(rows: list, num_stages: int) -> tuple:
+    """Per stage: peak number of forwards whose residuals are still needed, and whether its
+    backward arrives split into BWD_I and BWD_W tasks."""
+    peak, live, split = [0] * num_stages, [0] * num_stages, [False] * num_stages
+    for row in rows:
+        for e in row:
+            for t in (e if isinstance(e, FusedTask) else (e,)):
+                s_, k = t.stage_id, t.fwd_or_bwd
+                if k is TaskType.FWD:
+                    live[s_] += 1
+                    peak[s_] = max(peak[s_], live[s_])
+                elif k is TaskType.BWD or k is TaskType.BWD_W or \
+                        (k is TaskType.BWD_I and s_ == 0 and t.latency > 1):
+                    live[s_] -= 1
+                if k is TaskType.BWD_W:
+                    split[s_] = True
+    return peak, split
+
+
+def run_loop(tr, outputs, ops, n: int, schedule: BaseSchedule):
     from jaxpp_amd import runtime as rt
     fn = _active_function
     if fn is None:
@@ -294,56 +377,93 @@ def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSche
                              f"{mesh.mpmd_dim}")
     order = order_tasks(rows, S)
     fn.last_order = order
-    plans = [make_rank_plan(schedule, n, r) for r in range(len(rows))]
+    peak, split = _stage_lifetimes(rows, S)
 
-    spec = body.stage_layers[0][0][0]
+    # One executor per run of equally shaped layers inside a stage (a task is whatever lies
+    # between two markers: stages may differ in depth and in layer family).
+    stage_segs = [_segments(layers) for layers in body.stage_layers]
+    spec0 = body.stage_layers[0][0][0]
     lib = rt.load()
-    key = (spec, tuple(len(l) for l in body.stage_layers), type(schedule).__name__, S, n)
+    key = (tuple(tuple((sg.spec, len(sg.layers)) for sg in segs) for segs in stage_segs),
+           type(schedule).__name__, S, n, tuple(peak), tuple(split))
     if key not in fn._executors:
         fn.close()
         group = {}
-        for r, plan in enumerate(plans):
-            counts = {len(body.stage_layers[s]) for s in plan.stages}
-            specs = {sp for s in plan.stages for sp, _ in body.stage_layers[s]}
-            if len(counts) != 1 or specs != {spec}:
-                raise NotImplementedError("the stages of one rank must hold the same layers")
-            group[r] = rt.StageExecutor(spec, plan.n_chunks, counts.pop(), plan.max_live,
-                                        plan.split_backward, True)
+        for s_, segs in enumerate(stage_segs):
+            for g, sg in enumerate(segs):
+                group[s_, g] = rt.StageExecutor(sg.spec, 1, len(sg.layers), peak[s_], split[s_], True)
         fn._executors[key] = group
     execs = fn._executors[key]
-    chunk_of = {s: (r, plans[r].stages.index(s)) for r in range(len(plans)) for s in plans[r].stages}
-    for s, layers in enumerate(body.stage_layers):
-        r, c = chunk_of[s]
-        for li, (_, params) in enumerate(layers):
-            execs[r].set_params(c, li, params)
-    for ex in execs.values():
-        ex.zero_grads()
+    for s_, segs in enumerate(stage_segs):
+        for g, sg in enumerate(segs):
+            sg.ex = execs[s_, g]
+            for li, params in enumerate(sg.layers):
+                sg.ex.set_params(0, li, params)
+            sg.ex.zero_grads()
 
-    act_elems = spec.tokens * spec.hidden
-    if x.shape[1:] != (spec.tokens, spec.hidden):
-        x = x.reshape(n, spec.tokens, spec.hidden)
-    f32 = spec.dtype == "f32"           # an f32 model runs through the f32 operators
-    xs_dev = [execs[0].upload_activation(x[m]) for m in range(n)]
+    tokens, hidden = spec0.tokens, spec0.hidden
+    act_elems = tokens * hidden
+    f32 = spec0.dtype == "f32"           # an f32 model runs through the f32 operators
+    any_ex = execs[0, 0]
+
+    def microbatches(x):
+        if x.shape[1:] != (tokens, hidden):
+            if int(np.prod(x.shape[1:])) != act_elems:
+                raise ValueError(f"a microbatch of shape {x.shape[1:]} does not hold "
+                                 f"{tokens} x {hidden} values")
+            x = x.reshape(n, tokens, hidden)
+        return [any_ex.upload_activation(x[m]) for m in range(n)]
+
+    xs_dev = microbatches(tr.inputs[body.input_index][0])
+    tgt_dev = None
+    if body.has_loss:
+        kind, what = body.target
+        if kind == "input":
+            tgt_dev = xs_dev if what == body.input_index else microbatches(tr.inputs[what][0])
+        else:
+            const = any_ex.upload_activation(np.ascontiguousarray(what).reshape(tokens, hidden))
+            tgt_dev = [const] * n
     act, cot = {}, {}                   # (stage, mb) -> DeviceBuffer
     free = []
 
     def take():
-        return free.pop() if free else execs[0].new_activation()
+        return free.pop() if free else any_ex.new_activation()
+
+    def run_fwd(s_, m, src, dst):
+        segs = stage_segs[s_]
+        cur = src
+        for g, sg in enumerate(segs):
+            out = dst if g + 1 == len(segs) else take()
+            sg.ex.run_task(TaskType.FWD, 0, m, cur.ptr, out.ptr)
+            if cur is not src:
+                free.append(cur)        # the executor keeps its own copy of a task's input
+            cur = out
+
+    def run_bwd(s_, m, kind, src, dst):
+        segs = stage_segs[s_]
+        cur = src
+        for g in reversed(range(len(segs))):
+            out = dst if g == 0 else take()
+            segs[g].ex.run_task(kind, 0, m, cur.ptr, out.ptr)
+            if cur is not src:
+                free.append(cur)
+            cur = out
 
     loss_dev = rt.DeviceBuffer(4 * n)
     partial = rt.DeviceBuffer(4 * rt.NORM_PARTIALS)
     want_pred = any(isinstance(v, tracing.Traced) and v.shape != () for v in tracing.tree_leaves(outputs))
     preds = {}
-    loss_scale = None
-    for v in tracing.tree_leaves(outputs):
-        if isinstance(v, tracing.Traced) and v.shape == () and v.producer[0] == "mse":
-            loss_scale = v.producer[1]
+    # the scale of the value that is differentiated sets the cotangent; loss values returned
+    # with another scale are rescaled from it
+    diff = tr.differentiated
+    loss_scales = [v.producer[1] for v in tracing.tree_leaves(outputs)
+                   if isinstance(v, tracing.Traced) and v.shape == () and v.producer[0] == "mse"]
+    loss_scale = diff.producer[1] if diff is not None else (loss_scales[0] if loss_scales else 1.0)
 
     for te in order:
         members = tuple(te.entry) if isinstance(te.entry, FusedTask) else (te.entry,)
         for t in members:
             s, m = t.stage_id, t.mubatch_idx
-            r, c = chunk_of[s]
             kind = t.fwd_or_bwd
             if kind is TaskType.BWD_I and s == 0 and t.latency > 1:
                 kind = TaskType.BWD
@@ -354,33 +474,34 @@ def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSche
             if kind is TaskType.FWD:
                 src = xs_dev[m] if s == 0 else act.pop((s, m))
                 dst = take()
-                execs[r].run_task(kind, c, m, src.ptr, dst.ptr)
+                run_fwd(s, m, src, dst)
                 if s > 0:
                     free.append(src)
                 if s + 1 < S:
                     act[s + 1, m] = dst
                 else:
-                    if body.loss_scale is None:
+                    if not body.has_loss:
                         raise AssertionError("the last stage has no loss to differentiate")
                     d = take()
                     if f32:
-                        rt.check(lib.jpp_mse_loss_f32(None, dst.ptr, xs_dev[m].ptr, act_elems,
+                        rt.check(lib.jpp_mse_loss_f32(None, dst.ptr, tgt_dev[m].ptr, act_elems,
                                                       float(loss_scale), loss_dev.ptr + 4 * m,
                                                       d.ptr))
                     else:
-                        rt.check(lib.jpp_mse_loss(None, dst.ptr, xs_dev[m].ptr, act_elems,
+                        rt.check(lib.jpp_mse_loss(None, dst.ptr, tgt_dev[m].ptr, act_elems,
                                                   float(loss_scale), loss_dev.ptr + 4 * m, d.ptr,
                                                   partial.ptr))
                     cot[s, m] = d
                     if want_pred:
-                        preds[m] = execs[r].download_activation(dst, (spec.tokens, spec.hidden))
+                        preds[m] = any_ex.download_activation(dst, (tokens, hidden))
                     free.append(dst)
             elif kind is TaskType.BWD_W:
-                execs[r].run_task(kind, c, m)
+                for sg in reversed(stage_segs[s]):
+                    sg.ex.run_task(kind, 0, m)
             else:
                 src = cot.pop((s, m))
                 dst = take()
-                execs[r].run_task(kind, c, m, src.ptr, dst.ptr)
+                run_bwd(s, m, kind, src, dst)
                 free.append(src)
                 if s > 0:
                     cot[s - 1, m] = dst
@@ -391,18 +512,31 @@ def run_loop(tr, sym_in, outputs, ops, x: np.ndarray, n: int, schedule: BaseSche
                 _statistics[mk_task_name(s, t.fwd_or_bwd)].append((time.perf_counter() - t0) * 1e3)
     rt.sync()
     losses = loss_dev.download(np.float32, (n,))
-    grads = {s: [execs[chunk_of[s][0]].get_grads(chunk_of[s][1], li)
-                 for li in range(len(body.stage_layers[s]))] for s in range(S)}
+    grads = {}
+    for s_, segs in enumerate(stage_segs):
+        grads[s_] = []
+        for sg in segs:
+            grads[s_] += [sg.ex.get_grads(0, li) for li in range(len(sg.layers))]
 
     def reduce_leaf(v, op):
         if isinstance(v, tracing.GradOf):
             if type(op).__name__ != "AddT":
                 raise NotImplementedError("gradients are reduced with Add")
+            if diff is None:
+                raise AssertionError("gradients need value_and_grad around the loss")
             s, li, name = body.leaf_owner[v.leaf_id]
             return grads[s][li][name].reshape(v.shape)
         if isinstance(v, tracing.Traced):
-            per_mb = ([np.float32(losses[m]) for m in range(n)] if v.shape == ()
-                      else [preds[m].reshape(v.shape) for m in range(n)])
+            if v.shape == ():
+                if v.producer[0] != "mse":
+                    raise NotImplementedError(f"cannot return {v} from the loop body")
+                rescale = np.float32(v.producer[1] / loss_scale)
+                per_mb = [np.float32(losses[m]) * rescale for m in range(n)]
+            else:
+                if v.uid != body.final_uid:
+                    raise NotImplementedError("the only activation the loop can return is the "
+                                              "output of the last stage")
+                per_mb = [preds[m].reshape(v.shape) for m in range(n)]
             state = op.state(n, per_mb[0])
             for m in range(n):
                 state = op.update(state, per_mb[m], m)

@@ -87,8 +87,21 @@ def broadcast_ops(operation, outputs):
     raise TypeError(f"unexpected operation {operation!r}")
 
 
+def take(x, i, axis: int = 0):
+    """``x`` at position ``i`` of ``axis`` - ``jnp.take(x, i, axis)`` of the reference's loop
+    body (training.py:232-235).  With the loop index of ``treduce_i`` it makes ``x`` a
+    microbatched input of the loop and returns its per-microbatch placeholder; with an integer
+    it is ``numpy.take``."""
+    if isinstance(i, tracing.MicrobatchIndex):
+        tr = tracing.current()
+        if tr is None or tr.index is not i:
+            raise RuntimeError("the loop index is only meaningful while its loop body is traced")
+        return tr.add_input(x, axis)
+    return np.take(x, i, axis=axis)
+
+
 def treduce(fun: Callable, xs, schedule: BaseSchedule, axis: int = 0, operation=default_op):
-    """Temporally reduces ``fun`` over the microbatch axis of ``xs``
+    """Temporally reduces ``fun`` over the microbatch axis of ``xs``, a pytree of arrays
     (signature and meaning as the reference's, training.py:172-239)."""
     flat = tracing.tree_leaves(xs)
     n = flat[0].shape[axis]
@@ -96,31 +109,27 @@ def treduce(fun: Callable, xs, schedule: BaseSchedule, axis: int = 0, operation=
         raise AssertionError("Leading dimensions differing among xs")
 
     def wrap(i):
-        return fun(tracing.tree_map(lambda x: np.take(x, i, axis=axis), xs))
+        return fun(tracing.tree_map(lambda x: take(x, i, axis), xs))
 
-    wrap.__wrapped__ = fun
-    wrap._xs, wrap._axis = xs, axis
     return treduce_i(wrap, n, schedule=schedule, operation=operation)
 
 
 def treduce_i(fun: Callable, length: int, schedule: BaseSchedule, operation=default_op):
-    """``treduce`` with an explicit length: ``fun(i)`` is the i-th
-    microbatch's value (reference: training.py:248-340)."""
+    """``treduce`` with an explicit length: ``fun(i)`` is the i-th microbatch's value
+    (reference: training.py:248-340); the body picks its microbatch with ``take(x, i, axis)``.
+    The body is traced once on the symbolic index; every array it indexes must have ``length``
+    entries along the indexed axis."""
     from jaxpp_amd import core
-    xs = getattr(fun, "_xs", None)
-    if xs is None:
-        raise NotImplementedError(
-            "treduce_i needs the microbatched inputs; call it through treduce(fun, xs, ...)")
-    inner = fun.__wrapped__
-    axis = fun._axis
-    flat = tracing.tree_leaves(xs)
-    if len(flat) != 1:
-        raise NotImplementedError("the loop body takes one microbatched array (hidden states)")
-    x = np.asarray(flat[0])
-    x = np.moveaxis(x, axis, 0)
+    if length <= 0:
+        raise ValueError(f"treduce_i: length must be positive, got {length}")
     with tracing.tracing() as tr, yield_scope():
-        sym = tr.fresh(x.shape[1:], ("input",))
-        sym_in = tracing.tree_map(lambda _: sym, xs)
-        outputs = inner(sym_in)
+        outputs = fun(tr.index)
+    if not tr.inputs:
+        raise TypeError("the loop body never indexed an array with the loop index "
+                        "(take(x, i, axis)): there is nothing to iterate over")
+    for x, _ in tr.inputs:
+        if x.shape[0] != length:
+            raise AssertionError(f"an array indexed by the loop has {x.shape[0]} entries along "
+                                 f"the indexed axis, the loop runs {length} times")
     ops = broadcast_ops(operation, outputs)
-    return core.run_loop(tr, sym, outputs, ops, x, length, schedule)
+    return core.run_loop(tr, outputs, ops, length, schedule)

@@ -6,6 +6,8 @@ from functools import partial
 import numpy as np
 import pytest
 
+import parity
+
 import jaxpp_amd as jaxpp
 from jaxpp_amd import runtime as rt
 from jaxpp_amd.model import LayerSpec
@@ -16,9 +18,7 @@ pytestmark = pytest.mark.gpu
 
 
 def close(got, want, what, rtol=2e-2):
-    scale = float(np.abs(want).max()) + 1e-30
-    err = float(np.abs(np.asarray(got, np.float32) - want).max())
-    assert err <= rtol * scale, f"{what}: {err:.4g} vs {scale:.4g}"
+    parity.close_stage(np.asarray(got, np.float32), np.asarray(want), rtol, what)
 
 
 @pytest.mark.parametrize("schedule,n_mb,mpmd", [
@@ -106,4 +106,130 @@ def test_example_model_train_step():
             for k, v in want_acc[s][li].items():
                 got = grad["layers"][s * per + li][k]
                 close(got, v.reshape(got.shape), f"grad {s}/{li}/{k}")
+    train_step.close()
+
+
+def _mesh(pp):
+    return jaxpp.MpmdMesh(jaxpp.DeviceMesh(np.arange(pp).reshape(pp, 1), ("mpmd", "data")), "mpmd")
+
+
+def test_uneven_stages_and_mixed_layer_families():
+    """A task is whatever lies between two markers (reference: clusters_to_tasks,
+    src/jaxpp/core.py:1063-1118).  Three post-LN encoder layers in the first stage and, in the
+    second, one encoder layer followed by a pre-LN decoder block - stages of different depth
+    and a stage whose layers are of two families - with the markers placed by hand as
+    examples/basic.py:125-131 does.  ZeroBubble(2), so the second stage's backward runs split
+    across both of its executors.  Against the sequential loop of the oracle."""
+    rt.require_gpu()
+    bert = LayerSpec("bert", 256, 4, 512, 128, 1, eps=1e-12)
+    dec = LayerSpec("decoder", 256, 4, 512, 128, 1, causal=True, eps=1e-6, gelu_tanh=True)
+    enc, blk = jaxpp.nn.TransformerLayer(bert), jaxpp.nn.TransformerLayer(dec)
+    n_mb, schedule = 4, jaxpp.ZeroBubble(2)
+    rnd = lambda p: {k: L.bf16_round(v) for k, v in p.items()}
+    params = [rnd(enc.init(0, i, perturb=True)) for i in range(4)] + [rnd(blk.init(0, 4, perturb=True))]
+    layers = [enc, enc, enc, enc, blk]
+    batch = L.bf16_round(np.random.default_rng(3).standard_normal(
+        (n_mb, bert.tokens, bert.hidden)).astype(np.float32))
+
+    def loss_fn(pars, mb):
+        h = mb
+        for i, (layer, p) in enumerate(zip(layers, pars)):
+            if i == 3:
+                h = jaxpp.mark_stage_end(h)
+            h = layer.apply(p, h)
+        h = jaxpp.mark_stage_end(h)
+        return jaxpp.nn.mse_loss(h, mb) / n_mb
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=_mesh(2))
+    def train_step(pars, batch):
+        return jaxpp.treduce(partial(jaxpp.value_and_grad(loss_fn), pars), batch, schedule=schedule)
+
+    losses, grad = train_step(params, batch)
+    cfgs = {0: [L.LayerCfg(**bert.as_dict())] * 3,
+            1: [L.LayerCfg(**bert.as_dict()), L.LayerCfg(**dec.as_dict())]}
+    want_loss, want_acc = O.treduce_sequential(cfgs[0][0], [params[:3], params[3:]], list(batch),
+                                               L.Numerics.bf16(), layer_cfgs=cfgs)
+    close(losses, want_loss, "losses")
+    for i in range(5):
+        s, li = (0, i) if i < 3 else (1, i - 3)
+        for k, v in want_acc[s][li].items():
+            close(grad[i][k], v.reshape(grad[i][k].shape), f"grad layer {i}/{k}")
+    train_step.close()
+
+
+@pytest.mark.parametrize("target_kind", ["second-input", "constant"])
+def test_loss_against_a_target_that_is_not_the_input(target_kind):
+    """Two microbatched arrays in `xs` (hidden states and targets), or a constant target held by
+    the closure: the loss and its cotangent must come from that target, and a loss value
+    returned with another scale than the differentiated one must be reported with its own."""
+    rt.require_gpu()
+    spec = LayerSpec("bert", 256, 4, 512, 128, 1, eps=1e-12)
+    n_mb, pp = 4, 2
+    model = jaxpp.nn.TransformerStack(spec, n_layers=2, layers_per_stage=1)
+    params = model.init(seed=0, perturb=True)
+    params = {"layers": [{k: L.bf16_round(v) for k, v in p.items()} for p in params["layers"]]}
+    rng = np.random.default_rng(5)
+    batch = L.bf16_round(rng.standard_normal((n_mb, spec.tokens, spec.hidden)).astype(np.float32))
+    if target_kind == "second-input":
+        targets = L.bf16_round(rng.standard_normal(batch.shape).astype(np.float32))
+        xs = {"hidden": batch, "target": targets}
+    else:
+        const = L.bf16_round(rng.standard_normal(batch.shape[1:]).astype(np.float32))
+        targets = np.stack([const] * n_mb)
+        xs = {"hidden": batch}
+
+    def loss_fn(pars, mb):
+        res = model.apply(pars, mb["hidden"])
+        raw = jaxpp.nn.mse_loss(res, mb["target"] if target_kind == "second-input" else const)
+        return raw / n_mb, raw
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=_mesh(pp))
+    def train_step(pars, xs):
+        fun = partial(jaxpp.value_and_grad(loss_fn, has_aux=True), pars)
+        (losses, raw), grad = jaxpp.treduce(fun, xs, schedule=jaxpp.Std1F1B(pp),
+                                            operation=((jaxpp.Concat(), jaxpp.Concat()), jaxpp.Add))
+        return losses, raw, grad
+
+    losses, raw, grad = train_step(params, xs)
+    cfg = L.LayerCfg(**spec.as_dict())
+    stages = [[p] for p in params["layers"]]
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16(),
+                                               targets=list(targets))
+    close(losses, want_loss, "losses")
+    close(raw, want_loss * n_mb, "unscaled losses")
+    # the loss really is against the target: against the input it would be far off
+    assert abs(float(losses[0]) - float(L.mse_loss(batch[0], batch[0], n_mb)[0])) > 0.1 * float(want_loss[0])
+    for s in range(pp):
+        for k, v in want_acc[s][0].items():
+            close(grad["layers"][s][k], v.reshape(grad["layers"][s][k].shape), f"grad {s}/{k}")
+    train_step.close()
+
+
+def test_treduce_i_with_an_explicit_length():
+    """treduce_i(fun, length): the body picks its microbatch with take(x, i, axis) - here along
+    axis 1 of an array laid out [tokens, microbatch, hidden] (reference: training.py:248-340)."""
+    rt.require_gpu()
+    spec = LayerSpec("bert", 256, 4, 512, 128, 1, eps=1e-12)
+    n_mb = 2
+    layer = jaxpp.nn.TransformerLayer(spec)
+    p = {k: L.bf16_round(v) for k, v in layer.init(0, 0, perturb=True).items()}
+    batch = L.bf16_round(np.random.default_rng(7).standard_normal(
+        (n_mb, spec.tokens, spec.hidden)).astype(np.float32))
+    laid_out = np.ascontiguousarray(batch.transpose(1, 0, 2))      # [tokens, microbatch, hidden]
+
+    def body(pars, i):
+        mb = jaxpp.take(laid_out, i, axis=1)
+        return jaxpp.nn.mse_loss(jaxpp.mark_stage_end(layer.apply(pars, mb)), mb) / n_mb
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=_mesh(1))
+    def train_step(pars):
+        return jaxpp.treduce_i(partial(jaxpp.value_and_grad(body), pars), n_mb,
+                               schedule=jaxpp.Std1F1B(1))
+
+    losses, grad = train_step(p)
+    want_loss, want_acc = O.treduce_sequential(L.LayerCfg(**spec.as_dict()), [[p]], list(batch),
+                                               L.Numerics.bf16())
+    close(losses, want_loss, "losses")
+    for k, v in want_acc[0][0].items():
+        close(grad[k], v.reshape(grad[k].shape), f"grad {k}")
     train_step.close()

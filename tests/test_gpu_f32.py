@@ -8,6 +8,8 @@ import math
 import numpy as np
 import pytest
 
+import parity
+
 from jaxpp_amd import runtime as rt
 from oracle import layers as L
 
@@ -19,11 +21,7 @@ def _gpu():
     rt.require_gpu()
 
 
-def close(got, want, rtol, what):
-    scale = float(np.abs(want).max()) + 1e-30
-    err = float(np.abs(got.astype(np.float64) - want).max())
-    assert np.isfinite(got).all(), f"{what}: non-finite"
-    assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+close = parity.close
 
 
 def dev(a):
@@ -388,6 +386,61 @@ def test_cfg1_train_step_through_the_public_api():
                 got = grad["layers"][s * per + li][k]
                 close(got, v.reshape(got.shape).astype(np.float64), 1e-4, f"grad {s}/{li}/{k}")
     train_step.close()
+
+
+def test_cfg1_two_train_steps_with_adam_through_the_public_api():
+    """cfg1 with its optimizer: the train step of the reference's README (README.md:83-93) -
+    treduce, then `optimizer.update` and `apply_updates` - returning the updated parameters,
+    twice in a row with Adam lr 1e-3, against the oracle's sequential loop and Adam at 1e-4."""
+    from functools import partial
+
+    import jaxpp_amd as jaxpp
+    from oracle import stage as O
+
+    n_mb, pp, n_layers = 8, 2, 4
+    model = jaxpp.nn.TransformerStack(CFG1, n_layers=n_layers, layers_per_stage=n_layers // pp)
+    params = model.init(seed=0, perturb=True)
+    rng = np.random.default_rng(1)
+    mesh = jaxpp.MpmdMesh(jaxpp.DeviceMesh(np.arange(pp).reshape(pp, 1), ("mpmd", "data")), "mpmd")
+    schedule = jaxpp.Std1F1B(pp)
+    optimizer = jaxpp.optim.adam(1e-3)
+
+    def loss_fn(pars, mb):
+        res = model.apply(pars, mb)
+        return jaxpp.nn.mse_loss(res, mb) / n_mb, (res, 4)
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=mesh)
+    def pp_train_step(opt_state, pars, batch):
+        mubatch_grad = partial(jaxpp.value_and_grad(loss_fn, has_aux=True), pars)
+        (losses, (preds, _)), grad = jaxpp.treduce(mubatch_grad, batch, schedule=schedule)
+        updates, opt_state = optimizer.update(grad, opt_state, pars)
+        new_pars = jaxpp.optim.apply_updates(pars, updates)
+        return opt_state, new_pars, losses, preds
+
+    cfg = L.LayerCfg(**CFG1.as_dict())
+    per = n_layers // pp
+    want_p = [dict(p) for p in params["layers"]]
+    want_m = [{k: np.zeros_like(v) for k, v in p.items()} for p in want_p]
+    want_v = [{k: np.zeros_like(v) for k, v in p.items()} for p in want_p]
+    opt_state = optimizer.init(params)
+    for step in (1, 2):
+        batch = rng.standard_normal((n_mb, CFG1.tokens, CFG1.hidden), dtype=np.float32)
+        opt_state, params, losses, _ = pp_train_step(opt_state, params, batch)
+        stages = [want_p[s * per:(s + 1) * per] for s in range(pp)]
+        want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.f32())
+        close(losses, want_loss.astype(np.float64), 1e-4, f"step {step} losses")
+        for i in range(n_layers):
+            g = {k: v.reshape(want_p[i][k].shape) for k, v in want_acc[i // per][i % per].items()}
+            want_p[i] = O.adam_step(want_p[i], g, want_m[i], want_v[i], step, lr=1e-3)
+            for k in want_p[i]:
+                close(params["layers"][i][k], want_p[i][k].astype(np.float64), 1e-4,
+                      f"step {step} layer {i} {k}")
+                close(opt_state["mu"]["layers"][i][k], want_m[i][k].astype(np.float64), 1e-4,
+                      f"step {step} layer {i} m[{k}]")
+                close(opt_state["nu"]["layers"][i][k], want_v[i][k].astype(np.float64), 1e-4,
+                      f"step {step} layer {i} v[{k}]")
+        assert opt_state["count"] == step
+    pp_train_step.close()
 
 
 def test_f32_stage_adam_after_loop():

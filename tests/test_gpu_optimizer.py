@@ -8,6 +8,8 @@ kernel's own f32 weights."""
 import numpy as np
 import pytest
 
+import parity
+
 from jaxpp_amd import runtime as rt
 from jaxpp_amd import schedules as S
 from jaxpp_amd.model import LayerSpec, boundary_tensor, init_layer_params
@@ -25,11 +27,7 @@ def _gpu():
     rt.require_gpu()
 
 
-def close(got, want, tol, what):
-    scale = float(np.abs(want).max()) + 1e-30
-    err = float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max())
-    assert np.isfinite(got).all(), f"{what}: non-finite"
-    assert err <= tol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+close = parity.close
 
 
 @pytest.mark.parametrize("count", [8 * 256 * 33, 8 * 1000 + 5, 3])
@@ -153,4 +151,51 @@ def test_stage_adam_needs_init():
     ex = rt.StageExecutor(BERT, plan.n_chunks, 1, plan.max_live, plan.split_backward, True, False)
     with pytest.raises(rt.JppError, match="optimizer_init has not run"):
         ex.adam_step(1)
+    ex.close()
+
+
+def test_bf16_parameters_are_written_once_per_step_by_the_adam_pass():
+    """The reference hoists the cast of the f32 weights to bf16 out of the microbatch loop
+    (loop-invariant code motion, src/jaxpp/licm.py:531-644; PERF_GUIDE.md:29-41): the loop
+    reads a bf16 copy made once per step.  Here that copy is the stage's parameter storage:
+    no task of the loop writes it (its bits are the same after every task of the row), the
+    only launches of a step that touch it are the loop's reads and one Adam launch, and after
+    that launch it is exactly the rounded f32 weights."""
+    spec, schedule, n_mb, rank, lpc = LLAMA, S.Interleaved1F1B(4, 2), 4, 0, 1
+    plan = make_rank_plan(schedule, n_mb, rank)
+    shape = (spec.tokens, spec.hidden)
+    ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True, False)
+    for c, stage in enumerate(plan.stages):
+        ex.set_params(c, 0, {k: L.bf16_round(v) for k, v in
+                             init_layer_params(spec, 3, stage, perturb=True).items()})
+    ex.optimizer_init()
+    lib = rt.load()
+
+    def param_bits():
+        out = []
+        for c in range(plan.n_chunks):
+            for name, rows, cols in ex.params:
+                ptr = ex._ptr(lib.jpp_stage_param_ptr, c, 0, name)
+                out.append(rt.download_ptr(ptr, np.uint16, (rows * cols,)))
+        return np.concatenate(out)
+
+    x = rt.DeviceBuffer.from_f32_as_bf16(boundary_tensor("x", 0, 0, shape, 0))
+    out = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+    for step in (1, 2):
+        before = param_bits()
+        with rt.probe("adam") as pr:
+            for pt in plan.tasks:
+                ex.run_task(pt.exec_kind, pt.chunk, pt.task.mubatch_idx, x.ptr, out.ptr)
+                rt.sync()
+                np.testing.assert_array_equal(param_bits(), before,
+                                              err_msg=f"step {step}: {pt.task} wrote the parameters")
+            ex.adam_step(step, lr=1e-2, grad_scale=1.0 / n_mb)
+            rt.sync()
+        assert pr.launches == 1, "one Adam launch per step rewrites the bf16 copy"
+        after = param_bits()
+        assert (after != before).any(), "the Adam pass must rewrite the bf16 parameters"
+        for c in range(plan.n_chunks):
+            state, new_p = ex.get_opt_state(c, 0), ex.get_params(c, 0)
+            for k, (w, _, _) in state.items():
+                assert np.array_equal(new_p[k].reshape(w.shape), L.bf16_round(w)), k
     ex.close()

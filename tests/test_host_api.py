@@ -164,3 +164,126 @@ def test_rank_plans_for_the_benchmark_configs(sched, n, rank, stages, live, spli
     assert len(fw) == n * len(stages)
     if rank == 0:       # the first stage's backward is never split
         assert all(p.exec_kind is not TaskType.BWD_W for p in plan.tasks if p.task.stage_id == 0)
+
+
+# ---------------------------------------------------------------------------
+# tracing the loop body: what a stage may contain, and what the loss may read
+# ---------------------------------------------------------------------------
+def _trace(body):
+    from jaxpp_amd.pipelining import yield_scope
+    with tracing.tracing() as tr, yield_scope():
+        out = body(tr.index)
+    return tr, out
+
+
+def test_a_stage_is_whatever_lies_between_two_markers():
+    """Stages of different depth and of different layer families (reference:
+    clusters_to_tasks, src/jaxpp/core.py:1063-1118); examples/basic.py:125-131 places its
+    markers in front of layer i for i % n == 0, which splits 4 layers 3 + 1."""
+    dec = LayerSpec("decoder", 128, 2, 256, 128, 1, causal=True)
+    bert, block = jaxpp.nn.TransformerLayer(SPEC), jaxpp.nn.TransformerLayer(dec)
+    x = np.zeros((4, 128, 128), np.float32)
+    params = [bert.init(0, i) for i in range(3)] + [block.init(0, 3)]
+
+    def body(i):
+        h = jaxpp.take(x, i, 0)
+        for li, p in enumerate(params):
+            if li == 3:
+                h = jaxpp.mark_stage_end(h)
+            h = (bert if li < 3 else block).apply(p, h)
+        h = jaxpp.mark_stage_end(h)
+        return jaxpp.nn.mse_loss(h, jaxpp.take(x, i, 0)) / 4
+
+    tr, _ = _trace(body)
+    staged = core.cluster_ops(tr, 2)
+    assert [len(s) for s in staged.stage_layers] == [3, 1]
+    assert [sp.family for sp, _ in staged.stage_layers[0]] == ["bert"] * 3
+    assert staged.stage_layers[1][0][0].family == "decoder"
+    assert staged.input_index == 0 and staged.target == ("input", 0) and staged.has_loss
+    assert len(tr.inputs) == 1                    # the same array taken twice is one input
+    segs = core._segments(staged.stage_layers[0] + staged.stage_layers[1])
+    assert [(sg.spec.family, len(sg.layers), sg.first) for sg in segs] == [("bert", 3, 0), ("decoder", 1, 3)]
+    with pytest.raises(AssertionError, match="found 2 expected 3"):
+        core.cluster_ops(tr, 3)
+
+
+def test_loss_target_must_be_an_input_or_a_constant():
+    layer = jaxpp.nn.TransformerLayer(SPEC)
+    p = layer.init()
+    x, y = np.zeros((2, 128, 128), np.float32), np.ones((2, 128, 128), np.float32)
+
+    def second_input(i):
+        h = jaxpp.mark_stage_end(layer.apply(p, jaxpp.take(x, i)))
+        return jaxpp.nn.mse_loss(h, jaxpp.take(y, i))
+    tr, _ = _trace(second_input)
+    staged = core.cluster_ops(tr, 1)
+    assert staged.input_index == 0 and staged.target == ("input", 1) and len(tr.inputs) == 2
+
+    const = np.full((128, 128), 0.5, np.float32)
+    tr, _ = _trace(lambda i: jaxpp.nn.mse_loss(jaxpp.mark_stage_end(layer.apply(p, jaxpp.take(x, i))), const))
+    kind, arr = core.cluster_ops(tr, 1).target
+    assert kind == "const" and arr is not None and arr.shape == (128, 128)
+
+    def computed_target(i):
+        h = layer.apply(p, jaxpp.take(x, i))
+        return jaxpp.nn.mse_loss(jaxpp.mark_stage_end(h), h)
+    with pytest.raises(NotImplementedError, match="microbatched input of the loop or a constant"):
+        _trace(computed_target)
+    with pytest.raises(ValueError, match="target of shape"):
+        _trace(lambda i: jaxpp.nn.mse_loss(layer.apply(p, jaxpp.take(x, i)), np.zeros((3, 3))))
+
+    def loss_on_an_earlier_value(i):
+        h0 = layer.apply(p, jaxpp.take(x, i))
+        jaxpp.mark_stage_end(layer.apply(p, h0))
+        return jaxpp.nn.mse_loss(h0, jaxpp.take(x, i))
+    tr, _ = _trace(loss_on_an_earlier_value)
+    with pytest.raises(NotImplementedError, match="output of the last layer of the last stage"):
+        core.cluster_ops(tr, 1)
+
+    def not_a_chain(i):
+        a = layer.apply(p, jaxpp.take(x, i))
+        b = layer.apply(p, jaxpp.take(x, i))          # reads the input again, not `a`
+        return jaxpp.nn.mse_loss(jaxpp.mark_stage_end(b), jaxpp.take(x, i))
+    tr, _ = _trace(not_a_chain)
+    with pytest.raises(NotImplementedError, match="single chain"):
+        core.cluster_ops(tr, 1)
+
+
+def test_value_and_grad_remembers_what_it_differentiates():
+    layer = jaxpp.nn.TransformerLayer(SPEC)
+    p = layer.init()
+    x = np.zeros((2, 128, 128), np.float32)
+
+    def loss_fn(pars, mb):
+        res = jaxpp.mark_stage_end(layer.apply(pars, mb))
+        raw = jaxpp.nn.mse_loss(res, mb)
+        return raw / 2, (raw, res)            # differentiated: raw / 2; returned too: raw
+
+    tr, out = _trace(lambda i: jaxpp.value_and_grad(loss_fn, has_aux=True)(p, jaxpp.take(x, i)))
+    (scaled, (raw, _)), grads = out
+    assert tr.differentiated is scaled and scaled.producer == ("mse", 0.5) and raw.producer == ("mse", 1.0)
+    assert set(grads) == set(p) and all(isinstance(g, tracing.GradOf) for g in grads.values())
+    with pytest.raises(TypeError, match="differentiates a scalar loss"):
+        _trace(lambda i: jaxpp.value_and_grad(lambda pars, mb: layer.apply(pars, mb))(p, jaxpp.take(x, i)))
+
+
+def test_treduce_i_takes_the_loop_index():
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    np.testing.assert_array_equal(jaxpp.take(x, 1, axis=1), x[:, 1])
+    with pytest.raises(ValueError, match="length must be positive"):
+        jaxpp.treduce_i(lambda i: i, 0, S.Std1F1B(1))
+    with pytest.raises(TypeError, match="never indexed an array"):
+        jaxpp.treduce_i(lambda i: 0, 2, S.Std1F1B(1))
+    with pytest.raises(AssertionError, match="has 2 entries along the indexed axis, the loop runs 3"):
+        jaxpp.treduce_i(lambda i: jaxpp.take(x, i), 3, S.Std1F1B(1))
+    with pytest.raises(RuntimeError, match="only meaningful while its loop body is traced"):
+        jaxpp.take(x, tracing.MicrobatchIndex())
+
+
+def test_stage_lifetimes_per_stage():
+    rows = S.preprocess_schedule_tasks(S.ZeroBubble(2).tasks(4), 0, False)
+    peak, split = core._stage_lifetimes(rows, 2)
+    assert split == [False, True] and peak == [2, 2]
+    rows = S.preprocess_schedule_tasks(S.Interleaved1F1B(4, 2).tasks(4), 0, False)
+    peak, split = core._stage_lifetimes(rows, 4)
+    assert split == [False] * 4 and all(1 <= p <= 4 for p in peak)
