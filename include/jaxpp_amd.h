@@ -206,6 +206,18 @@ typedef struct {
 
 int jpp_norm_fwd(void* stream, const jpp_norm_args* args);
 int jpp_norm_bwd(void* stream, const jpp_norm_args* args);
+/* No counterpart in the reference.  jpp_norm_bwd for callers that cannot allocate device
+ * memory and have no workspace to pass (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): `args->partial` is ignored and the partial sums go to a
+ * buffer the library holds itself in static device memory (16 MiB per GPU, for the whole
+ * life of the process).  Same kernels, same summation order and bit-identical results as
+ * jpp_norm_bwd; cols <= 8192 (more is JPP_ERR_INVALID).  It calls no allocating routine
+ * (while a launch probe is active the probe's events are created as for any entry point).
+ * The first call on a device looks the buffer's address up (hipGetSymbolAddress): make that
+ * call outside a graph capture.  All calls on one GPU share the buffer, so two calls that
+ * overlap on one GPU (different streams, or two host threads) race; calls on one stream do
+ * not. */
+int jpp_norm_bwd_static(void* stream, const jpp_norm_args* args);
 
 /* ---- elementwise ------------------------------------------------------------ */
 /* s[t,j] = silu(gate[t,j]) * up[t,j]; backward writes dgu [T,2f] in gu's layout.

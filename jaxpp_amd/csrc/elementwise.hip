@@ -6,11 +6,43 @@
 // scheduling.
 #include <math.h>
 
+#include <mutex>
+
 #include "common.h"
+
+// Scratch of jpp_norm_bwd_static (the entry point that allocates nothing): the per-block
+// partial sums of the scale / shift gradients, 2 x JPP_NORM_PARTIALS rows of at most
+// kStaticNormCols columns (16 MiB).  Every GPU the library runs on holds its own copy at its
+// own address until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address comes from static_scratch() below and is what
+// kernels are given.
+constexpr int kStaticNormCols = 8192;
+static __device__ __align__(256) float scratch[2 * JPP_NORM_PARTIALS * kStaticNormCols];
 
 namespace {
 
 constexpr int kMaxChunksPerLane = 16;  // a wave holds one row of <= 8192 columns
+static_assert(kStaticNormCols == 8 * 64 * kMaxChunksPerLane, "scratch sized for the widest row");
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(float** out) {
+  int dev = -1;
+  JPP_CHECK_HIP(hipGetDevice(&dev));
+  JPP_REQUIRE(dev >= 0 && dev < kMaxDevices, "static scratch: device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    JPP_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    JPP_REQUIRE(ptr, "static scratch: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = (float*)ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return JPP_OK;
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -678,6 +710,21 @@ int jpp_norm_bwd(void* stream, const jpp_norm_args* a) {
   ProbeScope probe((hipStream_t)stream, "norm_bwd", 0, (a->resid ? 8.0 : 6.0) * a->rows * a->cols);
   return ln ? launch_norm_bwd<true>((hipStream_t)stream, a)
             : launch_norm_bwd<false>((hipStream_t)stream, a);
+}
+
+int jpp_norm_bwd_static(void* stream, const jpp_norm_args* a) {
+  JPP_REQUIRE(a, "norm_bwd_static: null operand");
+  JPP_REQUIRE(a->cols > 0 && a->cols <= kStaticNormCols,
+              "norm_bwd_static: %ld columns exceed the %d the library's own scratch holds",
+              (long)a->cols, kStaticNormCols);
+  float* ptr = nullptr;
+  if (int rc = static_scratch(&ptr)) return rc;
+  // The kernels write rows 0 .. JPP_NORM_PARTIALS-1 (and, for LayerNorm, the same number of
+  // rows behind them) of `cols` columns before the reduction reads exactly those, so nothing
+  // of an earlier call is read and nothing needs clearing.
+  jpp_norm_args b = *a;
+  b.partial = ptr;
+  return jpp_norm_bwd(stream, &b);
 }
 
 int jpp_swiglu_fwd(void* stream, const void* gu, void* s, int64_t rows, int64_t f,

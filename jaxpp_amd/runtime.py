@@ -106,7 +106,7 @@ EXPORTS = [
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_gemm_f32", "jpp_attn_fwd_f32", "jpp_attn_bwd_f32", "jpp_norm_fwd_f32", "jpp_norm_bwd_f32",
     "jpp_colsum_accum_f32", "jpp_mse_loss_f32", "jpp_rope_f32",
-    "jpp_norm_fwd", "jpp_norm_bwd", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
+    "jpp_norm_fwd", "jpp_norm_bwd", "jpp_norm_bwd_static", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
     "jpp_grad_accum_f32", "jpp_sum_accum_f32", "jpp_colsum_accum", "jpp_colsum_accum_multi", "jpp_mse_loss", "jpp_moe_capacity", "jpp_moe_route",
     "jpp_moe_gather", "jpp_moe_combine_fwd", "jpp_moe_bwd_prepare", "jpp_moe_combine_bwd",
     "jpp_moe_router_wgrad", "jpp_cast_f32_to_bf16", "jpp_cast_bf16_to_f32", "jpp_adam_step",
@@ -164,6 +164,7 @@ def load():
     lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_norm_fwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
     lib.jpp_norm_bwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
+    lib.jpp_norm_bwd_static.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
     lib.jpp_gemm_f32.argtypes = [C.c_void_p, C.POINTER(GemmArgs)]
     lib.jpp_attn_fwd_f32.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_attn_bwd_f32.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
