@@ -41,14 +41,14 @@ def synthetic_pool(n_elems: int, std: float, seed: int) -> np.ndarray:
 class Workbench:
     """Device state of one workload: executor, parameters, boundary tensors."""
 
-    def __init__(self, wl, fused=True, two_streams=False):
+    def __init__(self, wl, fused=True, two_streams=False, wgrad_group=0):
         self.wl = wl
         spec = wl.layer
         sched = getattr(S, wl.schedule)(**wl.schedule_kwargs)
         self.plan = make_rank_plan(sched, wl.n_mubatches, wl.rank)
         self.ex = rt.StageExecutor(spec, self.plan.n_chunks, wl.layers_per_stage,
                                    self.plan.max_live, self.plan.split_backward, fused,
-                                   two_streams)
+                                   two_streams, wgrad_group)
         lib = rt.load()
         # parameters: slices of one N(0, 0.02^2) pool at per-tensor offsets;
         # norm gains one, biases zero
@@ -123,6 +123,18 @@ def dominant_gemm_class(wl) -> str:
     return "gemm_tn_accf32_256x256w8" if big else "gemm_tn_accf32_128x128w8s3"
 
 
+def default_wgrad_group(wl, two_streams: bool) -> int:
+    """How many consecutive microbatches share one weight-gradient product per weight (the
+    fp32 accumulator is then read and written once per group).  Measured on MI355X, A/B on one
+    box: Llama-8B-shaped stage 1397-1402 ms/step ungrouped, 1393-1395 in pairs, 1373-1379 in
+    fours (73 GB); 70B-shaped 4579-4584 / 4545-4552 / 4543-4554 ms (197 / 215 / 251 GB), so
+    pairs there.  The expert layers' grouped products cannot be merged across microbatches
+    (their row groups differ) and narrow layers run two streams: ungrouped."""
+    if two_streams or wl.layer.family != "llama" or wl.layer.hidden < 4096:
+        return 1
+    return 4 if wl.layer.hidden < 8192 else 2
+
+
 def cpu_baseline(wl, budget_layers: int = 1):
     """The numpy oracle on the host cores: one microbatch through
     `budget_layers` layer(s), forward + backward-input + backward-weight +
@@ -175,6 +187,9 @@ def main():
                          "narrow for one kernel to fill the chip (hidden < 2048: +7%% at cfg2), off "
                          "otherwise (-1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
                          "include the other stream's kernels)")
+    ap.add_argument("--wgrad-group", type=int, default=None,
+                    help="weight gradients of this many consecutive microbatches as one product "
+                         "per weight (1: per microbatch; default: see default_wgrad_group)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
     ap.add_argument("--graph", action="store_true",
                     help="record the step into a HIP graph after the warm-up and time replays "
@@ -208,7 +223,10 @@ def main():
         import dataclasses
         wl = dataclasses.replace(wl, n_mubatches=args.n_mubatches)
     two = wl.layer.hidden < 2048 if args.two_streams == "auto" else args.two_streams == "on"
-    wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two)
+    group = args.wgrad_group if args.wgrad_group is not None else default_wgrad_group(wl, two)
+    if args.unfused_accumulate or two:
+        group = 1
+    wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two, wgrad_group=group)
     cls = args.probe or dominant_gemm_class(wl)
 
     # The host enqueues a step in a fraction of the time the GPU takes to run it.  It is kept at
@@ -275,7 +293,7 @@ def main():
             "layers": wl.layers_per_stage * wb.plan.n_chunks,
             "peak_live_microbatches": wb.plan.max_live,
             "fused_wgrad_accumulate": not args.unfused_accumulate,
-            "two_streams": two, "hip_graph": bool(args.graph),
+            "two_streams": two, "hip_graph": bool(args.graph), "wgrad_group": group,
             "device_bytes": wb.ex.nbytes,
         },
         "algorithmic_flops_per_step": flops,

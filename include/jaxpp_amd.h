@@ -163,6 +163,14 @@ typedef struct {
   const int32_t* seg_rows; /* device int32 [n_seg] or NULL: rows of each group that hold data;
                             * the rest of a group is zero padding, which JPP_GROUP_K then leaves
                             * out of the contraction (whole 64-row steps of it) */
+  /* One product over several operand pairs: with k_parts = 2..4 the contraction runs over
+   * (a, b), then (a_more[0], b_more[0]), ... - k elements each, same shapes and leading
+   * dimensions - as if the pairs were concatenated along the contraction index.  The
+   * weight gradients of several microbatches accumulate this way with one read and one write
+   * of the fp32 accumulator instead of one per microbatch.  0 or 1: one pair. */
+  const void* a_more[3];
+  const void* b_more[3];
+  int k_parts;
 } jpp_gemm_args;
 
 enum { JPP_GROUP_NONE = 0, JPP_GROUP_M = 1, JPP_GROUP_K = 2 };
@@ -377,6 +385,19 @@ typedef struct {
   int dtype;             /* jpp_dtype of parameters, activations and boundary tensors.
                             JPP_DTYPE_F32: every family, through the *_f32 operators and the
                             routing kernels' f32 form; gradient accumulators are f32 either way */
+  int wgrad_group;       /* 0, 1: each microbatch's weight gradients run in the task the table
+                            gives them.  2..4: the weight gradients of the microbatches
+                            g * wgrad_group .. + wgrad_group - 1 of a chunk run together, when
+                            the last of them is due, as one product per weight over all their
+                            tokens - the fp32 accumulator is then read and written once per
+                            group instead of once per microbatch.  A microbatch held back keeps
+                            its residual slot (the stage allocates wgrad_group - 1 slots per
+                            chunk beyond max_live, and jpp_stage_live_slots counts them);
+                            jpp_stage_join runs what is still held back, so call it (or
+                            jpp_stage_zero_grads / jpp_stage_adam_step, which do) before reading
+                            the accumulators.  Groups are fixed by microbatch index, so the
+                            accumulators do not depend on the order of tasks.  One stream,
+                            bf16, fused_wgrad_accum only. */
 } jpp_stage_desc;
 
 

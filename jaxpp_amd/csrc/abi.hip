@@ -62,7 +62,13 @@ bool jpp_probe_wants(const char* kernel_class) {
   return g_probe.active && g_probe.err == hipSuccess && g_probe.cls == kernel_class;
 }
 
+// A bracket opened inside another one on the same thread (a launcher that hands over to
+// another launcher of the same class) is ignored: the outer bracket covers it, and locking
+// launch_mu twice from one thread would never return.
+thread_local int t_probe_depth = 0;
+
 void jpp_probe_open(hipStream_t stream) {
+  if (t_probe_depth++ > 0) return;
   g_probe.launch_mu.lock();      // released by jpp_probe_close
   std::lock_guard<std::mutex> lock(g_probe.mu);
   Probe& p = g_probe;
@@ -97,6 +103,7 @@ void jpp_probe_open(hipStream_t stream) {
 }
 
 void jpp_probe_close(hipStream_t stream, double flops, double bytes) {
+  if (--t_probe_depth > 0) return;
   {
     std::lock_guard<std::mutex> lock(g_probe.mu);
     Probe& p = g_probe;

@@ -510,6 +510,7 @@ int attn_check(const jpp_attn_args* a, const char* who, Attn32& p) {
 extern "C" {
 
 int jpp_gemm_f32(void* stream, const jpp_gemm_args* a) {
+  JPP_REQUIRE(!a || a->k_parts <= 1, "gemm_f32: one operand pair per product");
   JPP_REQUIRE(a && a->a && a->b && a->c, "gemm_f32: null operand");
   const bool group_k = a->group_mode == JPP_GROUP_K;
   JPP_REQUIRE(a->m > 0 && a->n > 0 && (a->k > 0 || group_k) && a->m % 64 == 0 && a->n % 64 == 0 &&

@@ -34,6 +34,11 @@ namespace {
 struct GemmParams {
   const bf16_t* a;
   const bf16_t* b;
+  // a contraction spread over several operand pairs of k elements each (see k_parts in the
+  // header): pair i > 0 is (a_more[i-1], b_more[i-1]); kt_part = K-steps per pair
+  const bf16_t* a_more[3];
+  const bf16_t* b_more[3];
+  int k_parts, kt_part;
   void* c;
   void* c2;
   const bf16_t* bias;
@@ -112,7 +117,18 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = (pid % width) / gsize;
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS>
+// Operand tile of K-step kt when the contraction runs over up to four operand pairs of
+// kt_part K-steps each (all arguments wave-uniform).
+__device__ __forceinline__ const bf16_t* part_ptr(const bf16_t* p0, const bf16_t* p1,
+                                                  const bf16_t* p2, const bf16_t* p3, int kt,
+                                                  int kt_part, int k_parts, long step) {
+  if (k_parts <= 1) return p0 + (long)kt * step;
+  const int part = (kt >= kt_part) + (kt >= 2 * kt_part) + (kt >= 3 * kt_part);
+  const bf16_t* base = part == 0 ? p0 : part == 1 ? p1 : part == 2 ? p2 : p3;
+  return base + (long)(kt - part * kt_part) * step;
+}
+
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS, bool KP = false>
 __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   using TileA = DmaTile<BM, TA, NW>;
   using TileB = DmaTile<BN, TB, NW>;
@@ -133,9 +149,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
                 p.tiles_n, tm, tn);
   const long m0 = (long)tm * BM, n0 = (long)tn * BN;
 
-  const bf16_t* a_src = TA ? p.a + m0 : p.a + m0 * p.lda;
-  const bf16_t* b_src = TB ? p.b + n0 : p.b + n0 * p.ldb;
-  int kt_n = p.k / 64;
+  const long a_off = TA ? m0 : m0 * p.lda, b_off = TB ? n0 : n0 * p.ldb;
+  const bf16_t* a_src = p.a + a_off;
+  const bf16_t* b_src = p.b + b_off;
+  int kt_n = p.k / 64 * (KP ? p.k_parts : 1);
   if (p.group_mode == JPP_GROUP_M) {
     // rows of A and C are grouped by expert; each group multiplies its own B
     if (m0 >= p.seg[p.n_seg]) return;
@@ -157,6 +174,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   }
   const long a_step = TA ? 64 * p.lda : 64;
   const long b_step = TB ? 64 * p.ldb : 64;
+  // operand tiles of K-step kt: with several operand pairs the steps run through pair 0,
+  // then pair 1, ... (kt and the pair index are wave-uniform: scalar arithmetic; the pair
+  // pointers are picked by a chain of selects, never by indexing the kernel arguments)
+  // (kernels built without KP take one pair and keep the plain address arithmetic)
+  const int k_parts = KP ? p.k_parts : 1, kt_part = p.kt_part;
+  const bf16_t* const a1 = KP ? p.a_more[0] + a_off : a_src;
+  const bf16_t* const a2 = KP ? p.a_more[1] + a_off : a_src;
+  const bf16_t* const a3 = KP ? p.a_more[2] + a_off : a_src;
+  const bf16_t* const b1 = KP ? p.b_more[0] + b_off : b_src;
+  const bf16_t* const b2 = KP ? p.b_more[1] + b_off : b_src;
+  const bf16_t* const b3 = KP ? p.b_more[2] + b_off : b_src;
+#define a_at(kt) (KP ? part_ptr(a_src, a1, a2, a3, (kt), kt_part, k_parts, a_step) : a_src + (long)(kt) * a_step)
+#define b_at(kt) (KP ? part_ptr(b_src, b1, b2, b3, (kt), kt_part, k_parts, b_step) : b_src + (long)(kt) * b_step)
 
   // of tile (i, j) a lane holds row wm BM/2 + 16 i + lane % 16 and the four columns
   // wn BN/WN + 16 j + 4 (lane / 16) + {0..3}
@@ -206,9 +236,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       const int k = min(s, kt_n - 1);
-      TileA::template issue<0, IA>(uniform_ptr(a_src + k * a_step), offa, lds0 + s * STAGE, wave);
-      TileB::template issue<0, IB>(uniform_ptr(b_src + k * b_step), offb, lds0 + s * STAGE + A_BYTES,
-                                   wave);
+      TileA::template issue<0, IA>(uniform_ptr(a_at(k)), offa, lds0 + s * STAGE, wave);
+      TileB::template issue<0, IB>(uniform_ptr(b_at(k)), offb, lds0 + s * STAGE + A_BYTES, wave);
     }
     dma_wait<(NS - 1) * OPB>();  // stage 0 has landed; the others may still be in flight
   }
@@ -227,8 +256,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     const uint8_t* na = smem + nst * STAGE;
     // past the end the last K-step is fetched again, unused
     const int kn = min(kt + NS, kt_n - 1);
-    const bf16_t* ga = uniform_ptr(a_src + (long)kn * a_step);
-    const bf16_t* gb = uniform_ptr(b_src + (long)kn * b_step);
+    const bf16_t* ga = uniform_ptr(a_at(kn));
+    const bf16_t* gb = uniform_ptr(b_at(kn));
 #pragma unroll
     for (int ks = 0; ks < NB; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1, curw = ks / HS, part = ks % HS;
@@ -280,6 +309,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int i = 0; i < TMH; ++i) fx[0][i] = TileA::frag16(na, row_x + i * 16, 0, lane);
       }
+#ifdef JPP_SCHED_FENCE
+      // the fragment reads above are issued before this block's MFMAs and stay there: the
+      // compiler's scheduler would otherwise sink each read to just before its first use and
+      // expose the LDS latency in front of every few MFMAs
+      __builtin_amdgcn_sched_barrier(0);
+#endif
       // the refill of the retired stage is spread over this block's MFMAs: a wave that
       // issues its loads back to back waits on the memory pipeline with its MFMAs behind it
       constexpr int PARTS = TMH < IA && TMH < IB ? TMH : (IA < IB ? IA : IB);
@@ -309,6 +344,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
               acc[part * TMH + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                   fw[curw][j], fx[cur][i], acc[part * TMH + i][j], 0, 0, 0);
       }
+#ifdef JPP_SCHED_FENCE
+      __builtin_amdgcn_sched_barrier(0);
+#endif
     }
     if constexpr (EPI == JPP_EPI_ACC_F32) {
       if (stream_c && kt < NBT)
@@ -484,6 +522,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   }
 }
 
+#undef a_at
+#undef b_at
+
 template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS>
 const char* class_name() {
   // built once per instantiation; the initialisation of a function-local static is
@@ -501,23 +542,35 @@ const char* class_name() {
   return name.c_str();
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4, int NS = 2>
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW = 4, int NS = 2, bool KP = false>
 int launch(hipStream_t stream, GemmParams& p) {
   // two operand stages; the bf16 epilogues stage half a tile in fp32 with padded rows
   constexpr int SMEM_LOOP = NS * (BM + BN) * 128, SMEM_EPI = (BM / 2) * (BN * 4 + 16);
   // + NS+1 buffers of NW rows of the fp32 tile (padded) for C += A B
   constexpr int SMEM = EPI == JPP_EPI_ACC_F32 ? SMEM_LOOP + (NS + 1) * NW * (1024 + 16)
                        : (EPI == JPP_EPI_F32 || SMEM_LOOP > SMEM_EPI) ? SMEM_LOOP : SMEM_EPI;
+  if constexpr (!KP) {
+    // several operand pairs: only the accumulating weight-gradient kernels on 256-wide tiles
+    // are built for that
+    if (p.k_parts > 1) {
+      if constexpr (TA && TB && EPI == JPP_EPI_ACC_F32 && BN == 256 && NW == 8 && NS == 2)
+        return launch<BM, BN, TA, TB, EPI, NW, NS, true>(stream, p);
+      else
+        return jpp_set_error(JPP_ERR_INVALID, "gemm: several operand pairs are supported for "
+                             "accumulated weight gradients (tn, JPP_EPI_ACC_F32) on 256x256 and "
+                             "128x256 tiles");
+    }
+  }
   // algorithmic extent: grouped launches count the non-padding rows when the caller gave them
   const double cb = EPI == JPP_EPI_ACC_F32 || EPI == JPP_EPI_DSWIGLU ? 8
                     : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;
-  double am = p.m, ak = p.k, copies = 1;
+  double am = p.m, ak = (double)p.k * (p.k_parts > 1 ? p.k_parts : 1), copies = 1;
   if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
   if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
   const double b_bytes = 2.0 * p.n * ak * (p.group_mode == JPP_GROUP_M ? p.n_seg : 1);
   ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW, NS>(), 2.0 * am * p.n * ak,
                    2.0 * am * ak + b_bytes + copies * am * p.n * cb);
-  auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW, NS>;
+  auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW, NS, KP>;
   static_assert(SMEM <= 160 * 1024, "LDS of one CU");
   // the LDS limit of a kernel is sticky: set once per instantiation, by whichever host
   // thread launches it first (the others wait for that call and see its result)
@@ -574,6 +627,10 @@ int choose_tile(long m, long n) {
 void shift_origin(GemmParams& p, bool ta, bool tb, int epi, long m_off, long n_off) {
   p.a += ta ? m_off : m_off * p.lda;
   p.b += tb ? n_off : n_off * p.ldb;
+  for (int i = 0; i + 1 < p.k_parts; ++i) {
+    p.a_more[i] += ta ? m_off : m_off * p.lda;
+    p.b_more[i] += tb ? n_off : n_off * p.ldb;
+  }
   const long c_cols = epi == JPP_EPI_DSWIGLU ? 2 * n_off : n_off;  // dSwiGLU writes d gate, d up
   const bool f32 = epi == JPP_EPI_ACC_F32 || epi == JPP_EPI_F32;
   p.c = f32 ? (void*)((float*)p.c + m_off * p.ldc + c_cols)
@@ -640,6 +697,20 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   p.seg = a->seg; p.seg_rows = a->seg_rows; p.n_seg = a->n_seg; p.group_mode = a->group_mode;
   p.group_rows = a->group_rows;
   p.stride_b = a->stride_b; p.stride_c = a->stride_c;
+  p.k_parts = a->k_parts > 1 ? a->k_parts : 1;
+  p.kt_part = (int)(a->k / 64);
+  for (int i = 0; i < 3; ++i) {
+    p.a_more[i] = (const bf16_t*)a->a_more[i];
+    p.b_more[i] = (const bf16_t*)a->b_more[i];
+  }
+  if (a->k_parts > 1) {
+    JPP_REQUIRE(a->k_parts <= 4 && a->group_mode == JPP_GROUP_NONE,
+                "gemm: at most 4 operand pairs, and not in a grouped problem");
+    for (int i = 0; i + 1 < a->k_parts; ++i)
+      JPP_REQUIRE(a->a_more[i] && a->b_more[i] &&
+                      ((uintptr_t)a->a_more[i] | (uintptr_t)a->b_more[i]) % 16 == 0,
+                  "gemm: operand pair %d is null or not 16-byte aligned", i + 1);
+  }
   if (a->group_mode != JPP_GROUP_NONE) {
     JPP_REQUIRE(a->group_mode == JPP_GROUP_M || a->group_mode == JPP_GROUP_K,
                 "gemm: unknown group_mode %d", a->group_mode);

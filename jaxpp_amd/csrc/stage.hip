@@ -104,6 +104,12 @@ struct jpp_stage {
   hipEvent_t ev_tail = nullptr;          // last work queued on `side`
   bool tail_pending = false;
 
+  // Weight gradients of up to wg consecutive microbatches (aligned groups mubatch / wg) run as
+  // one product per weight: pend[chunk] lists the (microbatch, slot) pairs whose input-
+  // gradient half is done and whose weight-gradient half waits for the rest of its group.
+  int wg = 1;
+  std::vector<std::vector<std::pair<int, int>>> pend;
+
   bool f32() const { return d.dtype == JPP_DTYPE_F32; }
   void* P(int chunk, int layer, int i) {
     return params + (((size_t)chunk * d.layers_per_chunk + layer) * layer_elems + poff[i]) * es;
@@ -227,6 +233,25 @@ int wgrad(jpp_stage* s, hipStream_t st, const void* x, int64_t ldx, const void* 
   void* g = s->S<>(s->s_wg);
   RC(gemm(s, st, x, ldx, 1, dy, lddy, 1, g, cols, rows, cols, s->T, JPP_EPI_BF16));
   return jpp_grad_accum_f32(st, acc, g, rows * cols, 0);
+}
+
+// dW (+)= sum over n microbatches of X_i^T dY_i: one product over n operand pairs when the
+// matrix is large enough to fill the device, else one product per microbatch (in order)
+int wgrad_n(jpp_stage* s, hipStream_t st, int n, const void* const* xs, int64_t ldx,
+            const void* const* dys, int64_t lddy, float* acc, int64_t rows, int64_t cols) {
+  const bool big = rows % 256 == 0 && cols % 256 == 0 && (rows / 256) * (cols / 256) >= 192;
+  if (n == 1 || !big || s->f32() || !s->d.fused_wgrad_accum) {
+    for (int i = 0; i < n; ++i) RC(wgrad(s, st, xs[i], ldx, dys[i], lddy, acc, rows, cols));
+    return JPP_OK;
+  }
+  jpp_gemm_args g;
+  memset(&g, 0, sizeof(g));
+  g.a = xs[0]; g.b = dys[0]; g.c = acc; g.m = rows; g.n = cols; g.k = s->T;
+  g.lda = ldx; g.ldb = lddy; g.ldc = cols; g.trans_a = 1; g.trans_b = 1;
+  g.epilogue = JPP_EPI_ACC_F32;
+  g.k_parts = n;
+  for (int i = 1; i < n; ++i) { g.a_more[i - 1] = xs[i]; g.b_more[i - 1] = dys[i]; }
+  return jpp_gemm_bf16(st, &g);
 }
 
 int norm_f(jpp_stage* s, hipStream_t st, const void* x, const void* gamma, const void* beta,
@@ -495,6 +520,93 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
   return JPP_OK;
 }
 
+// Weight-gradient half of layer li for n microbatches of one chunk at once (their residuals
+// and cotangents in slots[0..n-1]); the dense products run over all of them together, the
+// experts' grouped products and the router's, whose row groups differ from microbatch to
+// microbatch, one microbatch after the other.
+int layer_bwd_w_group(jpp_stage* s, hipStream_t st, int chunk, int li, int n, uint8_t* const* slots) {
+  const LayerStash& L = s->lay[li];
+  const int64_t h = s->h, f = s->f;
+  const void* xs[4];
+  const void* dys[4];
+  auto gather = [&](const Buf& x, const Buf& dy) {
+    for (int i = 0; i < n; ++i) { xs[i] = slots[i] + x.off; dys[i] = slots[i] + dy.off; }
+  };
+  if (s->d.family == JPP_FAMILY_BERT) {
+    gather(L.g, L.dc);   RC(wgrad_n(s, st, n, xs, f, dys, h, s->G(chunk, li, B_W2), f, h));
+    gather(L.x1, L.du);  RC(wgrad_n(s, st, n, xs, h, dys, f, s->G(chunk, li, B_W1), h, f));
+    gather(L.ctx, L.da); RC(wgrad_n(s, st, n, xs, h, dys, h, s->G(chunk, li, B_Wo), h, h));
+    gather(L.x, L.dqkv); RC(wgrad_n(s, st, n, xs, h, dys, 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
+    return JPP_OK;
+  }
+  if (s->d.family == JPP_FAMILY_DECODER) {
+    gather(L.g, L.dyin);   RC(wgrad_n(s, st, n, xs, f, dys, h, s->G(chunk, li, B_W2), f, h));
+    gather(L.n2, L.du);    RC(wgrad_n(s, st, n, xs, h, dys, f, s->G(chunk, li, B_W1), h, f));
+    gather(L.ctx, L.dh1);  RC(wgrad_n(s, st, n, xs, h, dys, h, s->G(chunk, li, B_Wo), h, h));
+    gather(L.n1, L.dqkv);  RC(wgrad_n(s, st, n, xs, h, dys, 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
+    return JPP_OK;
+  }
+  if (s->d.family == JPP_FAMILY_MIXTRAL) {
+    float* partial = s->S<float>(s->s_partial);
+    const int E = s->d.n_experts;
+    for (int i = 0; i < n; ++i) {
+      uint8_t* slot = slots[i];
+      auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
+      jpp_moe_args ma;
+      moe_args(s, ma, slot, L, chunk, li);
+      RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.s), f, 1, at(L.deo), h, 1, 0, s->G(chunk, li, X_Wd), h,
+               f * h, f, h, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+      RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, at(L.dgu), 2 * f, 1, 0,
+               s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+      RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)at(L.dlogits), s->G(chunk, li, X_Wr),
+                              partial));
+    }
+    gather(L.ctx, L.dh1);  RC(wgrad_n(s, st, n, xs, s->ctxw, dys, h, s->G(chunk, li, X_Wo), s->ctxw, h));
+    gather(L.n1, L.dqkv);  RC(wgrad_n(s, st, n, xs, h, dys, s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw));
+    return JPP_OK;
+  }
+  gather(L.s, L.dyin);   RC(wgrad_n(s, st, n, xs, f, dys, h, s->G(chunk, li, L_Wd), f, h));
+  gather(L.n2, L.dgu);   RC(wgrad_n(s, st, n, xs, h, dys, 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f));
+  gather(L.ctx, L.dh1);  RC(wgrad_n(s, st, n, xs, s->ctxw, dys, h, s->G(chunk, li, L_Wo), s->ctxw, h));
+  gather(L.n1, L.dqkv);  RC(wgrad_n(s, st, n, xs, h, dys, s->qkvw, s->G(chunk, li, L_Wqkv), h, s->qkvw));
+  return JPP_OK;
+}
+
+// Runs the pending weight-gradient halves of a chunk (a whole group, or what a flush finds)
+// and releases their slots.
+int run_pending_w(jpp_stage* s, hipStream_t st, int chunk) {
+  auto& pend = s->pend[chunk];
+  if (pend.empty()) return JPP_OK;
+  uint8_t* slots[4];
+  const int n = (int)pend.size();
+  for (int i = 0; i < n; ++i) slots[i] = s->slots[pend[i].second];
+  for (int li = s->d.layers_per_chunk - 1; li >= 0; --li)
+    RC(layer_bwd_w_group(s, st, chunk, li, n, slots));
+  for (auto& e : pend) {
+    const auto key = std::make_pair(chunk, e.first);
+    s->free_slots.push_back(e.second);
+    s->live.erase(key);
+    s->phase.erase(key);
+  }
+  pend.clear();
+  return JPP_OK;
+}
+
+// The input-gradient half of (chunk, mb) is done: its weight-gradient half runs now if it
+// completes its group (microbatches mb / G * G .. + G - 1), else it waits.
+int defer_or_run_w(jpp_stage* s, hipStream_t st, int chunk, int mb, int slot_i) {
+  auto& pend = s->pend[chunk];
+  if (!pend.empty() && pend.front().first / s->wg != mb / s->wg) RC(run_pending_w(s, st, chunk));
+  pend.emplace_back(mb, slot_i);
+  if (mb % s->wg == s->wg - 1 || (int)pend.size() == s->wg) RC(run_pending_w(s, st, chunk));
+  return JPP_OK;
+}
+
+int flush_pending_w(jpp_stage* s, hipStream_t st) {
+  for (int c = 0; c < (int)s->pend.size(); ++c) RC(run_pending_w(s, st, c));
+  return JPP_OK;
+}
+
 void carve_layer(jpp_stage* s, Carver& c, LayerStash& L, bool with_w) {
   const size_t T = s->T, h = s->h, f = s->f, e = s->es;
   const size_t stat = (size_t)s->d.batch * s->d.n_heads * s->d.seq * 4;
@@ -608,8 +720,16 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
     JPP_REQUIRE(d->fused_wgrad_accum,
                 "stage_create: f32 stages accumulate in the weight-gradient GEMM");
 
+  JPP_REQUIRE(d->wgrad_group >= 0 && d->wgrad_group <= 4, "stage_create: wgrad_group must be 0..4");
+  if (d->wgrad_group > 1)
+    JPP_REQUIRE(!d->two_streams && d->fused_wgrad_accum && d->dtype == JPP_DTYPE_BF16,
+                "stage_create: grouped weight gradients need one stream, bf16 and accumulation "
+                "in the GEMM");
+
   jpp_stage* s = new jpp_stage();
   s->d = *d;
+  s->wg = d->wgrad_group > 1 ? d->wgrad_group : 1;
+  s->pend.resize(d->n_chunks);
   s->es = d->dtype == JPP_DTYPE_F32 ? 4 : 2;
   s->d.n_kv_heads = kvh;
   s->d.head_dim = hd;
@@ -639,15 +759,18 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   // residual slots
   Carver slot;
   s->lay.resize(d->layers_per_chunk);
+  // cotangents the weight-gradient half reads live in the slot whenever that half may run
+  // in a later task than the input-gradient half
+  const bool slot_w = d->split_backward || s->wg > 1;
   for (auto& L : s->lay) {
     carve_layer(s, slot, L, false);
-    if (d->split_backward) carve_w(s, slot, L);
+    if (slot_w) carve_w(s, slot, L);
   }
   s->slot_bytes = slot.total;
 
   // scratch
   Carver sc;
-  if (!d->split_backward)
+  if (!slot_w)
     for (int i = 0; i < (d->two_streams ? 3 : 1); ++i) carve_w(s, sc, s->wsets[i]);
   const size_t e = s->es;
   s->s_dx[0] = sc.take(T * h * e);
@@ -683,12 +806,14 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   hipError_t e3 = e2 == hipSuccess ? hipMalloc((void**)&s->scratch, s->scratch_bytes) : e2;
   hipError_t e4 = e3;
   if (e3 == hipSuccess) {
-    for (int i = 0; i < d->max_live; ++i) {
+    // a chunk may hold G - 1 microbatches back beyond the schedule's own peak
+    const int n_slots = d->max_live + d->n_chunks * (s->wg - 1);
+    for (int i = 0; i < n_slots; ++i) {
       uint8_t* p = nullptr;
       e4 = hipMalloc((void**)&p, s->slot_bytes);
       if (e4 != hipSuccess) break;
       s->slots.push_back(p);
-      s->free_slots.push_back(d->max_live - 1 - i);
+      s->free_slots.push_back(n_slots - 1 - i);
     }
   }
   if (e4 != hipSuccess) {
@@ -697,7 +822,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
                          hipGetErrorString(e4));
   }
   s->total_bytes = n_layers * s->layer_elems * (4 + s->es) + s->scratch_bytes +
-                   s->slot_bytes * d->max_live;
+                   s->slot_bytes * s->slots.size();
   hipMemset(s->params, 0, n_layers * s->layer_elems * s->es);
   hipMemset(s->grads, 0, n_layers * s->layer_elems * 4);
 
@@ -730,9 +855,9 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
     mk(&s->ev_fork);
     mk(&s->ev_tail);
     for (auto& ev : s->ev_set) mk(&ev);
-    s->ev_slot.assign(d->max_live, nullptr);
-    s->ev_bwd_i.assign(d->max_live, nullptr);
-    s->slot_pending.assign(d->max_live, 0);
+    s->ev_slot.assign(s->slots.size(), nullptr);
+    s->ev_bwd_i.assign(s->slots.size(), nullptr);
+    s->slot_pending.assign(s->slots.size(), 0);
     for (auto& ev : s->ev_slot) mk(&ev);
     for (auto& ev : s->ev_bwd_i) mk(&ev);
   }
@@ -798,12 +923,17 @@ int jpp_stage_grad_ptr(jpp_stage* s, int chunk, int layer, int i, float** ptr) {
 
 int jpp_stage_join(jpp_stage* s, void* stream) {
   JPP_REQUIRE(s, "stage: null");
+  RC(flush_pending_w(s, (hipStream_t)stream));   // weight gradients held back for their group
   if (s->tail_pending) JPP_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, s->ev_tail, 0));
   return JPP_OK;
 }
 
 int jpp_stage_quiesce(jpp_stage* s) {
   JPP_REQUIRE(s, "stage: null");
+  for (auto& pend : s->pend)
+    if (!pend.empty())
+      return jpp_set_error(JPP_ERR_STATE, "stage_quiesce: weight gradients of %d microbatch(es) are "
+                           "held back for their group; call jpp_stage_join first", (int)pend.size());
   if (s->side) JPP_CHECK_HIP(hipStreamSynchronize(s->side));
   // nothing of the stage's own stream is in flight: no later task has to wait for it
   std::fill(s->slot_pending.begin(), s->slot_pending.end(), 0);
@@ -909,7 +1039,7 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
     if (s->free_slots.empty())
       return jpp_set_error(JPP_ERR_STATE,
                            "run_task(FWD): all %d residual slots are live; the schedule needs a "
-                           "larger max_live", s->d.max_live);
+                           "larger max_live", (int)s->slots.size());
     const int slot_i = s->free_slots.back();
     s->free_slots.pop_back();
     s->live[key] = slot_i;
@@ -971,21 +1101,22 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
       }
       return JPP_OK;
     };
+    const bool slot_w = split || s->wg > 1;   // cotangents for the weight gradients: in the slot
     const void* dy = in;
     for (int li = nl - 1; li >= 0; --li) {
-      uint8_t* wbase = split ? slot : s->scratch;
-      const LayerStash& W = split ? s->lay[li] : s->wsets[set_of(li)];
-      if (!split) {
+      uint8_t* wbase = slot_w ? slot : s->scratch;
+      const LayerStash& W = slot_w ? s->lay[li] : s->wsets[set_of(li)];
+      if (!slot_w) {
         // this layer writes its own set and (its result) the set of the layer below
         RC(wait_set(set_of(li)));
         if (li > 0 && !bert) RC(wait_set(set_of(li - 1)));
       }
       void* dx;
       if (li == 0) dx = out;
-      else if (split && !bert) dx = slot + s->lay[li - 1].dyin.off;
+      else if (slot_w && !bert) dx = slot + s->lay[li - 1].dyin.off;
       else if (two && !bert) dx = s->scratch + s->wsets[set_of(li - 1)].dyin.off;
       else dx = s->S<>(s->s_dx[li & 1]);
-      if (!bert && li == nl - 1 && (split || two)) {
+      if (!bert && li == nl - 1 && (slot_w || two)) {
         // the weight gradients read the incoming cotangent later (a BWD_W task, or the
         // second stream after this call has returned): keep a copy
         uint8_t* keep = wbase + W.dyin.off;
@@ -993,7 +1124,7 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
         dy = keep;
       }
       RC(layer_bwd_i(s, st, chunk, li, slot, wbase, W, dy, dx));
-      if (kind == JPP_BWD) {
+      if (kind == JPP_BWD && s->wg == 1) {
         if (two) {
           RC(fork());
           RC(layer_bwd_w(s, s->side, chunk, li, slot, wbase, W, dy));
@@ -1007,7 +1138,10 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
       }
       dy = dx;
     }
-    if (kind == JPP_BWD) {
+    if (kind == JPP_BWD && s->wg > 1) {
+      s->phase[key] = 3;                       // both halves issued or handed to the group
+      RC(defer_or_run_w(s, st, chunk, mb, slot_i));
+    } else if (kind == JPP_BWD) {
       if (two) RC(side_done_with_slot());
       s->free_slots.push_back(slot_i);
       s->live.erase(it);
@@ -1026,6 +1160,10 @@ int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in
     if (ph != 2)
       return jpp_set_error(JPP_ERR_STATE, "run_task(BWD_W): BWD_I of (chunk %d, mubatch %d) has not run",
                            chunk, mb);
+    if (s->wg > 1) {
+      s->phase[key] = 3;
+      return defer_or_run_w(s, st, chunk, mb, slot_i);
+    }
     hipStream_t ws = st;
     if (two) {
       // everything it needs was complete when the BWD_I task ended on the caller's stream

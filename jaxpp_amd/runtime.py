@@ -15,7 +15,9 @@ import numpy as np
 
 from jaxpp_amd.types import TaskType
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libjaxpp_amd.so")
+# JAXPP_AMD_LIB names another build of the library (A/B runs of two builds on one machine)
+_LIB_PATH = os.environ.get("JAXPP_AMD_LIB") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "lib", "libjaxpp_amd.so")
 _lib = None
 
 
@@ -37,7 +39,8 @@ class GemmArgs(C.Structure):
                 ("gelu_tanh", C.c_int), ("tile", C.c_int),
                 ("seg", C.c_void_p), ("n_seg", C.c_int), ("group_mode", C.c_int),
                 ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("group_rows", C.c_int64),
-                ("seg_rows", C.c_void_p)]
+                ("seg_rows", C.c_void_p),
+                ("a_more", C.c_void_p * 3), ("b_more", C.c_void_p * 3), ("k_parts", C.c_int)]
 
 
 class AttnArgs(C.Structure):
@@ -86,7 +89,7 @@ class StageDesc(C.Structure):
                 ("n_experts", C.c_int), ("top_k", C.c_int), ("n_chunks", C.c_int),
                 ("layers_per_chunk", C.c_int), ("max_live", C.c_int),
                 ("split_backward", C.c_int), ("fused_wgrad_accum", C.c_int),
-                ("two_streams", C.c_int), ("dtype", C.c_int)]
+                ("two_streams", C.c_int), ("dtype", C.c_int), ("wgrad_group", C.c_int)]
 
 
 EPI_BF16, EPI_GELU, EPI_DGELU, EPI_ACC_F32, EPI_F32, EPI_SWIGLU, EPI_DSWIGLU = range(7)
@@ -440,10 +443,15 @@ class probe:
 def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, bias=None,
          resid=None, ldresid=0, aux=None, ldaux=0, c2=None, ldc2=0, gelu_tanh=0, tile=0,
          stream=None, seg=None, n_seg=0, group_mode=0, stride_b=0, stride_c=0, group_rows=0,
-         seg_rows=None, f32=False):
+         seg_rows=None, f32=False, more=()):
+    """`more`: further (a, b) operand pairs the contraction continues over (k elements each)."""
     g = GemmArgs(a, b, c, c2, bias, resid, aux, m, n, k, lda, ldb, ldc, ldc2, ldresid, ldaux,
                  int(trans_a), int(trans_b), epilogue, gelu_tanh, tile, seg, n_seg, group_mode,
                  stride_b, stride_c, group_rows, seg_rows)
+    if more:
+        g.a_more = (C.c_void_p * 3)(*([pa for pa, _ in more] + [None] * (3 - len(more))))
+        g.b_more = (C.c_void_p * 3)(*([pb for _, pb in more] + [None] * (3 - len(more))))
+        g.k_parts = 1 + len(more)
     check((load().jpp_gemm_f32 if f32 else load().jpp_gemm_bf16)(stream, C.byref(g)))
 
 
@@ -468,7 +476,7 @@ class StageExecutor:
 
     def __init__(self, spec, n_chunks: int, layers_per_chunk: int, max_live: int,
                  split_backward: bool = False, fused_wgrad_accum: bool = True,
-                 two_streams: bool = False):
+                 two_streams: bool = False, wgrad_group: int = 0):
         require_gpu()
         self.spec = spec
         self.dtype = getattr(spec, "dtype", "bf16")
@@ -477,7 +485,7 @@ class StageExecutor:
                       spec.seq, spec.batch, int(spec.causal), spec.rope_theta, spec.eps,
                       int(spec.gelu_tanh), spec.n_experts, spec.top_k, n_chunks,
                       layers_per_chunk, max_live, int(split_backward), int(fused_wgrad_accum),
-                      int(two_streams), DTYPE[self.dtype])
+                      int(two_streams), DTYPE[self.dtype], int(wgrad_group))
         h = C.c_void_p()
         check(load().jpp_stage_create(C.byref(d), C.byref(h)))
         self.handle = h.value

@@ -368,11 +368,11 @@ def test_llama_70b_layer_on_a_zero_bubble_row_matches_oracle():
 
 
 # The oracle multiplies on the host: at the bench's 2 x 4096 tokens the eight layer passes of a
-# DualPipeV(4, 2) row are 1.6e14 FLOP there (minutes), so the sequences are 1024 long here.  All
+# DualPipeV(4, 2) row are 1.6e14 FLOP there (minutes), so the sequences are 512 long here.  All
 # widths are the bench's: hidden 4096, 32 / 8 heads, 8 experts of SwiGLU 14336, top-2.  The
 # expert products over the bench's 16 384 token copies are covered by
 # test_grouped_gemms_at_full_size.
-MIXTRAL_8X7B_LAYER = LayerSpec("mixtral", 4096, 32, 14336, 1024, 2, n_kv_heads=8, head_dim=128,
+MIXTRAL_8X7B_LAYER = LayerSpec("mixtral", 4096, 32, 14336, 512, 2, n_kv_heads=8, head_dim=128,
                                causal=True, rope_theta=5e5, eps=1e-5, n_experts=8, top_k=2)
 
 
@@ -462,3 +462,27 @@ def test_bench_row_equals_sequential_order(name, peak):
             for pname, v in gd.items():
                 np.testing.assert_array_equal(g[i][pname], v, err_msg=f"{what}: grad {i}/{pname}")
     ex.close()
+    group = bench.default_wgrad_group(wl, two)
+    if group > 1:
+        # the mode the bench runs by default: weight gradients of `group` microbatches as one
+        # product per weight.  Outputs bit-identical; accumulators equal up to f32
+        # reassociation; a microbatch held back keeps its slot, so the peak is higher.
+        del wb, outs_sched, outs_loop, grads_sched, grads_loop
+        wb = bench.Workbench(wl, fused=True, two_streams=two, wgrad_group=group)
+        ex = wb.ex
+        ex.zero_grads()
+        for b in outs.values():
+            b.zero()
+        live_peak = 0
+        for pt in plan.tasks:
+            ex.run_task(pt.exec_kind, pt.chunk, pt.task.mubatch_idx, *io(pt))
+            live_peak = max(live_peak, ex.live_slots())
+        assert peak < live_peak <= peak + plan.n_chunks * (group - 1)
+        outs_grp, grads_grp = snapshot()
+        assert ex.live_slots() == 0
+        for k, v in outs_seq.items():
+            np.testing.assert_array_equal(outs_grp[k], v, err_msg=f"grouped: output of {k}")
+        for i, gd in enumerate(grads_seq):
+            for pname, v in gd.items():
+                parity.close(grads_grp[i][pname], v, 1e-5, f"grouped: grad {i}/{pname}")
+        ex.close()

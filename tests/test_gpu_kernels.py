@@ -107,6 +107,30 @@ def test_gemm(ta, tb, epi, tile, m, n, k):
               "gemm gelu")
 
 
+@pytest.mark.parametrize("parts,m,n,k,tile", [(2, 256, 512, 192, 4), (4, 512, 256, 640, 4), (3, 1024, 768, 1024, 3),
+                                              (4, 4096, 3072, 512, 0), (2, 4096, 6144, 2048, 0)])
+def test_gemm_contraction_over_several_operand_pairs(parts, m, n, k, tile):
+    """C += sum_i A_i^T B_i in one launch (the weight gradients of several microbatches):
+    against numpy on the concatenated operands, and bit-identical to ... nothing else: the
+    summation order is the launch's own, so the check is numerical."""
+    rng = np.random.default_rng(parts + m + n + k)
+    As = [rnd(rng, k, m) for _ in range(parts)]          # stored [K, M]: trans_a = 1
+    Bs = [rnd(rng, k, n, scale=0.05) for _ in range(parts)]
+    prev = rng.standard_normal((m, n)).astype(np.float32)
+    want = prev + sum(a.astype(np.float64).T @ b.astype(np.float64) for a, b in zip(As, Bs))
+    dA, dB = [dev_bf16(a) for a in As], [dev_bf16(b) for b in Bs]
+    dc = rt.DeviceBuffer.from_numpy(prev)
+    rt.gemm(dA[0].ptr, dB[0].ptr, dc.ptr, m, n, k, m, n, n, 1, 1, rt.EPI_ACC_F32, tile=tile,
+            more=[(a.ptr, b.ptr) for a, b in zip(dA[1:], dB[1:])])
+    rt.sync()
+    close(dc.download(np.float32, (m, n)), want, 1e-4 * math.sqrt(k * parts), "gemm over operand pairs")
+    with pytest.raises(rt.JppError, match="operand pair 1 is null"):
+        rt.gemm(dA[0].ptr, dB[0].ptr, dc.ptr, m, n, k, m, n, n, 1, 1, rt.EPI_ACC_F32, more=[(None, dB[0].ptr)])
+    with pytest.raises(rt.JppError, match="several operand pairs are supported for"):
+        rt.gemm(dA[0].ptr, dB[0].ptr, dc.ptr, m, n, k, m, n, n, 1, 1, rt.EPI_F32, tile=4,
+                more=[(dA[0].ptr, dB[0].ptr)])
+
+
 def test_gemm_rejects_bad_shapes():
     d = rt.DeviceBuffer(1 << 16)
     with pytest.raises(rt.JppError, match="multiples of 128"):

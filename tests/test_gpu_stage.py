@@ -40,13 +40,14 @@ def _gpu():
 close = parity.close
 
 
-def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_streams=True):
+def run_on_gpu(spec, plan, layers_per_chunk, params, fused=True, seed=0, two_streams=True,
+               wgrad_group=0):
     """Runs the rank's row.  With two_streams the row is queued without host waits in between:
     weight gradients trail on the stage's stream and the forward of a fused entry runs on a
     second caller stream (RankLoop); otherwise one task at a time with a device sync."""
     shape = (spec.tokens, spec.hidden)
     ex = rt.StageExecutor(spec, plan.n_chunks, layers_per_chunk, plan.max_live,
-                          plan.split_backward, fused, two_streams)
+                          plan.split_backward, fused, two_streams, wgrad_group)
     for c, stage in enumerate(plan.stages):
         for li in range(layers_per_chunk):
             ex.set_params(c, li, params[stage][li])
@@ -174,6 +175,78 @@ def test_task_order_does_not_change_gradients():
             np.testing.assert_array_equal(other[2][0][0][k], v, err_msg=k)
         for k, v in res[0][1].items():
             np.testing.assert_array_equal(other[1][k], v)
+
+
+WIDE_LLAMA = LayerSpec("llama", 2048, 16, 3072, 512, 2, n_kv_heads=4, head_dim=128, causal=True,
+                       rope_theta=5e5, eps=1e-5)
+
+
+@pytest.mark.parametrize("name,spec,sched,n,rank", [
+    ("llama-interleaved", WIDE_LLAMA, S.Interleaved1F1B(4, 2), 6, 0),   # 2 chunks, groups {0..3}, {4, 5}
+    ("llama-zb", WIDE_LLAMA, S.ZeroBubble(2), 5, 1),                    # explicit BWD_W tasks
+    ("mixtral-dualpipev", MIXTRAL, S.DualPipeV(4, 2), 5, 0),
+    ("bert-1f1b", BERT, S.Std1F1B(2), 5, 0),
+], ids=lambda v: v if isinstance(v, str) else None)
+def test_grouped_weight_gradients(name, spec, sched, n, rank):
+    """wgrad_group: the weight gradients of 2 or 4 consecutive microbatches as one product per
+    weight (WIDE_LLAMA's gate/up and QKV matrices are large enough for that; its other weights
+    and the small layers take one product per microbatch from the same deferred task).
+    Outputs and input cotangents must be bit-identical to the ungrouped run, the accumulators
+    equal up to f32 reassociation (1e-5) and within the bf16 bar of the oracle; a group's last
+    member being absent (n not a multiple of the group) is settled by jpp_stage_join."""
+    plan = make_rank_plan(sched, n, rank)
+    params = make_params(spec, plan.stages, 1)
+    base = run_on_gpu(spec, plan, 1, params, two_streams=False)
+    row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
+    _, _, acc_w = run_on_oracle(spec, plan, params, row)
+    for group in (2, 4):
+        got = run_on_gpu(spec, plan, 1, params, two_streams=False, wgrad_group=group)
+        for k, v in base[0].items():
+            np.testing.assert_array_equal(got[0][k], v, err_msg=f"group {group}: y{k}")
+        for k, v in base[1].items():
+            np.testing.assert_array_equal(got[1][k], v, err_msg=f"group {group}: dx{k}")
+        for st in plan.stages:
+            for pname, v in base[2][st][0].items():
+                close(got[2][st][0][pname], v, 1e-5, f"group {group}: grad {st}/{pname} vs ungrouped")
+                if not (spec.family == "mixtral" and pname in ("Wr", "Wgu", "Wd")):
+                    want = acc_w[st][0][pname].reshape(v.shape)
+                    parity.close_stage(got[2][st][0][pname], want, 2e-2, f"group {group}: grad {st}/{pname}")
+
+
+def test_grouped_weight_gradients_do_not_depend_on_task_order():
+    spec, n = WIDE_LLAMA, 4
+    params = make_params(spec, [0], 1)
+    res = [run_on_gpu(spec, make_rank_plan(sched, n, 0), 1, params, two_streams=False, wgrad_group=2)
+           for sched in (S.GPipe(2), S.Std1F1B(2), S.ZeroBubble(2))]
+    for other in res[1:]:
+        for k, v in res[0][2][0][0].items():
+            np.testing.assert_array_equal(other[2][0][0][k], v, err_msg=k)
+
+
+def test_grouped_weight_gradients_hold_their_slots():
+    """A microbatch whose weight gradients wait for their group keeps its residual slot; join
+    runs what is held back; quiesce refuses while something is."""
+    spec = BERT
+    ex = rt.StageExecutor(spec, 1, 1, 1, False, True, False, wgrad_group=2)
+    buf = rt.DeviceBuffer(spec.tokens * spec.hidden * 2)
+    buf.zero()
+    ex.run_task(TaskType.FWD, 0, 0, buf.ptr, buf.ptr)
+    ex.run_task(TaskType.BWD, 0, 0, buf.ptr, buf.ptr)
+    assert ex.live_slots() == 1                     # held back: microbatch 1 completes the group
+    with pytest.raises(rt.JppError, match="held back for their group"):
+        ex.quiesce()
+    ex.run_task(TaskType.FWD, 0, 1, buf.ptr, buf.ptr)       # the extra slot of the group
+    ex.run_task(TaskType.BWD, 0, 1, buf.ptr, buf.ptr)
+    assert ex.live_slots() == 0
+    ex.run_task(TaskType.FWD, 0, 2, buf.ptr, buf.ptr)
+    ex.run_task(TaskType.BWD, 0, 2, buf.ptr, buf.ptr)
+    assert ex.live_slots() == 1
+    ex.join()
+    assert ex.live_slots() == 0
+    rt.sync()
+    ex.close()
+    with pytest.raises(rt.JppError, match="grouped weight gradients need one stream"):
+        rt.StageExecutor(spec, 1, 1, 1, False, True, True, wgrad_group=2)
 
 
 def test_unfused_accumulate_path_is_close():
