@@ -99,6 +99,13 @@ int jpp_graph_destroy(void* graph_exec);
  *   swiglu_bwd, rope, grad_accum, colsum, adam */
 int jpp_probe_begin(const char* kernel_class);
 int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, double* total_bytes);
+/* With jpp_probe_begin("*") every class is bracketed and jpp_probe_end returns the totals over
+ * all of them; jpp_probe_class then reads class `index` (0, 1, ... until JPP_ERR_INVALID) of
+ * the probe that has just ended: its name (valid until the next jpp_probe_begin) and its own
+ * figures.  Further classes: attn_delta, sum_accum, mse, fill, cast, moe_route, moe_gather,
+ * moe_combine_fwd, moe_bwd_prepare, moe_combine_bwd, moe_router_wgrad. */
+int jpp_probe_class(int index, const char** name, int64_t* launches, double* total_ms,
+                    double* total_flops, double* total_bytes);
 /* No counterpart in the reference: a measurement aid.  TFLOP/s this device sustains on
  * a register-only loop of bf16 MFMAs on every SIMD (shape 32: 32x32x16, 16: 16x16x32;
  * operands all zero, or random and different from one MFMA to the next as in a GEMM).
@@ -195,6 +202,20 @@ typedef struct {
 
 int jpp_attn_fwd(void* stream, const jpp_attn_args* args);
 int jpp_attn_bwd(void* stream, const jpp_attn_args* args);
+
+/* ---- scratch sizes ---------------------------------------------------------
+ * Bytes of the caller-provided scratch buffer an operator needs (under JAX: what the FFI
+ * handler asks the scratch allocator for).  d0, d1, d2 per operator; 0 for an unknown one. */
+typedef enum {
+  JPP_WS_NORM_BWD = 0,         /* jpp_norm_args.partial: d0 = cols */
+  JPP_WS_COLSUM = 1,           /* jpp_colsum_accum(_multi) partial: d0 = cols (summed over the tensors) */
+  JPP_WS_ATTN_DELTA = 2,       /* jpp_attn_args.delta: d0 = batch, d1 = n_heads, d2 = seq */
+  JPP_WS_MSE = 3,              /* jpp_mse_loss partial */
+  JPP_WS_MOE_WORK = 4,         /* jpp_moe_args.work: d0 = tokens, d1 = n_experts */
+  JPP_WS_MOE_ROUTER_WGRAD = 5, /* jpp_moe_router_wgrad partial: d0 = hidden, d1 = n_experts */
+  JPP_WS_SPLIT_WGRAD = 6       /* `parts` of jpp_sum_accum_f32: d0 = n_parts, d1 = rows, d2 = cols */
+} jpp_workspace_op;
+size_t jpp_workspace_bytes(int op, int64_t d0, int64_t d1, int64_t d2);
 
 /* ---- row-wise norms ---------------------------------------------------------
  * x, y, dy, dx: bf16 [rows, cols]; gamma/beta bf16 [cols]; mean/rstd f32

@@ -30,10 +30,20 @@ struct Probe {
   bool active = false;
   std::string cls;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> ring;  // created on demand, reused
+  std::vector<int> ring_class;   // class of the launch a pair brackets
   size_t head = 0, live = 0;     // oldest pair in flight, number in flight
   bool open = false;             // ring[(head + live) % size].first has been recorded
-  int64_t launches = 0;
-  double ms = 0, flops = 0, bytes = 0;
+  int open_class = 0;
+  // per class (one entry unless the probe was opened for every class, "*")
+  struct Stat { std::string name; int64_t launches = 0; double ms = 0, flops = 0, bytes = 0; };
+  std::vector<Stat> stats;
+  int class_id(const char* name) {
+    for (size_t i = 0; i < stats.size(); ++i)
+      if (stats[i].name == name) return (int)i;
+    stats.emplace_back();
+    stats.back().name = name;
+    return (int)stats.size() - 1;
+  }
   hipError_t err = hipSuccess;
   char err_what[96] = "";
 
@@ -50,7 +60,7 @@ struct Probe {
     hipError_t e = hipEventSynchronize(ev.second);
     if (e == hipSuccess) e = hipEventElapsedTime(&t, ev.first, ev.second);
     if (e != hipSuccess) fail(e, "reading a launch's events");
-    else ms += t;
+    else stats[ring_class[head]].ms += t;
     head = (head + 1) % ring.size();
     --live;
   }
@@ -59,7 +69,8 @@ struct Probe {
 
 bool jpp_probe_wants(const char* kernel_class) {
   std::lock_guard<std::mutex> lock(g_probe.mu);
-  return g_probe.active && g_probe.err == hipSuccess && g_probe.cls == kernel_class;
+  return g_probe.active && g_probe.err == hipSuccess &&
+         (g_probe.cls == "*" || g_probe.cls == kernel_class);
 }
 
 // A bracket opened inside another one on the same thread (a launcher that hands over to
@@ -67,7 +78,7 @@ bool jpp_probe_wants(const char* kernel_class) {
 // launch_mu twice from one thread would never return.
 thread_local int t_probe_depth = 0;
 
-void jpp_probe_open(hipStream_t stream) {
+void jpp_probe_open(hipStream_t stream, const char* kernel_class) {
   if (t_probe_depth++ > 0) return;
   g_probe.launch_mu.lock();      // released by jpp_probe_close
   std::lock_guard<std::mutex> lock(g_probe.mu);
@@ -86,9 +97,11 @@ void jpp_probe_open(hipStream_t stream) {
       }
       if (p.head != 0) {         // rotate so that the oldest pair is first again
         std::rotate(p.ring.begin(), p.ring.begin() + p.head, p.ring.end());
+        std::rotate(p.ring_class.begin(), p.ring_class.begin() + p.head, p.ring_class.end());
         p.head = 0;
       }
       p.ring.emplace_back(a, b);
+      p.ring_class.push_back(0);
     } else {
       p.retire_oldest();
     }
@@ -100,6 +113,7 @@ void jpp_probe_open(hipStream_t stream) {
     return;
   }
   p.open = true;
+  p.open_class = p.class_id(kernel_class);
 }
 
 void jpp_probe_close(hipStream_t stream, double flops, double bytes) {
@@ -114,10 +128,12 @@ void jpp_probe_close(hipStream_t stream, double flops, double bytes) {
       if (e != hipSuccess) {
         p.fail(e, "hipEventRecord behind a launch");
       } else {
+        p.ring_class[(p.head + p.live) % p.ring.size()] = p.open_class;
         ++p.live;
-        ++p.launches;
-        p.flops += flops;
-        p.bytes += bytes;
+        Probe::Stat& st = p.stats[p.open_class];
+        ++st.launches;
+        st.flops += flops;
+        st.bytes += bytes;
       }
     }
   }
@@ -257,8 +273,7 @@ int jpp_probe_begin(const char* kernel_class) {
   g_probe.cls = kernel_class;
   g_probe.head = g_probe.live = 0;
   g_probe.open = false;
-  g_probe.launches = 0;
-  g_probe.ms = g_probe.flops = g_probe.bytes = 0;
+  g_probe.stats.clear();
   g_probe.err = hipSuccess;
   g_probe.err_what[0] = 0;
   return JPP_OK;
@@ -270,14 +285,46 @@ int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, doub
   JPP_REQUIRE(p.active, "probe_end: no active probe");
   p.active = false;
   while (p.live) p.retire_oldest();
-  if (launches) *launches = p.launches;
-  if (total_ms) *total_ms = p.ms;
-  if (total_flops) *total_flops = p.flops;
-  if (total_bytes) *total_bytes = p.bytes;
+  int64_t n = 0;
+  double ms = 0, flops = 0, bytes = 0;
+  for (auto& st : p.stats) { n += st.launches; ms += st.ms; flops += st.flops; bytes += st.bytes; }
+  if (launches) *launches = n;
+  if (total_ms) *total_ms = ms;
+  if (total_flops) *total_flops = flops;
+  if (total_bytes) *total_bytes = bytes;
   if (p.err != hipSuccess)
     return jpp_set_error(JPP_ERR_HIP, "probe: %s failed: %s (timings are incomplete)", p.err_what,
                          hipGetErrorString(p.err));
   return JPP_OK;
+}
+int jpp_probe_class(int index, const char** name, int64_t* launches, double* total_ms,
+                    double* total_flops, double* total_bytes) {
+  std::lock_guard<std::mutex> lock(g_probe.mu);
+  Probe& p = g_probe;
+  JPP_REQUIRE(!p.active, "probe_class: the probe is still open");
+  if (index < 0 || index >= (int)p.stats.size())
+    return jpp_set_error(JPP_ERR_INVALID, "probe_class: index %d of %d classes", index,
+                         (int)p.stats.size());
+  const Probe::Stat& st = p.stats[index];
+  if (name) *name = st.name.c_str();
+  if (launches) *launches = st.launches;
+  if (total_ms) *total_ms = st.ms;
+  if (total_flops) *total_flops = st.flops;
+  if (total_bytes) *total_bytes = st.bytes;
+  return JPP_OK;
+}
+size_t jpp_workspace_bytes(int op, int64_t d0, int64_t d1, int64_t d2) {
+  if (d0 < 0 || d1 < 0 || d2 < 0) return 0;
+  switch (op) {
+    case JPP_WS_NORM_BWD: return (size_t)2 * JPP_NORM_PARTIALS * d0 * 4;
+    case JPP_WS_COLSUM: return (size_t)JPP_NORM_PARTIALS * d0 * 4;
+    case JPP_WS_ATTN_DELTA: return (size_t)d0 * d1 * d2 * 4;
+    case JPP_WS_MSE: return (size_t)JPP_NORM_PARTIALS * 4;
+    case JPP_WS_MOE_WORK: return (size_t)2 * ((d0 + 255) / 256) * d1 * 4;
+    case JPP_WS_MOE_ROUTER_WGRAD: return (size_t)64 * d0 * d1 * 4;
+    case JPP_WS_SPLIT_WGRAD: return (size_t)d0 * d1 * d2 * 4;
+    default: return 0;
+  }
 }
 int jpp_mem_info(size_t* free_bytes, size_t* total_bytes) {
   JPP_REQUIRE(free_bytes && total_bytes, "mem_info: null");

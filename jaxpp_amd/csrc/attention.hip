@@ -13,9 +13,8 @@
 //     dV^T[dv,key] += dO^T P        A = dO^T(LDS),  B = P from S registers
 //
 // An accumulator tile enumerates its row index as (reg/4, lane/32, reg%4); the
-// LDS-side operand of the second GEMM is stored with bits 2 and 3 of the
-// contraction index swapped (TileLoader KPERM) so that 8 consecutive
-// accumulator registers form one 16-element MFMA step.
+// LDS-side operand of the second GEMM is read in the same order (slab_frag_tr), so
+// that 8 consecutive accumulator registers form one 16-element MFMA step.
 #include "attention_common.h"
 
 using namespace jpp_attn;
@@ -567,7 +566,10 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
                     (a->causal ? 0.5 : 1.0);
 #define JPP_AB(D_, C_)                                                              \
   do {                                                                              \
-    hipLaunchKernelGGL((attn_delta_kernel<D_>), gdelta, dim3(256), 0, st, p);       \
+    {                                                                               \
+      ProbeScope probe(st, "attn_delta", 0, 4.0 * a->batch * a->seq * a->n_heads * D_); \
+      hipLaunchKernelGGL((attn_delta_kernel<D_>), gdelta, dim3(256), 0, st, p);     \
+    }                                                                               \
     if (int rc = set_smem(attn_bwd_dq_kernel<D_, C_>, 4 * D_ * 128)) return rc;     \
     {                                                                               \
       ProbeScope probe(st, "attn_bwd_dq", fl * 0.4, 0);                             \

@@ -41,7 +41,7 @@ int jpp_set_error(int code, const char* fmt, ...);
 // matches is bracketed by HIP events on its own stream; jpp_probe_end sums the
 // durations and the algorithmic work the launcher declared.
 bool jpp_probe_wants(const char* kernel_class);
-void jpp_probe_open(hipStream_t stream);
+void jpp_probe_open(hipStream_t stream, const char* kernel_class);
 void jpp_probe_close(hipStream_t stream, double flops, double bytes);
 
 struct ProbeScope {
@@ -50,7 +50,7 @@ struct ProbeScope {
   bool on;
   ProbeScope(hipStream_t s, const char* cls, double fl, double by)
       : stream(s), flops(fl), bytes(by), on(jpp_probe_wants(cls)) {
-    if (on) jpp_probe_open(stream);
+    if (on) jpp_probe_open(stream, cls);
   }
   ~ProbeScope() {
     if (on) jpp_probe_close(stream, flops, bytes);
@@ -102,80 +102,6 @@ __device__ __forceinline__ bf16x8 slab_frag(const uint8_t* slab, int row0, int k
   int row = row0 + (lane & 31);
   return *(const bf16x8*)(slab + slab_off(row, kstep * 2 + (lane >> 5)));
 }
-
-// Swap bits 2 and 3 of a contraction index.  An operand built straight from
-// MFMA accumulator registers enumerates its contraction index in the order
-// (reg/4, lane/32, reg%4); storing the LDS-side operand with those two bits
-// swapped makes both sides agree while keeping 16-byte fragment reads.
-__device__ __forceinline__ int swap_bits23(int k) {
-  return (k & ~0xC) | ((k & 4) << 1) | ((k & 8) >> 1);
-}
-
-// Cooperative loader of a (64 x ROWS) or (ROWS x 64) bf16 tile for 256 threads.
-//  TRANS = false: memory holds [ROWS][64..] with the contraction index
-//                 contiguous; a thread moves ROWS/32 16-byte chunks.
-//  TRANS = true : memory holds [64][ROWS..] (contraction index is the slow
-//                 one); a thread reads a (ROWS/32 x 8) block, transposes it in
-//                 registers and writes 8 short runs of contraction elements.
-//  KPERM        : store contraction index k at position swap_bits23(k).
-template <int ROWS, bool TRANS, bool KPERM = false>
-struct TileLoader {
-  static constexpr int NV = ROWS / 32;
-  static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "ROWS");
-  static_assert(!KPERM || (TRANS && NV <= 4), "KPERM needs short transposed runs");
-  typedef uint4 Regs[NV];
-
-  static __device__ __forceinline__ void load(Regs& r, const bf16_t* __restrict__ src, long ld,
-                                              int tid) {
-    if constexpr (!TRANS) {
-#pragma unroll
-      for (int i = 0; i < NV; ++i)
-        r[i] = *(const uint4*)(src + (long)((tid >> 3) + 32 * i) * ld + (tid & 7) * 8);
-    } else {
-      const int rb = tid % (ROWS / 8), kb = tid / (ROWS / 8);
-#pragma unroll
-      for (int j = 0; j < NV; ++j)
-        r[j] = *(const uint4*)(src + (long)(kb * NV + j) * ld + rb * 8);
-    }
-  }
-
-  static __device__ __forceinline__ void store(const Regs& r, uint8_t* slab, int tid) {
-    if constexpr (!TRANS) {
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        int row = (tid >> 3) + 32 * i;
-        *(uint4*)(slab + slab_off(row, tid & 7)) = r[i];
-      }
-    } else {
-      const int rb = tid % (ROWS / 8), kb = tid / (ROWS / 8);
-      int k0 = kb * NV;
-      if constexpr (KPERM) k0 = swap_bits23(k0);
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const int row = rb * 8 + c;
-        uint32_t w[NV];
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-          const uint4 v = r[j];
-          w[j] = (c >> 1) == 0 ? v.x : (c >> 1) == 1 ? v.y : (c >> 1) == 2 ? v.z : v.w;
-        }
-        uint32_t o[NV / 2];
-#pragma unroll
-        for (int q = 0; q < NV / 2; ++q)
-          o[q] = (c & 1) ? ((w[2 * q] >> 16) | (w[2 * q + 1] & 0xffff0000u))
-                         : ((w[2 * q] & 0xffffu) | (w[2 * q + 1] << 16));
-        uint8_t* dst = slab + slab_off(row, k0 >> 3) + (k0 & 7) * 2;
-        if constexpr (NV == 8) {
-          *(uint4*)dst = make_uint4(o[0], o[1], o[2], o[3]);
-        } else if constexpr (NV == 4) {
-          *(uint2*)dst = make_uint2(o[0], o[1]);
-        } else {
-          *(uint32_t*)dst = o[0];
-        }
-      }
-    }
-  }
-};
 
 // ---------------------------------------------------------------------------
 // Direct-to-LDS tiles (global_load_lds_dwordx4): no register staging.

@@ -861,6 +861,7 @@ int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t coun
   hipStream_t st = (hipStream_t)stream;
   const long n8 = count / 8;
   const int nb = (int)(n8 < JPP_NORM_PARTIALS ? n8 : JPP_NORM_PARTIALS);
+  ProbeScope probe(st, "mse", 0, 6.0 * count);
   hipLaunchKernelGGL(mse_partial_kernel, dim3(nb), dim3(256), 0, st, (const bf16_t*)out,
                      (const bf16_t*)target, n8, 2.0f * scale / (float)count, (bf16_t*)dout, partial);
   hipLaunchKernelGGL(mse_final_kernel, dim3(1), dim3(64), 0, st, partial, nb,
@@ -871,6 +872,7 @@ int jpp_mse_loss(void* stream, const void* out, const void* target, int64_t coun
 
 int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t count) {
   JPP_REQUIRE(src && dst && count > 0, "cast: bad arguments");
+  ProbeScope probe((hipStream_t)stream, "cast", 0, 6.0 * count);
   hipLaunchKernelGGL(cast_f32_bf16_kernel, dim3(grid_for(count)), dim3(256), 0,
                      (hipStream_t)stream, src, (bf16_t*)dst, (long)count);
   JPP_LAUNCH_CHECK();
@@ -879,6 +881,7 @@ int jpp_cast_f32_to_bf16(void* stream, const float* src, void* dst, int64_t coun
 
 int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t count) {
   JPP_REQUIRE(src && dst && count > 0, "cast: bad arguments");
+  ProbeScope probe((hipStream_t)stream, "cast", 0, 6.0 * count);
   hipLaunchKernelGGL(cast_bf16_f32_kernel, dim3(grid_for(count)), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)src, dst, (long)count);
   JPP_LAUNCH_CHECK();
@@ -888,6 +891,7 @@ int jpp_cast_bf16_to_f32(void* stream, const void* src, float* dst, int64_t coun
 int jpp_fill_u32(void* dst, uint32_t value, size_t count, void* stream) {
   JPP_REQUIRE(dst || count == 0, "fill: null destination");
   if (count == 0) return JPP_OK;
+  ProbeScope probe((hipStream_t)stream, "fill", 0, 4.0 * count);
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for((long)count)), dim3(256), 0,
                      (hipStream_t)stream, (uint32_t*)dst, value, (long)count);
   JPP_LAUNCH_CHECK();

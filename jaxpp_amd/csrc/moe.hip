@@ -343,6 +343,7 @@ int jpp_moe_route(void* stream, const jpp_moe_args* a) {
   JPP_REQUIRE(a->dtype == JPP_DTYPE_BF16 || a->dtype == JPP_DTYPE_F32, "moe_route: unknown dtype %d",
               a->dtype);
   hipStream_t st = (hipStream_t)stream;
+  ProbeScope probe(st, "moe_route", 0, (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden);   // reads x once
   const long T = a->tokens;
   const int nblk = (int)((T + 255) / 256);
   int* cnt = (int*)a->work;
@@ -367,6 +368,7 @@ int jpp_moe_route(void* stream, const jpp_moe_args* a) {
 int jpp_moe_gather(void* stream, const jpp_moe_args* a, const void* x, void* xp) {
   JPP_REQUIRE(a && x && xp, "moe_gather: null operand");
   const long cap = jpp_moe_capacity(a->tokens, kE, 2);
+  ProbeScope probe((hipStream_t)stream, "moe_gather", 0, 2 * (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->top_k * a->hidden);
   if (a->dtype == JPP_DTYPE_F32) {
     hipLaunchKernelGGL(gather_kernel<float>, dim3(grid_for(cap * (a->hidden / 8))), dim3(256), 0,
                        (hipStream_t)stream, (const float*)x, a->tok_of, a->seg, (int)a->hidden,
@@ -383,6 +385,8 @@ int jpp_moe_gather(void* stream, const jpp_moe_args* a, const void* x, void* xp)
 int jpp_moe_combine_fwd(void* stream, const jpp_moe_args* a, const void* eo, const void* resid,
                         void* y) {
   JPP_REQUIRE(a && eo && resid && y, "moe_combine_fwd: null operand");
+  ProbeScope probe((hipStream_t)stream, "moe_combine_fwd", 0,
+                   (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden * (a->top_k + 2));   // top_k rows + residual in, y out
   if (a->dtype == JPP_DTYPE_F32) {
     hipLaunchKernelGGL(combine_fwd_kernel<float>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
                        (hipStream_t)stream, (const float*)eo, a->row_of, a->gates,
@@ -400,6 +404,8 @@ int jpp_moe_bwd_prepare(void* stream, const jpp_moe_args* a, const void* dy, con
                         float* dlogits, void* deo) {
   JPP_REQUIRE(a && dy && eo && dlogits && deo, "moe_bwd_prepare: null operand");
   hipStream_t st = (hipStream_t)stream;
+  // gate gradients read dy and top_k rows of eo; the scatter reads dy again per copy, writes deo
+  ProbeScope probe(st, "moe_bwd_prepare", 0, (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden * (1 + 3 * a->top_k));
   const long cap = jpp_moe_capacity(a->tokens, kE, 2);
   if (a->dtype == JPP_DTYPE_F32) {
     hipLaunchKernelGGL(gate_bwd_kernel<float>, dim3((unsigned)((a->tokens + 3) / 4)), dim3(256), 0, st,
@@ -426,6 +432,8 @@ int jpp_moe_bwd_prepare(void* stream, const jpp_moe_args* a, const void* dy, con
 int jpp_moe_combine_bwd(void* stream, const jpp_moe_args* a, const void* dxp,
                         const float* dlogits, void* dx) {
   JPP_REQUIRE(a && dxp && dlogits && dx, "moe_combine_bwd: null operand");
+  ProbeScope probe((hipStream_t)stream, "moe_combine_bwd", 0,
+                   (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden * (a->top_k + 1));
   if (a->dtype == JPP_DTYPE_F32) {
     hipLaunchKernelGGL(combine_bwd_kernel<float>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
                        (hipStream_t)stream, (const float*)dxp, a->row_of, dlogits,
@@ -443,6 +451,7 @@ int jpp_moe_router_wgrad(void* stream, const jpp_moe_args* a, const void* x, con
                          float* acc, float* partial) {
   JPP_REQUIRE(a && x && dlogits && acc && partial, "moe_router_wgrad: null operand");
   hipStream_t st = (hipStream_t)stream;
+  ProbeScope probe(st, "moe_router_wgrad", 0, (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden);
   const int nb = 64;
   if (a->dtype == JPP_DTYPE_F32) {
     hipLaunchKernelGGL(wr_partial_kernel<float>, dim3(nb, (unsigned)((a->hidden + 255) / 256)), dim3(256), 0,

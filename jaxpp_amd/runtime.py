@@ -104,8 +104,8 @@ EXPORTS = [
     "jpp_stream_create", "jpp_stream_destroy", "jpp_stream_sync", "jpp_stream_wait_event",
     "jpp_device_sync",
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
-    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_graph_begin", "jpp_graph_end", "jpp_graph_launch",
-    "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_mfma_rate",
+    "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_workspace_bytes", "jpp_graph_begin", "jpp_graph_end", "jpp_graph_launch",
+    "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_probe_class", "jpp_mfma_rate",
     "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_gemm_f32", "jpp_attn_fwd_f32", "jpp_attn_bwd_f32", "jpp_norm_fwd_f32", "jpp_norm_bwd_f32",
     "jpp_colsum_accum_f32", "jpp_mse_loss_f32", "jpp_rope_f32",
@@ -137,6 +137,8 @@ def load():
             "(there is no fallback path)")
     lib = C.CDLL(_LIB_PATH)
     lib.jpp_last_error.restype = C.c_char_p
+    lib.jpp_workspace_bytes.restype = C.c_size_t
+    lib.jpp_workspace_bytes.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64]
     lib.jpp_stage_bytes.restype = C.c_size_t
     lib.jpp_stage_bytes.argtypes = [C.c_void_p]
     lib.jpp_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
@@ -162,6 +164,9 @@ def load():
     lib.jpp_probe_begin.argtypes = [C.c_char_p]
     lib.jpp_probe_end.argtypes = [C.POINTER(C.c_int64), C.POINTER(C.c_double),
                                   C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    lib.jpp_probe_class.argtypes = [C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_int64),
+                                    C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                    C.POINTER(C.c_double)]
     lib.jpp_gemm_bf16.argtypes = [C.c_void_p, C.POINTER(GemmArgs)]
     lib.jpp_attn_fwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
@@ -434,6 +439,16 @@ class probe:
         n, ms, fl, by = C.c_int64(), C.c_double(), C.c_double(), C.c_double()
         check(load().jpp_probe_end(C.byref(n), C.byref(ms), C.byref(fl), C.byref(by)))
         self.launches, self.total_ms, self.flops, self.bytes = n.value, ms.value, fl.value, by.value
+        # per class: {name: (launches, total ms, flops, bytes)}; one entry unless the class is "*"
+        self.classes = {}
+        i = 0
+        while True:
+            name = C.c_char_p()
+            if load().jpp_probe_class(i, C.byref(name), C.byref(n), C.byref(ms), C.byref(fl),
+                                      C.byref(by)) != 0:
+                break
+            self.classes[name.value.decode()] = (n.value, ms.value, fl.value, by.value)
+            i += 1
         return False
 
 

@@ -40,6 +40,19 @@ def test_error_convention_without_gpu():
     assert lib.jpp_stage_adam_step(None, None, 1, 0.0, 0.0, 0.0, 0.0, 0.0) == -1
 
 
+def test_workspace_sizes():
+    """jpp_workspace_bytes: what the tests allocate by hand for each operator's scratch."""
+    lib = rt.load()
+    assert lib.jpp_workspace_bytes(0, 8192, 0, 0) == 2 * rt.NORM_PARTIALS * 8192 * 4     # norm backward
+    assert lib.jpp_workspace_bytes(1, 1024 + 4096, 0, 0) == rt.NORM_PARTIALS * 5120 * 4  # column sums
+    assert lib.jpp_workspace_bytes(2, 2, 32, 4096) == 2 * 32 * 4096 * 4                  # attention delta
+    assert lib.jpp_workspace_bytes(3, 0, 0, 0) == rt.NORM_PARTIALS * 4
+    assert lib.jpp_workspace_bytes(4, 8192, 8, 0) == 2 * 32 * 8 * 4
+    assert lib.jpp_workspace_bytes(5, 4096, 8, 0) == 64 * 4096 * 8 * 4
+    assert lib.jpp_workspace_bytes(6, 4, 1024, 1024) == 4 * 1024 * 1024 * 4
+    assert lib.jpp_workspace_bytes(99, 1, 1, 1) == 0 and lib.jpp_workspace_bytes(0, -1, 0, 0) == 0
+
+
 def test_struct_layouts_match_header_sizes():
     # 7 pointers + 9 int64 + 5 int (+ padding) ; guards against field drift
     assert ctypes.sizeof(rt.GemmArgs) == 7 * 8 + 9 * 8 + 5 * 4 + 4 + 8 + 2 * 4 + 3 * 8 + 8 + 6 * 8 + 8
