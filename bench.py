@@ -118,8 +118,11 @@ class Workbench:
 
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size)
-MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8"): 1.005e9}
+# (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size), keyed by
+# (workload, kernel class, microbatches per weight-gradient launch): a launch over four
+# microbatches reads four operand pairs and the accumulator once
+MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8", 4): 2.879e9,
+                    ("cfg3", "gemm_tn_accf32_256x256w8", 1): 1.005e9}
 
 
 def dominant_gemm_class(wl) -> str:
@@ -328,7 +331,7 @@ def main():
             "peak": (HBM_PEAK / 1e9) if hbm else (MFMA_BF16_PEAK / 1e12),
             "unit": "GB/s" if hbm else "TFLOP/s",
             "frac": ach / (HBM_PEAK if hbm else MFMA_BF16_PEAK),
-            "traffic": MEASURED_TRAFFIC.get((wl.name, cls)),
+            "traffic": MEASURED_TRAFFIC.get((wl.name, cls, max(group, 1))),
             "launches": pr.launches, "avg_launch_ms": avg_ms,
             "algorithmic_per_launch": (pr.bytes if hbm else pr.flops) / pr.launches,
         }

@@ -57,7 +57,10 @@ GEMM_CASES = [  # (trans_a, trans_b, epilogue)
                                         (0, 768, 256, 128),
                                         # 384 tiles of 256x256: the half-filled second round runs as
                                         # a launch of 128x256 tiles over the last columns / rows
-                                        (0, 4096, 6144, 128), (0, 6144, 4096, 192)])
+                                        (0, 4096, 6144, 128), (0, 6144, 4096, 192),
+                                        # two rounds of 256x256 tiles and more, the second
+                                        # with a 128x256 launch for the last half round
+                                        (0, 4096, 8192, 128), (0, 8192, 5120, 192)])
 def test_gemm(ta, tb, epi, tile, m, n, k):
     print(f"gemm ta={ta} tb={tb} epi={epi} tile={tile} {m}x{n}x{k}", flush=True)
     rng = np.random.default_rng(m + n + k + 7 * epi)
@@ -108,7 +111,8 @@ def test_gemm(ta, tb, epi, tile, m, n, k):
 
 
 @pytest.mark.parametrize("parts,m,n,k,tile", [(2, 256, 512, 192, 4), (4, 512, 256, 640, 4), (3, 1024, 768, 1024, 3),
-                                              (4, 4096, 3072, 512, 0), (2, 4096, 6144, 2048, 0)])
+                                              (4, 4096, 3072, 512, 0), (2, 4096, 6144, 2048, 0),
+                                              (2, 8192, 4096, 256, 0)])   # two rounds of tiles
 def test_gemm_contraction_over_several_operand_pairs(parts, m, n, k, tile):
     """C += sum_i A_i^T B_i in one launch (the weight gradients of several microbatches):
     against numpy on the concatenated operands, and bit-identical to ... nothing else: the
@@ -463,7 +467,8 @@ def test_grouped_gemm():
                                         (3, 384, 256, 128),
                                         # split into 256x256 + 128x256 launches: the forward at
                                         # f = 3072 (N = 6144), the backward at f = 6144
-                                        (0, 4096, 3072, 128), (0, 4096, 6144, 64)])
+                                        (0, 4096, 3072, 128), (0, 4096, 6144, 64),
+                                        (0, 8192, 4096, 128)])   # several rounds of tiles
 def test_gemm_swiglu_epilogues(tile, m, f, k):
     rng = np.random.default_rng(21)
     x = rnd(rng, m, k)
