@@ -121,8 +121,9 @@ class Workbench:
 # (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size), keyed by
 # (workload, kernel class, microbatches per weight-gradient launch): a launch over four
 # microbatches reads four operand pairs and the accumulator once
-MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8", 4): 2.879e9,
-                    ("cfg3", "gemm_tn_accf32_256x256w8", 1): 1.005e9}
+MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8_multi", 4): 1.3344e10,  # a layer per launch
+                    ("cfg3", "gemm_tn_accf32_256x256w8", 4): 2.879e9,
+                    ("cfg3", "gemm_tn_accf32_256x256w8", 1): 1.005e9}  # one weight per launch
 
 
 def dominant_gemm_class(wl) -> str:
@@ -131,6 +132,17 @@ def dominant_gemm_class(wl) -> str:
     # (narrow layers: 128x128 tiles, at most two per CU, so the 3-stage variant)
     big = wl.layer.hidden >= 4096
     return "gemm_tn_accf32_256x256w8" if big else "gemm_tn_accf32_128x128w8s3"
+
+
+def measured_dominant_class(wb, wl) -> str:
+    """The weight-gradient class that takes the most time in one (untimed) step with every
+    class probed: which launches the stage uses - per weight, or a layer's weight gradients as
+    one grid - follows from the shapes, so it is read off rather than restated here."""
+    with rt.probe("*") as pr:
+        wb.step()
+        rt.sync()
+    acc = {k: v[1] for k, v in pr.classes.items() if k.startswith("gemm_tn_accf32")}
+    return max(acc, key=acc.get) if acc else dominant_gemm_class(wl)
 
 
 def default_wgrad_group(wl, two_streams: bool) -> int:
@@ -246,7 +258,6 @@ def main():
     if args.unfused_accumulate or two:
         group = 1
     wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two, wgrad_group=group)
-    cls = args.probe or dominant_gemm_class(wl)
     if args.kernel_table:
         print(json.dumps(kernel_table(wb, wl, args.steps, args.warmup, two, group)))
         return
@@ -265,6 +276,7 @@ def main():
         ev.record()
         ends.append(ev)
 
+    cls = args.probe or (measured_dominant_class(wb, wl) if args.warmup else dominant_gemm_class(wl))
     for _ in range(args.warmup):
         paced_step()
     rt.sync()

@@ -184,6 +184,18 @@ enum { JPP_GROUP_NONE = 0, JPP_GROUP_M = 1, JPP_GROUP_K = 2 };
 
 int jpp_gemm_bf16(void* stream, const jpp_gemm_args* args);
 
+/* Up to four independent accumulated weight gradients - every problem with trans_a = trans_b =
+ * 1, JPP_EPI_ACC_F32, no groups, M and N multiples of 256, the same k and k_parts - as ONE
+ * grid of 256x256 tiles, problem after problem.  Stands where the reference's weight-gradient
+ * task holds several independent dot_generals (one per parameter of the layer,
+ * src/jaxpp/jaxpr_utils.py:138-167 puts them all into BWD_W): launched one by one, each leaves
+ * its last round of tiles partly empty (a 6144 x 4096 gradient is 384 tiles on 256 CUs);
+ * together they close up.  Every output element is computed by one workgroup in a fixed order
+ * (deterministic), the same order as in a single launch on 256x256 tiles; a single launch that
+ * runs its last round on 128x256 tiles adds the old accumulator value at another point of the
+ * sum there, so the two agree to fp32 rounding.  n_problems = 1 is jpp_gemm_bf16. */
+int jpp_gemm_bf16_multi(void* stream, const jpp_gemm_args* problems, int n_problems);
+
 /* ---- fused attention (softmax(QK^T/sqrt(d)) V), forward and backward -------
  * q: [batch*seq, *] with head h at columns h*head_dim (row stride ldq); k, v
  * likewise with n_kv_heads heads; query head h reads kv head h / (n_heads /

@@ -21,6 +21,7 @@
 // 32x32x16 shape (2.03 against 1.82 PFLOP/s in a register-only loop; jpp_mfma_rate).
 #include <math.h>
 #include <stdio.h>
+#include <string.h>
 
 #include <mutex>
 #include <string>
@@ -54,6 +55,27 @@ struct GemmParams {
   int n_seg, group_mode;
   int64_t group_rows;
   long stride_b, stride_c;
+};
+
+// One more problem of a launch that covers several independent products of one kind (same
+// orientations, epilogue, contraction length and number of operand pairs): its operands and
+// its place in the grid.  Workgroups first .. first + tiles_m tiles_n - 1 work on it.
+struct GemmProblem {
+  const bf16_t* a[4];
+  const bf16_t* b[4];
+  void* c;
+  long lda, ldb, ldc;
+  int tiles_m, tiles_n, first;
+};
+// kernel arguments: one problem, or (MP) up to four
+template <bool MP>
+struct GemmArgs {
+  GemmParams p;
+};
+template <>
+struct GemmArgs<true> {
+  GemmParams p;          // problem 0 and everything the problems share
+  GemmProblem more[3];   // problems 1..3; `first` past the grid for those not in use
 };
 
 __device__ __forceinline__ float gelu_f(float u, int tanh_form) {
@@ -128,8 +150,34 @@ __device__ __forceinline__ const bf16_t* part_ptr(const bf16_t* p0, const bf16_t
   return base + (long)(kt - part * kt_part) * step;
 }
 
-template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS, bool KP = false>
-__global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
+template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS, bool KP = false, bool MP = false>
+__global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
+  GemmParams p = args.p;
+  int bid = blockIdx.x;  // this workgroup's tile within its problem
+  if constexpr (MP) {
+    // which problem this workgroup belongs to (wave-uniform: scalar compares and selects,
+    // field by field - never an index into the kernel arguments)
+    const bool s1 = bid >= args.more[0].first, s2 = bid >= args.more[1].first,
+               s3 = bid >= args.more[2].first;
+#define JPP_PICK(own, field) \
+  (s3 ? args.more[2].field : s2 ? args.more[1].field : s1 ? args.more[0].field : (own))
+    p.a = JPP_PICK(p.a, a[0]);
+    p.b = JPP_PICK(p.b, b[0]);
+    p.a_more[0] = JPP_PICK(p.a_more[0], a[1]);
+    p.a_more[1] = JPP_PICK(p.a_more[1], a[2]);
+    p.a_more[2] = JPP_PICK(p.a_more[2], a[3]);
+    p.b_more[0] = JPP_PICK(p.b_more[0], b[1]);
+    p.b_more[1] = JPP_PICK(p.b_more[1], b[2]);
+    p.b_more[2] = JPP_PICK(p.b_more[2], b[3]);
+    p.c = JPP_PICK(p.c, c);
+    p.lda = JPP_PICK(p.lda, lda);
+    p.ldb = JPP_PICK(p.ldb, ldb);
+    p.ldc = JPP_PICK(p.ldc, ldc);
+    p.tiles_m = JPP_PICK(p.tiles_m, tiles_m);
+    p.tiles_n = JPP_PICK(p.tiles_n, tiles_n);
+    bid -= JPP_PICK(0, first);
+#undef JPP_PICK
+  }
   using TileA = DmaTile<BM, TA, NW>;
   using TileB = DmaTile<BN, TB, NW>;
   constexpr int A_BYTES = TileA::BYTES, STAGE = TileA::BYTES + TileB::BYTES;
@@ -145,8 +193,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
   const int wm = wave / WN, wn = wave % WN;
   int tm, tn;
   const int tiles = p.tiles_m * p.tiles_n;
-  tile_of_block(p.group_mode == JPP_GROUP_K ? (int)blockIdx.x % tiles : (int)blockIdx.x, p.tiles_m,
-                p.tiles_n, tm, tn);
+  tile_of_block(p.group_mode == JPP_GROUP_K ? bid % tiles : bid, p.tiles_m, p.tiles_n, tm, tn);
   const long m0 = (long)tm * BM, n0 = (long)tn * BN;
 
   const long a_off = TA ? m0 : m0 * p.lda, b_off = TB ? n0 : n0 * p.ldb;
@@ -161,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmParams p) {
     b_src += (long)e * p.stride_b;
   } else if (p.group_mode == JPP_GROUP_K) {
     // one output per expert; the contraction runs over the expert's rows
-    const int e = blockIdx.x / tiles;
+    const int e = bid / tiles;
     const long r0 = p.seg[e];
     // rows past the group's data are zero padding: steps made of nothing else are skipped
     const int rows = p.seg_rows ? min(p.seg_rows[e], p.seg[e + 1] - p.seg[e]) : p.seg[e + 1] - p.seg[e];
@@ -584,7 +631,54 @@ int launch(hipStream_t stream, GemmParams& p) {
   p.tiles_m = p.m / BM;
   p.tiles_n = p.n / BN;
   const int blocks = p.tiles_m * p.tiles_n * (p.group_mode == JPP_GROUP_K ? p.n_seg : 1);
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(NW * 64), SMEM, stream, p);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(NW * 64), SMEM, stream, GemmArgs<false>{p});
+  JPP_LAUNCH_CHECK();
+  return JPP_OK;
+}
+
+// Several accumulated weight gradients (C_i += sum_j A_ij^T B_ij) as one grid of 256x256
+// tiles: problem i's tiles follow problem i-1's, so the half-filled last rounds of the single
+// launches (384 or 896 tiles on 256 CUs) close up - the four weight gradients of a
+// Llama-3-8B-shaped layer are 13 full rounds together.
+int launch_multi(hipStream_t stream, GemmParams* ps, int n) {
+  constexpr int BM = 256, BN = 256, NW = 8, NS = 2;
+  constexpr int SMEM = NS * (BM + BN) * 128 + (NS + 1) * NW * (1024 + 16);
+  GemmArgs<true> args;
+  args.p = ps[0];
+  int first = 0;
+  double flops = 0, bytes = 0;
+  for (int i = 0; i < n; ++i) {
+    GemmParams& p = ps[i];
+    p.tiles_m = p.m / BM;
+    p.tiles_n = p.n / BN;
+    const double ak = (double)p.k * p.k_parts;
+    flops += 2.0 * p.m * p.n * ak;
+    bytes += 2.0 * ak * (p.m + p.n) + 8.0 * p.m * p.n;
+    if (i > 0) {
+      GemmProblem& q = args.more[i - 1];
+      q.a[0] = p.a; q.b[0] = p.b;
+      for (int j = 0; j < 3; ++j) { q.a[j + 1] = p.a_more[j]; q.b[j + 1] = p.b_more[j]; }
+      q.c = p.c; q.lda = p.lda; q.ldb = p.ldb; q.ldc = p.ldc;
+      q.tiles_m = p.tiles_m; q.tiles_n = p.tiles_n; q.first = first;
+    }
+    first += p.tiles_m * p.tiles_n;
+  }
+  args.p.tiles_m = ps[0].tiles_m;
+  args.p.tiles_n = ps[0].tiles_n;
+  for (int i = n; i < 4; ++i) {
+    memset(&args.more[i - 1], 0, sizeof(GemmProblem));
+    args.more[i - 1].first = 0x7fffffff;
+  }
+  ProbeScope probe(stream, "gemm_tn_accf32_256x256w8_multi", flops, bytes);
+  auto kern = gemm_kernel<BM, BN, true, true, JPP_EPI_ACC_F32, NW, NS, true, true>;
+  static std::once_flag configured;
+  static hipError_t configure_rc = hipSuccess;
+  std::call_once(configured, [&] {
+    configure_rc = hipFuncSetAttribute((const void*)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+  });
+  JPP_CHECK_HIP(configure_rc);
+  hipLaunchKernelGGL(kern, dim3(first), dim3(NW * 64), SMEM, stream, args);
   JPP_LAUNCH_CHECK();
   return JPP_OK;
 }
@@ -662,10 +756,8 @@ int dispatch(hipStream_t stream, const jpp_gemm_args* a, GemmParams& p, int tile
                        ta, tb, e);
 }
 
-}  // namespace
-
-extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
-  hipStream_t stream = (hipStream_t)stream_;
+// checks one problem's arguments and fills the kernel's view of it
+int prepare(const jpp_gemm_args* a, GemmParams& p) {
   JPP_REQUIRE(a && a->a && a->b && a->c, "gemm: null operand");
   const bool group_k = a->group_mode == JPP_GROUP_K;
   JPP_REQUIRE(a->m > 0 && a->n > 0 && (a->k > 0 || group_k), "gemm: empty problem %ldx%ldx%ld",
@@ -682,7 +774,6 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   JPP_REQUIRE(((uintptr_t)a->a | (uintptr_t)a->b | (uintptr_t)a->c) % 16 == 0,
               "gemm: operands must be 16-byte aligned");
   JPP_REQUIRE(a->m < (1L << 31) && a->n < (1L << 31) && a->k < (1L << 31), "gemm: too large");
-  GemmParams p;
   p.a = (const bf16_t*)a->a;
   p.b = (const bf16_t*)a->b;
   p.c = a->c;
@@ -736,6 +827,15 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     JPP_REQUIRE((double)a->m * a->ldc * 4 < 4294967296.0,
                 "gemm: an accumulated output must span less than 4 GiB (32-bit offsets)");
   if (a->resid) JPP_REQUIRE(a->ldresid >= a->n && a->ldresid % 4 == 0, "gemm: bad ldresid");
+  return JPP_OK;
+}
+
+}  // namespace
+
+extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GemmParams p;
+  if (int rc = prepare(a, p)) return rc;
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
   // row groups come in 256-row segments; a contraction split into groups takes any tile
   if (a->group_mode == JPP_GROUP_M || (a->group_mode == JPP_GROUP_K && !a->tile)) tile = 4;
@@ -769,4 +869,28 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     }
   }
   return dispatch(stream, a, p, tile);
+}
+
+extern "C" int jpp_gemm_bf16_multi(void* stream_, const jpp_gemm_args* problems, int n_problems) {
+  hipStream_t stream = (hipStream_t)stream_;
+  JPP_REQUIRE(problems && n_problems >= 1 && n_problems <= 4, "gemm_multi: 1 to 4 problems");
+  if (n_problems == 1) return jpp_gemm_bf16(stream_, problems);
+  GemmParams ps[4];
+  long tiles = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    const jpp_gemm_args* a = problems + i;
+    if (int rc = prepare(a, ps[i])) return rc;
+    JPP_REQUIRE(a->trans_a && a->trans_b && a->epilogue == JPP_EPI_ACC_F32 &&
+                    a->group_mode == JPP_GROUP_NONE && !a->bias && !a->resid && !a->tile,
+                "gemm_multi: problem %d is not a plain accumulated weight gradient (trans_a = "
+                "trans_b = 1, JPP_EPI_ACC_F32, no groups, bias, residual or tile choice)", i);
+    JPP_REQUIRE(a->m % 256 == 0 && a->n % 256 == 0,
+                "gemm_multi: problem %d: M and N must be multiples of 256, got %ldx%ld", i,
+                (long)a->m, (long)a->n);
+    JPP_REQUIRE(a->k == problems[0].k && ps[i].k_parts == ps[0].k_parts,
+                "gemm_multi: problem %d differs from problem 0 in k or k_parts", i);
+    tiles += (a->m / 256) * (a->n / 256);
+  }
+  JPP_REQUIRE(tiles < (1L << 30), "gemm_multi: too many tiles");
+  return launch_multi(stream, ps, n_problems);
 }

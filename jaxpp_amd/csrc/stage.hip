@@ -254,6 +254,60 @@ int wgrad_n(jpp_stage* s, hipStream_t st, int n, const void* const* xs, int64_t 
   return jpp_gemm_bf16(st, &g);
 }
 
+// The dense weight gradients of one layer, gathered so that they can leave as one launch.
+struct WgradBatch {
+  jpp_gemm_args g[4];
+  int n = 0;
+  void add(jpp_stage* s, int pairs, const void* const* xs, int64_t ldx, const void* const* dys,
+           int64_t lddy, float* acc, int64_t rows, int64_t cols) {
+    jpp_gemm_args& q = g[n++];
+    memset(&q, 0, sizeof(q));
+    q.a = xs[0]; q.b = dys[0]; q.c = acc; q.m = rows; q.n = cols; q.k = s->T;
+    q.lda = ldx; q.ldb = lddy; q.ldc = cols; q.trans_a = 1; q.trans_b = 1;
+    q.epilogue = JPP_EPI_ACC_F32;
+    q.k_parts = pairs;
+    for (int i = 1; i < pairs; ++i) { q.a_more[i - 1] = xs[i]; q.b_more[i - 1] = dys[i]; }
+  }
+  void add1(jpp_stage* s, const void* x, int64_t ldx, const void* dy, int64_t lddy, float* acc,
+            int64_t rows, int64_t cols) {
+    add(s, 1, &x, ldx, &dy, lddy, acc, rows, cols);
+  }
+};
+
+// Runs a layer's gathered weight gradients: as one grid of 256x256 tiles when that takes
+// fewer rounds of the 256 CUs than the launches one by one (whose last rounds stay partly
+// empty: a round of 128x256 tiles for a rest of at most 128 tiles costs about 0.77 of a full
+// one), else one by one.  Which way is taken depends on the shapes only.
+int run_wgrads(jpp_stage* s, hipStream_t st, WgradBatch& w) {
+  bool multi = w.n >= 2 && !s->f32() && s->d.fused_wgrad_accum;
+  long total = 0;
+  double apart = 0;
+  for (int i = 0; i < w.n && multi; ++i) {
+    const jpp_gemm_args& q = w.g[i];
+    if (q.m % 256 || q.n % 256) { multi = false; break; }
+    const long t = (q.m / 256) * (q.n / 256), rest = t % 256;
+    total += t;
+    apart += (double)(t / 256) + (rest == 0 ? 0.0 : (rest <= 128 && t > 256 ? 0.77 : 1.0));
+  }
+  if (multi && (double)((total + 255) / 256) < apart - 0.25) {
+    // smallest first: measured 1 % faster than largest first at the Llama-3-8B shapes
+    jpp_gemm_args order[4];
+    for (int i = 0; i < w.n; ++i) order[i] = w.g[i];
+    std::stable_sort(order, order + w.n, [](const jpp_gemm_args& a, const jpp_gemm_args& b) {
+      return a.m * a.n < b.m * b.n;
+    });
+    return jpp_gemm_bf16_multi(st, order, w.n);
+  }
+  for (int i = 0; i < w.n; ++i) {
+    const jpp_gemm_args& q = w.g[i];
+    const int pairs = q.k_parts > 1 ? q.k_parts : 1;
+    const void* xs[4] = {q.a, q.a_more[0], q.a_more[1], q.a_more[2]};
+    const void* dys[4] = {q.b, q.b_more[0], q.b_more[1], q.b_more[2]};
+    RC(wgrad_n(s, st, pairs, xs, q.lda, dys, q.ldb, (float*)q.c, q.m, q.n));
+  }
+  return JPP_OK;
+}
+
 int norm_f(jpp_stage* s, hipStream_t st, const void* x, const void* gamma, const void* beta,
            void* y, float* mean, float* rstd) {
   jpp_norm_args a;
@@ -485,19 +539,20 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
   const int64_t h = s->h, f = s->f;
   auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
   auto wt = [&](const Buf& b) { return (void*)(wbase + b.off); };
+  WgradBatch wb;
   if (s->d.family == JPP_FAMILY_BERT) {
-    RC(wgrad(s, st, at(L.g), f, wt(W.dc), h, s->G(chunk, li, B_W2), f, h));
-    RC(wgrad(s, st, at(L.x1), h, wt(W.du), f, s->G(chunk, li, B_W1), h, f));
-    RC(wgrad(s, st, at(L.ctx), h, wt(W.da), h, s->G(chunk, li, B_Wo), h, h));
-    RC(wgrad(s, st, at(L.x), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
-    return JPP_OK;
+    wb.add1(s, at(L.g), f, wt(W.dc), h, s->G(chunk, li, B_W2), f, h);
+    wb.add1(s, at(L.x1), h, wt(W.du), f, s->G(chunk, li, B_W1), h, f);
+    wb.add1(s, at(L.ctx), h, wt(W.da), h, s->G(chunk, li, B_Wo), h, h);
+    wb.add1(s, at(L.x), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h);
+    return run_wgrads(s, st, wb);
   }
   if (s->d.family == JPP_FAMILY_DECODER) {
-    RC(wgrad(s, st, at(L.g), f, dy, h, s->G(chunk, li, B_W2), f, h));
-    RC(wgrad(s, st, at(L.n2), h, wt(W.du), f, s->G(chunk, li, B_W1), h, f));
-    RC(wgrad(s, st, at(L.ctx), h, wt(W.dh1), h, s->G(chunk, li, B_Wo), h, h));
-    RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
-    return JPP_OK;
+    wb.add1(s, at(L.g), f, dy, h, s->G(chunk, li, B_W2), f, h);
+    wb.add1(s, at(L.n2), h, wt(W.du), f, s->G(chunk, li, B_W1), h, f);
+    wb.add1(s, at(L.ctx), h, wt(W.dh1), h, s->G(chunk, li, B_Wo), h, h);
+    wb.add1(s, at(L.n1), h, wt(W.dqkv), 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h);
+    return run_wgrads(s, st, wb);
   }
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
     jpp_moe_args ma;
@@ -509,15 +564,15 @@ int layer_bwd_w(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
              s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
     RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)wt(W.dlogits), s->G(chunk, li, X_Wr),
                             partial));
-    RC(wgrad(s, st, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, X_Wo), s->ctxw, h));
-    RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw));
-    return JPP_OK;
+    wb.add1(s, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, X_Wo), s->ctxw, h);
+    wb.add1(s, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw);
+    return run_wgrads(s, st, wb);
   }
-  RC(wgrad(s, st, at(L.s), f, dy, h, s->G(chunk, li, L_Wd), f, h));
-  RC(wgrad(s, st, at(L.n2), h, wt(W.dgu), 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f));
-  RC(wgrad(s, st, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, L_Wo), s->ctxw, h));
-  RC(wgrad(s, st, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, L_Wqkv), h, s->qkvw));
-  return JPP_OK;
+  wb.add1(s, at(L.s), f, dy, h, s->G(chunk, li, L_Wd), f, h);
+  wb.add1(s, at(L.n2), h, wt(W.dgu), 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f);
+  wb.add1(s, at(L.ctx), s->ctxw, wt(W.dh1), h, s->G(chunk, li, L_Wo), s->ctxw, h);
+  wb.add1(s, at(L.n1), h, wt(W.dqkv), s->qkvw, s->G(chunk, li, L_Wqkv), h, s->qkvw);
+  return run_wgrads(s, st, wb);
 }
 
 // Weight-gradient half of layer li for n microbatches of one chunk at once (their residuals
@@ -532,19 +587,20 @@ int layer_bwd_w_group(jpp_stage* s, hipStream_t st, int chunk, int li, int n, ui
   auto gather = [&](const Buf& x, const Buf& dy) {
     for (int i = 0; i < n; ++i) { xs[i] = slots[i] + x.off; dys[i] = slots[i] + dy.off; }
   };
+  WgradBatch wb;
   if (s->d.family == JPP_FAMILY_BERT) {
-    gather(L.g, L.dc);   RC(wgrad_n(s, st, n, xs, f, dys, h, s->G(chunk, li, B_W2), f, h));
-    gather(L.x1, L.du);  RC(wgrad_n(s, st, n, xs, h, dys, f, s->G(chunk, li, B_W1), h, f));
-    gather(L.ctx, L.da); RC(wgrad_n(s, st, n, xs, h, dys, h, s->G(chunk, li, B_Wo), h, h));
-    gather(L.x, L.dqkv); RC(wgrad_n(s, st, n, xs, h, dys, 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
-    return JPP_OK;
+    gather(L.g, L.dc);   wb.add(s, n, xs, f, dys, h, s->G(chunk, li, B_W2), f, h);
+    gather(L.x1, L.du);  wb.add(s, n, xs, h, dys, f, s->G(chunk, li, B_W1), h, f);
+    gather(L.ctx, L.da); wb.add(s, n, xs, h, dys, h, s->G(chunk, li, B_Wo), h, h);
+    gather(L.x, L.dqkv); wb.add(s, n, xs, h, dys, 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h);
+    return run_wgrads(s, st, wb);
   }
   if (s->d.family == JPP_FAMILY_DECODER) {
-    gather(L.g, L.dyin);   RC(wgrad_n(s, st, n, xs, f, dys, h, s->G(chunk, li, B_W2), f, h));
-    gather(L.n2, L.du);    RC(wgrad_n(s, st, n, xs, h, dys, f, s->G(chunk, li, B_W1), h, f));
-    gather(L.ctx, L.dh1);  RC(wgrad_n(s, st, n, xs, h, dys, h, s->G(chunk, li, B_Wo), h, h));
-    gather(L.n1, L.dqkv);  RC(wgrad_n(s, st, n, xs, h, dys, 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h));
-    return JPP_OK;
+    gather(L.g, L.dyin);   wb.add(s, n, xs, f, dys, h, s->G(chunk, li, B_W2), f, h);
+    gather(L.n2, L.du);    wb.add(s, n, xs, h, dys, f, s->G(chunk, li, B_W1), h, f);
+    gather(L.ctx, L.dh1);  wb.add(s, n, xs, h, dys, h, s->G(chunk, li, B_Wo), h, h);
+    gather(L.n1, L.dqkv);  wb.add(s, n, xs, h, dys, 3 * h, s->G(chunk, li, B_Wqkv), h, 3 * h);
+    return run_wgrads(s, st, wb);
   }
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
     float* partial = s->S<float>(s->s_partial);
@@ -561,15 +617,15 @@ int layer_bwd_w_group(jpp_stage* s, hipStream_t st, int chunk, int li, int n, ui
       RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)at(L.dlogits), s->G(chunk, li, X_Wr),
                               partial));
     }
-    gather(L.ctx, L.dh1);  RC(wgrad_n(s, st, n, xs, s->ctxw, dys, h, s->G(chunk, li, X_Wo), s->ctxw, h));
-    gather(L.n1, L.dqkv);  RC(wgrad_n(s, st, n, xs, h, dys, s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw));
-    return JPP_OK;
+    gather(L.ctx, L.dh1);  wb.add(s, n, xs, s->ctxw, dys, h, s->G(chunk, li, X_Wo), s->ctxw, h);
+    gather(L.n1, L.dqkv);  wb.add(s, n, xs, h, dys, s->qkvw, s->G(chunk, li, X_Wqkv), h, s->qkvw);
+    return run_wgrads(s, st, wb);
   }
-  gather(L.s, L.dyin);   RC(wgrad_n(s, st, n, xs, f, dys, h, s->G(chunk, li, L_Wd), f, h));
-  gather(L.n2, L.dgu);   RC(wgrad_n(s, st, n, xs, h, dys, 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f));
-  gather(L.ctx, L.dh1);  RC(wgrad_n(s, st, n, xs, s->ctxw, dys, h, s->G(chunk, li, L_Wo), s->ctxw, h));
-  gather(L.n1, L.dqkv);  RC(wgrad_n(s, st, n, xs, h, dys, s->qkvw, s->G(chunk, li, L_Wqkv), h, s->qkvw));
-  return JPP_OK;
+  gather(L.s, L.dyin);   wb.add(s, n, xs, f, dys, h, s->G(chunk, li, L_Wd), f, h);
+  gather(L.n2, L.dgu);   wb.add(s, n, xs, h, dys, 2 * f, s->G(chunk, li, L_Wgu), h, 2 * f);
+  gather(L.ctx, L.dh1);  wb.add(s, n, xs, s->ctxw, dys, h, s->G(chunk, li, L_Wo), s->ctxw, h);
+  gather(L.n1, L.dqkv);  wb.add(s, n, xs, h, dys, s->qkvw, s->G(chunk, li, L_Wqkv), h, s->qkvw);
+  return run_wgrads(s, st, wb);
 }
 
 // Runs the pending weight-gradient halves of a chunk (a whole group, or what a flush finds)

@@ -106,7 +106,7 @@ EXPORTS = [
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
     "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_workspace_bytes", "jpp_graph_begin", "jpp_graph_end", "jpp_graph_launch",
     "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_probe_class", "jpp_mfma_rate",
-    "jpp_gemm_bf16", "jpp_attn_fwd", "jpp_attn_bwd",
+    "jpp_gemm_bf16", "jpp_gemm_bf16_multi", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_gemm_f32", "jpp_attn_fwd_f32", "jpp_attn_bwd_f32", "jpp_norm_fwd_f32", "jpp_norm_bwd_f32",
     "jpp_colsum_accum_f32", "jpp_mse_loss_f32", "jpp_rope_f32",
     "jpp_norm_fwd", "jpp_norm_bwd", "jpp_norm_bwd_static", "jpp_swiglu_fwd", "jpp_swiglu_bwd", "jpp_rope",
@@ -168,6 +168,7 @@ def load():
                                     C.POINTER(C.c_double), C.POINTER(C.c_double),
                                     C.POINTER(C.c_double)]
     lib.jpp_gemm_bf16.argtypes = [C.c_void_p, C.POINTER(GemmArgs)]
+    lib.jpp_gemm_bf16_multi.argtypes = [C.c_void_p, C.POINTER(GemmArgs), C.c_int]
     lib.jpp_attn_fwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_attn_bwd.argtypes = [C.c_void_p, C.POINTER(AttnArgs)]
     lib.jpp_norm_fwd.argtypes = [C.c_void_p, C.POINTER(NormArgs)]
@@ -468,6 +469,24 @@ def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, b
         g.b_more = (C.c_void_p * 3)(*([pb for _, pb in more] + [None] * (3 - len(more))))
         g.k_parts = 1 + len(more)
     check((load().jpp_gemm_f32 if f32 else load().jpp_gemm_bf16)(stream, C.byref(g)))
+
+
+def gemm_multi(problems, stream=None):
+    """Up to four accumulated weight gradients as one launch (jpp_gemm_bf16_multi).  Each
+    problem is a dict: a, b, c (device pointers), m, n, k, lda, ldb, ldc and optionally
+    `more` = further (a, b) operand pairs."""
+    arr = (GemmArgs * len(problems))()
+    for i, q in enumerate(problems):
+        g = GemmArgs(q["a"], q["b"], q["c"], None, None, None, None, q["m"], q["n"], q["k"],
+                     q["lda"], q["ldb"], q["ldc"], 0, 0, 0, 1, 1, q.get("epilogue", EPI_ACC_F32),
+                     0, q.get("tile", 0), None, 0, 0, 0, 0, 0, None)
+        more = q.get("more", ())
+        if more:
+            g.a_more = (C.c_void_p * 3)(*([pa for pa, _ in more] + [None] * (3 - len(more))))
+            g.b_more = (C.c_void_p * 3)(*([pb for _, pb in more] + [None] * (3 - len(more))))
+            g.k_parts = 1 + len(more)
+        arr[i] = g
+    check(load().jpp_gemm_bf16_multi(stream, arr, len(problems)))
 
 
 def mfma_rate(shape: int, random_operands: bool, iters: int = 100000) -> float:

@@ -484,5 +484,6 @@ def test_bench_row_equals_sequential_order(name, peak):
             np.testing.assert_array_equal(outs_grp[k], v, err_msg=f"grouped: output of {k}")
         for i, gd in enumerate(grads_seq):
             for pname, v in gd.items():
-                parity.close(grads_grp[i][pname], v, 1e-5, f"grouped: grad {i}/{pname}")
+                # sums of 32 x 4096 products in another order: a few fp32 ulps of the terms
+                parity.close(grads_grp[i][pname], v, 3e-5, f"grouped: grad {i}/{pname}")
         ex.close()

@@ -135,6 +135,49 @@ def test_gemm_contraction_over_several_operand_pairs(parts, m, n, k, tile):
                 more=[(dA[0].ptr, dB[0].ptr)])
 
 
+@pytest.mark.parametrize("parts,k,shapes", [
+    (1, 192, [(512, 256), (256, 768)]),
+    (4, 128, [(1536, 1024), (1024, 1024), (1024, 7168), (3584, 1024)]),   # 13 x 64 tiles
+    (2, 256, [(4096, 6144), (4096, 4096), (256, 256)])])                  # 384 + 256 + 1 tiles
+def test_gemm_several_weight_gradients_in_one_launch(parts, k, shapes):
+    """jpp_gemm_bf16_multi: independent accumulated weight gradients as one grid of tiles.
+    Against numpy, and bit for bit against the same problems launched one by one (contractions
+    this short add the old accumulator value in the epilogue whatever the tile, so an output
+    element sees the same sum in the same order whichever launch computes it)."""
+    rng = np.random.default_rng(parts + k + len(shapes))
+    probs, keep, wants, prevs = [], [], [], []
+    for m, n in shapes:
+        As = [rnd(rng, k, m) for _ in range(parts)]
+        Bs = [rnd(rng, k, n, scale=0.05) for _ in range(parts)]
+        prev = rng.standard_normal((m, n)).astype(np.float32)
+        wants.append(prev + sum(a.astype(np.float64).T @ b.astype(np.float64) for a, b in zip(As, Bs)))
+        dA, dB = [dev_bf16(a) for a in As], [dev_bf16(b) for b in Bs]
+        dc = rt.DeviceBuffer.from_numpy(prev)
+        keep.append((dA, dB, dc))
+        prevs.append(prev)
+        probs.append(dict(a=dA[0].ptr, b=dB[0].ptr, c=dc.ptr, m=m, n=n, k=k, lda=m, ldb=n, ldc=n,
+                          more=[(a.ptr, b.ptr) for a, b in zip(dA[1:], dB[1:])]))
+    rt.gemm_multi(probs)
+    rt.sync()
+    got = [dc.download(np.float32, shp) for (_, _, dc), shp in zip(keep, shapes)]
+    for g, w, shp in zip(got, wants, shapes):
+        close(g, w, 1e-4 * math.sqrt(k * parts), f"multi {shp}")
+    for (dA, dB, dc), prev, (m, n), g in zip(keep, prevs, shapes, got):
+        dc.upload(prev)
+        # (several operand pairs: only the 256-wide tiles are built for that)
+        rt.gemm(dA[0].ptr, dB[0].ptr, dc.ptr, m, n, k, m, n, n, 1, 1, rt.EPI_ACC_F32,
+                tile=4 if parts > 1 and (m // 256) * (n // 256) < 192 else 0,
+                more=[(a.ptr, b.ptr) for a, b in zip(dA[1:], dB[1:])])
+        rt.sync()
+        np.testing.assert_array_equal(dc.download(np.float32, (m, n)), g)
+    with pytest.raises(rt.JppError, match="differs from problem 0 in k or k_parts"):
+        rt.gemm_multi([probs[0], dict(probs[1], k=64)])
+    with pytest.raises(rt.JppError, match="not a plain accumulated weight gradient"):
+        rt.gemm_multi([probs[0], dict(probs[1], epilogue=rt.EPI_F32)])
+    with pytest.raises(rt.JppError, match="1 to 4 problems"):
+        rt.gemm_multi([probs[0]] * 5)
+
+
 def test_gemm_rejects_bad_shapes():
     d = rt.DeviceBuffer(1 << 16)
     with pytest.raises(rt.JppError, match="multiples of 128"):
