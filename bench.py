@@ -213,11 +213,13 @@ def main():
                     help="weight gradients of this many consecutive microbatches as one product "
                          "per weight (1: per microbatch; default: see default_wgrad_group)")
     ap.add_argument("--probe", default=None, help="kernel class to time (default: dominant GEMM)")
-    ap.add_argument("--graph", action="store_true",
+    ap.add_argument("--graph", choices=["auto", "on", "off"], default="auto", nargs="?", const="on",
                     help="record the step into a HIP graph after the warm-up and time replays "
                          "of it (no host launch work in the timed region); the per-kernel probe "
                          "cannot see inside a replay, so `roofline` then comes from one more "
-                         "eager step after the timed ones")
+                         "eager step after the timed ones.  auto: for narrow layers (hidden < "
+                         "2048: thousands of small launches per step, +3 %), not for wide ones "
+                         "(the GPU is busy 99.8 % of an eager step)")
     ap.add_argument("--kernel-table", action="store_true",
                     help="instead of the one-line result, time every kernel class of the step "
                          "with HIP events (jpp_probe_begin(\"*\")) over the timed steps and print "
@@ -257,6 +259,7 @@ def main():
     group = args.wgrad_group if args.wgrad_group is not None else default_wgrad_group(wl, two)
     if args.unfused_accumulate or two:
         group = 1
+    args.graph = args.graph == "on" or (args.graph == "auto" and wl.layer.hidden < 2048)
     wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two, wgrad_group=group)
     if args.kernel_table:
         print(json.dumps(kernel_table(wb, wl, args.steps, args.warmup, two, group)))

@@ -286,6 +286,9 @@ int run_wgrads(jpp_stage* s, hipStream_t st, WgradBatch& w) {
     const jpp_gemm_args& q = w.g[i];
     if (q.m % 256 || q.n % 256) { multi = false; break; }
     const long t = (q.m / 256) * (q.n / 256), rest = t % 256;
+    // smaller matrices run on 128x128 tiles, split over the tokens where that fills the
+    // device: not this comparison
+    if (t < 192) { multi = false; break; }
     total += t;
     apart += (double)(t / 256) + (rest == 0 ? 0.0 : (rest <= 128 && t > 256 ? 0.77 : 1.0));
   }
