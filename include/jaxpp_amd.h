@@ -210,6 +210,12 @@ typedef struct {
   float* delta;             /* bwd scratch, f32 [batch, n_heads, seq] */
   int64_t ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv;
   int batch, seq, n_heads, n_kv_heads, head_dim, causal;
+  /* Backward only, optional (NULL: off): f32 [seq, head_dim/2] tables of the half-split rotary
+   * embedding the caller applied to q and k before the forward.  dq and dk are then written
+   * already rotated back (by the negative angle), i.e. as jpp_rope(..., inverse = 1) would
+   * leave them: the cotangents of the un-rotated q and k, without a pass of their own. */
+  const float* rope_cos;
+  const float* rope_sin;
 } jpp_attn_args;
 
 int jpp_attn_fwd(void* stream, const jpp_attn_args* args);

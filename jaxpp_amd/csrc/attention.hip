@@ -322,6 +322,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
     __syncthreads();
   }
 
+  if (p.rope_cos) rope_back<D, DT>(dqacc, p.rope_cos, p.rope_sin, qi, lane);
   bf16_t* drow = p.dq + (row0 + qi) * p.lddq + h * D;
 #pragma unroll
   for (int i = 0; i < DT; ++i)
@@ -519,6 +520,8 @@ AttnParams make_params(const jpp_attn_args* a) {
   p.lddo = a->lddo; p.lddq = a->lddq; p.lddk = a->lddk; p.lddv = a->lddv;
   p.batch = a->batch; p.seq = a->seq; p.n_heads = a->n_heads; p.n_kv_heads = a->n_kv_heads;
   p.scale = 1.0f / sqrtf((float)a->head_dim);
+  p.rope_cos = nullptr;
+  p.rope_sin = nullptr;
   return p;
 }
 
@@ -555,7 +558,11 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
   JPP_REQUIRE((a->lddo | a->lddq | a->lddk | a->lddv) % 8 == 0 &&
                   ((uintptr_t)a->d_o | (uintptr_t)a->dq | (uintptr_t)a->dk | (uintptr_t)a->dv) % 16 == 0,
               "attn_bwd: operands must keep 16-byte alignment");
+  JPP_REQUIRE(!a->rope_cos == !a->rope_sin, "attn_bwd: rope_cos and rope_sin go together");
   AttnParams p = make_params(a);
+  // the causal kernels rotate dq / dk back themselves; without a mask a pass of its own does
+  const bool fused_rope = a->rope_cos && a->causal;
+  if (fused_rope) { p.rope_cos = a->rope_cos; p.rope_sin = a->rope_sin; }
   hipStream_t st = (hipStream_t)stream;
   const long items = (long)a->batch * a->seq * a->n_heads * (a->head_dim / 8);
   dim3 gdelta((unsigned)((items + 255) / 256));
@@ -587,5 +594,12 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
   else { if (a->causal) JPP_AB(128, true); else JPP_AB(128, false); }
 #undef JPP_AB
   JPP_LAUNCH_CHECK();
+  if (a->rope_cos && !fused_rope) {
+    if (int rc = jpp_rope(stream, a->dq, a->lddq, a->rope_cos, a->rope_sin, a->batch, a->seq,
+                          a->n_heads, a->head_dim, 1))
+      return rc;
+    return jpp_rope(stream, a->dk, a->lddk, a->rope_cos, a->rope_sin, a->batch, a->seq,
+                    a->n_kv_heads, a->head_dim, 1);
+  }
   return JPP_OK;
 }

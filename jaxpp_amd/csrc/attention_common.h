@@ -21,7 +21,37 @@ struct AttnParams {
   long ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv;
   int batch, seq, n_heads, n_kv_heads;
   float scale;
+  const float* rope_cos;  // backward: dq / dk leave rotated back when set
+  const float* rope_sin;
 };
+
+// Transpose of the half-split rotary embedding on an accumulator row: the lane holds, of
+// the row at sequence position `pos`, the head's elements d = 32 i + 8 (r / 4) + 4 (lane /
+// 32) + r % 4 in acc[i][r]; element d < D/2 pairs with d + D/2, i.e. acc[i] with
+// acc[i + DT/2], same r.  The values are rounded to bf16 first, as a separate pass would
+// read them back from memory.
+template <int D, int DT>
+__device__ __forceinline__ void rope_back(f32x16 (&acc)[DT], const float* cos_tab,
+                                          const float* sin_tab, int pos, int lane) {
+  static_assert(DT * 32 == D && DT % 2 == 0, "head of D elements in DT tiles of 32");
+  const float* ct = cos_tab + (long)pos * (D / 2) + (lane >> 5) * 4;
+  const float* st = sin_tab + (long)pos * (D / 2) + (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < DT / 2; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 c4 = *(const float4*)(ct + i * 32 + g * 8);
+      const float4 s4 = *(const float4*)(st + i * 32 + g * 8);
+      const float cs[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {-s4.x, -s4.y, -s4.z, -s4.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float a = (float)(__bf16)acc[i][4 * g + e];
+        const float b = (float)(__bf16)acc[i + DT / 2][4 * g + e];
+        acc[i][4 * g + e] = a * cs[e] - b * sn[e];
+        acc[i + DT / 2][4 * g + e] = b * cs[e] + a * sn[e];
+      }
+    }
+}
 
 // 8 consecutive accumulator registers -> one bf16 MFMA operand
 __device__ __forceinline__ bf16x8 acc_to_frag(const f32x16& a, int base) {

@@ -206,12 +206,15 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
       bf16_t* dkrow = p.dk + (row0 + ki) * p.lddk + hk * D;
       bf16_t* dvrow = p.dv + (row0 + ki) * p.lddv + hk * D;
 #pragma unroll
-      for (int i = 0; i < DT; ++i) {
+      for (int i = 0; i < DT; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           dkacc[i][r] += xch[(i * 16 + r) * 64];
           dvacc[i][r] += xch[((DT + i) * 16 + r) * 64];
         }
+      if (p.rope_cos) rope_back<D, DT>(dkacc, p.rope_cos, p.rope_sin, ki, lane);
+#pragma unroll
+      for (int i = 0; i < DT; ++i) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int d = i * 32 + g * 8 + (lane >> 5) * 4;

@@ -524,8 +524,15 @@ int layer_bwd_i(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, 
   aa.dv = dqkv + (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd * s->es;
   aa.lddq = aa.lddk = aa.lddv = s->qkvw;
   aa.delta = s->S<float>(s->s_delta);
-  RC(attn_b(s, st, &aa));
-  RC(rope(s, st, dqkv, 1));
+  if (s->f32()) {
+    RC(attn_b(s, st, &aa));
+    RC(rope(s, st, dqkv, 1));
+  } else {
+    // dq and dk leave the attention backward already rotated back
+    aa.rope_cos = s->S<float>(s->s_cos);
+    aa.rope_sin = s->S<float>(s->s_sin);
+    RC(attn_b(s, st, &aa));
+  }
   RC(gemm(s, st, dqkv, s->qkvw, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 0, dn, h, T, h, s->qkvw,
           JPP_EPI_BF16));
   RC(norm_b(s, st, dn, at(L.x), nullptr, (float*)at(L.rstd1), s->P(chunk, li, L_rms1), wt(W.dh1),

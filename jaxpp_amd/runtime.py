@@ -51,7 +51,8 @@ class AttnArgs(C.Structure):
                 ("lddo", C.c_int64), ("lddq", C.c_int64), ("lddk", C.c_int64),
                 ("lddv", C.c_int64),
                 ("batch", C.c_int), ("seq", C.c_int), ("n_heads", C.c_int),
-                ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("causal", C.c_int)]
+                ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("causal", C.c_int),
+                ("rope_cos", C.c_void_p), ("rope_sin", C.c_void_p)]
 
 
 class NormArgs(C.Structure):

@@ -241,6 +241,18 @@ def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
     close(got[:, :hq * d], dqkv_w[:, :hq * d], 2e-2, "dq")
     close(got[:, hq * d:(hq + hkv) * d], dqkv_w[:, hq * d:(hq + hkv) * d], 2e-2, "dk")
     close(got[:, (hq + hkv) * d:], dqkv_w[:, (hq + hkv) * d:], 2e-2, "dv")
+    # with rotary tables the backward writes dq and dk already rotated back: the same values
+    # a pass of jpp_rope(inverse) over the plain result leaves (q and k heads are adjacent)
+    cos, sin = L.rope_tables(seq, d, 5e5, np.float32)
+    bc, bs = rt.DeviceBuffer.from_numpy(cos), rt.DeviceBuffer.from_numpy(sin)
+    rt.check(rt.load().jpp_rope(None, dqkv_d.ptr, width, bc.ptr, bs.ptr, batch, seq, hq + hkv, d, 1))
+    rt.sync()
+    want_r = dqkv_d.download_bf16((T, width))
+    dqkv_d.zero()
+    a.rope_cos, a.rope_sin = bc.ptr, bs.ptr
+    rt.check(rt.load().jpp_attn_bwd(None, C.byref(a)))
+    rt.sync()
+    np.testing.assert_array_equal(dqkv_d.download_bf16((T, width)), want_r)
 
 
 @pytest.mark.parametrize("ln,rows,cols", [(True, 300, 256), (True, 1024, 1024), (False, 512, 4096),
