@@ -220,6 +220,12 @@ def main():
                          "eager step after the timed ones.  auto: for narrow layers (hidden < "
                          "2048: thousands of small launches per step, +3 %), not for wide ones "
                          "(the GPU is busy 99.8 % of an eager step)")
+    ap.add_argument("--extra-fills", type=int, default=0,
+                    help="diagnostic: after every step, clear a 6 GiB scratch buffer this many "
+                         "times (about 2 ms each of memory-bound, low-power work).  The step "
+                         "grows by less than the fills take alone: the device holds an average "
+                         "power, and what the matrix-core kernels lose to it they partly get "
+                         "back while something cheaper runs.  Not a valid headline run.")
     ap.add_argument("--kernel-table", action="store_true",
                     help="instead of the one-line result, time every kernel class of the step "
                          "with HIP events (jpp_probe_begin(\"*\")) over the timed steps and print "
@@ -271,10 +277,14 @@ def main():
     # 100 000 launches.
     ends = []
 
+    filler = rt.DeviceBuffer(6 << 30) if args.extra_fills else None
+
     def paced_step():
         if len(ends) >= 2:
             ends.pop(0).sync()
         wb.step()
+        for _ in range(args.extra_fills):
+            filler.zero()
         ev = rt.Event()
         ev.record()
         ends.append(ev)
@@ -331,6 +341,7 @@ def main():
             "peak_live_microbatches": wb.plan.max_live,
             "fused_wgrad_accumulate": not args.unfused_accumulate,
             "two_streams": two, "hip_graph": bool(args.graph), "wgrad_group": group,
+            **({"extra_fills": args.extra_fills} if args.extra_fills else {}),
             "device_bytes": wb.ex.nbytes,
         },
         "algorithmic_flops_per_step": flops,
