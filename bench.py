@@ -150,10 +150,13 @@ def default_wgrad_group(wl, two_streams: bool) -> int:
     fp32 accumulator is then read and written once per group).  Measured on MI355X, A/B on one
     box: Llama-8B-shaped stage 1397-1402 ms/step ungrouped, 1393-1395 in pairs, 1373-1379 in
     fours (73 GB); 70B-shaped 4579-4584 / 4545-4552 / 4543-4554 ms (197 / 215 / 251 GB), so
-    pairs there.  The expert layers' grouped products cannot be merged across microbatches
-    (their row groups differ) and narrow layers run two streams: ungrouped."""
-    if two_streams or wl.layer.family != "llama" or wl.layer.hidden < 4096:
+    pairs there.  The Mixtral-shaped stage 2671-2699 ms ungrouped, 2615-2627 in pairs (206 /
+    236 GB; the experts' grouped contraction takes the pairs' own row groups): pairs, fours do
+    not fit.  Narrow layers run two streams: ungrouped."""
+    if two_streams or wl.layer.family not in ("llama", "mixtral") or wl.layer.hidden < 4096:
         return 1
+    if wl.layer.family == "mixtral":
+        return 2
     return 4 if wl.layer.hidden < 8192 else 2
 
 

@@ -178,6 +178,12 @@ typedef struct {
   const void* a_more[3];
   const void* b_more[3];
   int k_parts;
+  /* JPP_GROUP_K over several operand pairs: pair i > 0 has its own row groups,
+   * seg_more[i-1] (device int32 [n_seg + 1]) and, if seg_rows is given, seg_rows_more[i-1]
+   * (device int32 [n_seg]); C_e then gets the products over group e of every pair (the expert
+   * weight gradients of several microbatches, whose routing differs). */
+  const int32_t* seg_more[3];
+  const int32_t* seg_rows_more[3];
 } jpp_gemm_args;
 
 enum { JPP_GROUP_NONE = 0, JPP_GROUP_M = 1, JPP_GROUP_K = 2 };

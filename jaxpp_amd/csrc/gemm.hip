@@ -40,6 +40,9 @@ struct GemmParams {
   const bf16_t* a_more[3];
   const bf16_t* b_more[3];
   int k_parts, kt_part;
+  // JPP_GROUP_K over several pairs: row groups of pair i > 0
+  const int* seg_more[3];
+  const int* seg_rows_more[3];
   void* c;
   void* c2;
   const bf16_t* bias;
@@ -139,15 +142,21 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
   tn = (pid % width) / gsize;
 }
 
-// Operand tile of K-step kt when the contraction runs over up to four operand pairs of
-// kt_part K-steps each (all arguments wave-uniform).
+// Operand tile of K-step kt when the contraction runs over up to four operand pairs: pair i
+// starts at K-step c_i (c_0 = 0; c_1 <= c_2 <= c_3, equal where a pair has no steps).  All
+// arguments are wave-uniform.
 __device__ __forceinline__ const bf16_t* part_ptr(const bf16_t* p0, const bf16_t* p1,
                                                   const bf16_t* p2, const bf16_t* p3, int kt,
-                                                  int kt_part, int k_parts, long step) {
-  if (k_parts <= 1) return p0 + (long)kt * step;
-  const int part = (kt >= kt_part) + (kt >= 2 * kt_part) + (kt >= 3 * kt_part);
+                                                  int c1, int c2, int c3, long step) {
+  const int part = (kt >= c1) + (kt >= c2) + (kt >= c3);
   const bf16_t* base = part == 0 ? p0 : part == 1 ? p1 : part == 2 ? p2 : p3;
-  return base + (long)(kt - part * kt_part) * step;
+  const int start = part == 0 ? 0 : part == 1 ? c1 : part == 2 ? c2 : c3;
+  return base + (long)(kt - start) * step;
+}
+// K-steps that hold data of row group e of a grouped contraction
+__device__ __forceinline__ int group_steps(const int* seg, const int* seg_rows, int e) {
+  const int rows = seg_rows ? min(seg_rows[e], seg[e + 1] - seg[e]) : seg[e + 1] - seg[e];
+  return (rows + 63) / 64;
 }
 
 template <int BM, int BN, bool TA, bool TB, int EPI, int NW, int NS, bool KP = false, bool MP = false>
@@ -200,6 +209,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   const bf16_t* a_src = p.a + a_off;
   const bf16_t* b_src = p.b + b_off;
   int kt_n = p.k / 64 * (KP ? p.k_parts : 1);
+  // several operand pairs: first K-step of pairs 1..3 and their operands at this tile
+  int c1 = p.kt_part, c2 = 2 * p.kt_part, c3 = 3 * p.kt_part;
+  const bf16_t* a1 = KP ? p.a_more[0] + a_off : a_src;
+  const bf16_t* a2 = KP ? p.a_more[1] + a_off : a_src;
+  const bf16_t* a3 = KP ? p.a_more[2] + a_off : a_src;
+  const bf16_t* b1 = KP ? p.b_more[0] + b_off : b_src;
+  const bf16_t* b2 = KP ? p.b_more[1] + b_off : b_src;
+  const bf16_t* b3 = KP ? p.b_more[2] + b_off : b_src;
   if (p.group_mode == JPP_GROUP_M) {
     // rows of A and C are grouped by expert; each group multiplies its own B
     if (m0 >= p.seg[p.n_seg]) return;
@@ -211,10 +228,31 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
     const int e = bid / tiles;
     const long r0 = p.seg[e];
     // rows past the group's data are zero padding: steps made of nothing else are skipped
-    const int rows = p.seg_rows ? min(p.seg_rows[e], p.seg[e + 1] - p.seg[e]) : p.seg[e + 1] - p.seg[e];
-    kt_n = (rows + 63) / 64;
+    kt_n = group_steps(p.seg, p.seg_rows, e);
     a_src += r0 * p.lda;
     b_src += r0 * p.ldb;
+    if constexpr (KP) {
+      // every further pair brings its own row groups (pair by pair, never an index into the
+      // kernel arguments); a pair past k_parts starts where the contraction ends
+      c1 = c2 = c3 = kt_n;
+      if (p.k_parts > 1) {
+        const long r = p.seg_more[0][e];
+        a1 += r * p.lda; b1 += r * p.ldb;
+        kt_n += group_steps(p.seg_more[0], p.seg_rows_more[0], e);
+        c2 = c3 = kt_n;
+      }
+      if (p.k_parts > 2) {
+        const long r = p.seg_more[1][e];
+        a2 += r * p.lda; b2 += r * p.ldb;
+        kt_n += group_steps(p.seg_more[1], p.seg_rows_more[1], e);
+        c3 = kt_n;
+      }
+      if (p.k_parts > 3) {
+        const long r = p.seg_more[2][e];
+        a3 += r * p.lda; b3 += r * p.ldb;
+        kt_n += group_steps(p.seg_more[2], p.seg_rows_more[2], e);
+      }
+    }
     p.c = EPI == JPP_EPI_BF16 ? (void*)((bf16_t*)p.c + (long)e * p.stride_c)
                               : (void*)((float*)p.c + (long)e * p.stride_c);
     if (kt_n == 0 && EPI == JPP_EPI_ACC_F32) return;
@@ -225,15 +263,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   // then pair 1, ... (kt and the pair index are wave-uniform: scalar arithmetic; the pair
   // pointers are picked by a chain of selects, never by indexing the kernel arguments)
   // (kernels built without KP take one pair and keep the plain address arithmetic)
-  const int k_parts = KP ? p.k_parts : 1, kt_part = p.kt_part;
-  const bf16_t* const a1 = KP ? p.a_more[0] + a_off : a_src;
-  const bf16_t* const a2 = KP ? p.a_more[1] + a_off : a_src;
-  const bf16_t* const a3 = KP ? p.a_more[2] + a_off : a_src;
-  const bf16_t* const b1 = KP ? p.b_more[0] + b_off : b_src;
-  const bf16_t* const b2 = KP ? p.b_more[1] + b_off : b_src;
-  const bf16_t* const b3 = KP ? p.b_more[2] + b_off : b_src;
-#define a_at(kt) (KP ? part_ptr(a_src, a1, a2, a3, (kt), kt_part, k_parts, a_step) : a_src + (long)(kt) * a_step)
-#define b_at(kt) (KP ? part_ptr(b_src, b1, b2, b3, (kt), kt_part, k_parts, b_step) : b_src + (long)(kt) * b_step)
+#define a_at(kt) (KP ? part_ptr(a_src, a1, a2, a3, (kt), c1, c2, c3, a_step) : a_src + (long)(kt) * a_step)
+#define b_at(kt) (KP ? part_ptr(b_src, b1, b2, b3, (kt), c1, c2, c3, b_step) : b_src + (long)(kt) * b_step)
 
   // of tile (i, j) a lane holds row wm BM/2 + 16 i + lane % 16 and the four columns
   // wn BN/WN + 16 j + 4 (lane / 16) + {0..3}
@@ -801,14 +832,21 @@ int prepare(const jpp_gemm_args* a, GemmParams& p) {
   for (int i = 0; i < 3; ++i) {
     p.a_more[i] = (const bf16_t*)a->a_more[i];
     p.b_more[i] = (const bf16_t*)a->b_more[i];
+    p.seg_more[i] = a->seg_more[i];
+    p.seg_rows_more[i] = a->seg_rows_more[i];
   }
   if (a->k_parts > 1) {
-    JPP_REQUIRE(a->k_parts <= 4 && a->group_mode == JPP_GROUP_NONE,
-                "gemm: at most 4 operand pairs, and not in a grouped problem");
-    for (int i = 0; i + 1 < a->k_parts; ++i)
+    JPP_REQUIRE(a->k_parts <= 4 && a->group_mode != JPP_GROUP_M,
+                "gemm: at most 4 operand pairs, and not with grouped rows (JPP_GROUP_M)");
+    for (int i = 0; i + 1 < a->k_parts; ++i) {
       JPP_REQUIRE(a->a_more[i] && a->b_more[i] &&
                       ((uintptr_t)a->a_more[i] | (uintptr_t)a->b_more[i]) % 16 == 0,
                   "gemm: operand pair %d is null or not 16-byte aligned", i + 1);
+      if (group_k)
+        JPP_REQUIRE(a->seg_more[i] && !a->seg_rows_more[i] == !a->seg_rows,
+                    "gemm: operand pair %d of a grouped contraction needs its row groups "
+                    "(seg_more, and seg_rows_more when seg_rows is given)", i + 1);
+    }
   }
   if (a->group_mode != JPP_GROUP_NONE) {
     JPP_REQUIRE(a->group_mode == JPP_GROUP_M || a->group_mode == JPP_GROUP_K,

@@ -615,15 +615,44 @@ int layer_bwd_w_group(jpp_stage* s, hipStream_t st, int chunk, int li, int n, ui
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
     float* partial = s->S<float>(s->s_partial);
     const int E = s->d.n_experts;
+    // the experts' weight gradients over all n microbatches at once where the grouped
+    // contraction takes several operand pairs (each with its own row groups: the routing
+    // differs from microbatch to microbatch), else microbatch by microbatch
+    const bool together = n > 1 && !s->f32() && s->d.fused_wgrad_accum;
+    if (together) {
+      auto experts = [&](const Buf& x, int64_t ldx, const Buf& dy, int64_t lddy, float* acc,
+                         int64_t rows, int64_t cols) {
+        jpp_gemm_args g;
+        memset(&g, 0, sizeof(g));
+        g.m = rows; g.n = cols; g.lda = ldx; g.ldb = lddy; g.ldc = cols;
+        g.trans_a = 1; g.trans_b = 1; g.epilogue = JPP_EPI_ACC_F32;
+        g.group_mode = JPP_GROUP_K; g.n_seg = E; g.stride_c = rows * cols;
+        g.group_rows = (int64_t)n * s->T * s->d.top_k;
+        g.c = acc; g.k_parts = n;
+        for (int i = 0; i < n; ++i) {
+          const int32_t* seg = (const int32_t*)(slots[i] + L.seg.off);
+          const void* a = slots[i] + x.off;
+          const void* b = slots[i] + dy.off;
+          if (i == 0) { g.a = a; g.b = b; g.seg = seg; g.seg_rows = seg + E + 1; }
+          else { g.a_more[i - 1] = a; g.b_more[i - 1] = b; g.seg_more[i - 1] = seg;
+                 g.seg_rows_more[i - 1] = seg + E + 1; }
+        }
+        return jpp_gemm_bf16(st, &g);
+      };
+      RC(experts(L.s, f, L.deo, h, s->G(chunk, li, X_Wd), f, h));
+      RC(experts(L.xp, h, L.dgu, 2 * f, s->G(chunk, li, X_Wgu), h, 2 * f));
+    }
     for (int i = 0; i < n; ++i) {
       uint8_t* slot = slots[i];
       auto at = [&](const Buf& b) { return (void*)(slot + b.off); };
       jpp_moe_args ma;
       moe_args(s, ma, slot, L, chunk, li);
-      RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.s), f, 1, at(L.deo), h, 1, 0, s->G(chunk, li, X_Wd), h,
-               f * h, f, h, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
-      RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, at(L.dgu), 2 * f, 1, 0,
-               s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+      if (!together) {
+        RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.s), f, 1, at(L.deo), h, 1, 0, s->G(chunk, li, X_Wd), h,
+                 f * h, f, h, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+        RC(ggemm(s, st, JPP_GROUP_K, ma.seg, E, at(L.xp), h, 1, at(L.dgu), 2 * f, 1, 0,
+                 s->G(chunk, li, X_Wgu), 2 * f, h * 2 * f, h, 2 * f, 0, JPP_EPI_ACC_F32, s->T * s->d.top_k));
+      }
       RC(jpp_moe_router_wgrad(st, &ma, at(L.n2), (const float*)at(L.dlogits), s->G(chunk, li, X_Wr),
                               partial));
     }

@@ -516,6 +516,33 @@ def test_grouped_gemm():
         want = acc0[e] + xp[seg[e]:seg[e + 1]].T @ dy[seg[e]:seg[e + 1]]
         close(got2[e], want, 1e-3, f"dW group {e}, padding steps skipped")
     np.testing.assert_array_equal(got2[1], acc0[1])
+    # several operand pairs, each with its own row groups (the expert weight gradients of
+    # several microbatches, routed differently): one launch adds all of them
+    counts_b = [0, 300, 256, 1, 0, 515, 70, 64]
+    seg_b = np.zeros(E + 1, np.int32)
+    for e, c in enumerate(counts_b):
+        seg_b[e + 1] = seg_b[e] + (c + 255) // 256 * 256
+    cap_b = int(seg_b[E]) + 256
+    xp_b, dy_b = np.zeros((cap_b, h), np.float32), np.zeros((cap_b, f), np.float32)
+    for e, c in enumerate(counts_b):
+        xp_b[seg_b[e]:seg_b[e] + c] = rnd(rng, c, h)
+        dy_b[seg_b[e]:seg_b[e] + c] = rnd(rng, c, f)
+    d_seg_b, d_rows_b = rt.DeviceBuffer.from_numpy(seg_b), rt.DeviceBuffer.from_numpy(np.array(counts_b, np.int32))
+    d_xp_b, d_dy_b = dev_bf16(xp_b), dev_bf16(dy_b)
+    b_acc3 = rt.DeviceBuffer.from_numpy(acc0)
+    rt.gemm(b_xp.ptr, b_dy.ptr, b_acc3.ptr, h, f, 0, h, f, f, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
+            n_seg=E, group_mode=2, stride_c=h * f, seg_rows=b_rows.ptr, tile=4,
+            more=[(d_xp_b.ptr, d_dy_b.ptr), (b_xp.ptr, b_dy.ptr)],
+            more_seg=[(d_seg_b.ptr, d_rows_b.ptr), (b_seg.ptr, b_rows.ptr)])
+    rt.sync()
+    got3 = b_acc3.download(np.float32, (E, h, f))
+    for e in range(E):
+        want = (acc0[e] + 2 * (xp[seg[e]:seg[e + 1]].T @ dy[seg[e]:seg[e + 1]])
+                + xp_b[seg_b[e]:seg_b[e + 1]].T @ dy_b[seg_b[e]:seg_b[e + 1]])
+        close(got3[e], want, 2e-3, f"dW group {e} over three operand pairs")
+    with pytest.raises(rt.JppError, match="needs its row groups"):
+        rt.gemm(b_xp.ptr, b_dy.ptr, b_acc3.ptr, h, f, 0, h, f, f, 1, 1, rt.EPI_ACC_F32, seg=b_seg.ptr,
+                n_seg=E, group_mode=2, stride_c=h * f, tile=4, more=[(d_xp_b.ptr, d_dy_b.ptr)])
 
 
 @pytest.mark.parametrize("tile,m,f,k", [(1, 128, 128, 64), (2, 256, 256, 128), (4, 512, 256, 192),
