@@ -262,14 +262,15 @@ def big_params(spec, stages, layers_per_chunk, seed=7):
     return out
 
 
-def run_on_gpu_with_routing(spec, plan, lpc, params, seed=0):
+def run_on_gpu_with_routing(spec, plan, lpc, params, seed=0, wgrad_group=0):
     """The rank's row, one task at a time; after every forward of a mixture stage the routing
     it chose is read back (jpp_stage_routing).  Returns run_on_gpu's triple and
     {(stage, microbatch): [expert ids per layer]}."""
     from jaxpp_amd.model import boundary_tensor
     from jaxpp_amd.types import TaskType
     shape = (spec.tokens, spec.hidden)
-    ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True, False)
+    ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True, False,
+                          wgrad_group=wgrad_group)
     for c, stage in enumerate(plan.stages):
         for li in range(lpc):
             ex.set_params(c, li, params[stage][li])
@@ -309,7 +310,7 @@ def run_on_gpu_with_routing(spec, plan, lpc, params, seed=0):
 NEAR_TIE_MARGIN = 2e-2
 
 
-def check_rank_row(spec, sched, n, rank, lpc, bad_frac=parity.STAGE_BAD_FRAC):
+def check_rank_row(spec, sched, n, rank, lpc, bad_frac=parity.STAGE_BAD_FRAC, wgrad_group=0):
     from jaxpp_amd.model import boundary_tensor
     from oracle import stage as O
     plan = make_rank_plan(sched, n, rank)
@@ -317,7 +318,7 @@ def check_rank_row(spec, sched, n, rank, lpc, bad_frac=parity.STAGE_BAD_FRAC):
     row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
     shape = (spec.tokens, spec.hidden)
     print(f"  gpu: {len(plan.tasks)} tasks", flush=True)
-    ys, dxs, grads, routing = run_on_gpu_with_routing(spec, plan, lpc, params)
+    ys, dxs, grads, routing = run_on_gpu_with_routing(spec, plan, lpc, params, wgrad_group=wgrad_group)
     print("  oracle", flush=True)
     ro = O.RankOracle(L.LayerCfg(**spec.as_dict()), {s_: params[s_] for s_ in plan.stages},
                       L.Numerics.bf16())
@@ -364,7 +365,8 @@ def test_llama_70b_layer_on_a_zero_bubble_row_matches_oracle():
     2e-4 of the input cotangent's, the first tokens of the sequence ahead; the GPU against the
     oracle: 1.6e-3 (up to 3.7 x) and 4.9e-4 (2.6 x)."""
     print("70B-shaped layer, ZeroBubble(2) rank 1", flush=True)
-    check_rank_row(LLAMA_70B_LAYER, S.ZeroBubble(2), 2, 1, 1, bad_frac=4e-3)
+    # weight gradients of the two microbatches as one product per weight, as the bench runs them
+    check_rank_row(LLAMA_70B_LAYER, S.ZeroBubble(2), 2, 1, 1, bad_frac=4e-3, wgrad_group=2)
 
 
 # The oracle multiplies on the host: at the bench's 2 x 4096 tokens the eight layer passes of a
@@ -380,7 +382,9 @@ def test_mixtral_8x7b_layer_on_a_dualpipev_row_matches_oracle():
     """One Mixtral-8x7B-shaped layer per stage on rank 0 of DualPipeV(4, 2) (stages 0 and 3:
     an unsplit first-stage backward and a split one), four microbatches, against the oracle."""
     print("Mixtral-shaped layers, DualPipeV(4,2) rank 0", flush=True)
-    check_rank_row(MIXTRAL_8X7B_LAYER, S.DualPipeV(4, 2), 4, 0, 1)
+    # weight gradients in pairs of microbatches, the experts' with each microbatch's own row
+    # groups, as the bench runs them
+    check_rank_row(MIXTRAL_8X7B_LAYER, S.DualPipeV(4, 2), 4, 0, 1, wgrad_group=2)
 
 
 @pytest.mark.parametrize("name,peak", [("cfg3", 11), ("cfg2", 4)])
