@@ -286,13 +286,14 @@ int run_wgrads(jpp_stage* s, hipStream_t st, WgradBatch& w) {
     const jpp_gemm_args& q = w.g[i];
     if (q.m % 256 || q.n % 256) { multi = false; break; }
     const long t = (q.m / 256) * (q.n / 256), rest = t % 256;
-    // smaller matrices run on 128x128 tiles, split over the tokens where that fills the
-    // device: not this comparison
-    if (t < 192) { multi = false; break; }
     total += t;
     apart += (double)(t / 256) + (rest == 0 ? 0.0 : (rest <= 128 && t > 256 ? 0.77 : 1.0));
   }
-  if (multi && (double)((total + 255) / 256) < apart - 0.25) {
+  // (matrices of fewer than 192 tiles would run one by one on 128x128 tiles, each launch
+  // leaving most of the device idle: BERT-large's four are 192 tiles of 256x256 together,
+  // one round, -3.3 % step time; below half a round in total the single launches, which
+  // split the contraction over workgroups, keep the device busier)
+  if (multi && total >= 128 && (double)((total + 255) / 256) < apart - 0.25) {
     // smallest first: measured 1 % faster than largest first at the Llama-3-8B shapes
     jpp_gemm_args order[4];
     for (int i = 0; i < w.n; ++i) order[i] = w.g[i];
