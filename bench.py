@@ -292,7 +292,7 @@ def main():
         ev.record()
         ends.append(ev)
 
-    cls = args.probe or (measured_dominant_class(wb, wl) if args.warmup else dominant_gemm_class(wl))
+    cls = args.probe or measured_dominant_class(wb, wl)
     for _ in range(args.warmup):
         paced_step()
     rt.sync()
