@@ -3,8 +3,10 @@
 The reference turns the members of a ``FusedTask`` into one task whose parts
 the compiler is free to overlap (src/jaxpp/core.py:2444-2513, ``fuse_groups``;
 src/jaxpp/schedules.py:48-54).  Here the forward member of a fused entry goes
-out on a second stream and the backward member on the first one; the streams
-meet again at the end of the entry, so everything after it sees both results.
+out on a second stream and the backward member on the first one - unless they
+belong to the same microbatch: that backward reads the forward's residuals, so
+the two run in order.  The streams meet again at the end of the entry, so
+everything after it sees both results.
 """
 from __future__ import annotations
 
@@ -30,9 +32,13 @@ class RankLoop:
         fused forwards on the loop's second stream."""
         ex = self.ex
         for entry in self.entries:
-            beside = self.overlap and len(entry) > 1 and \
-                any(pt.exec_kind is TaskType.FWD for pt in entry) and \
-                any(pt.exec_kind is not TaskType.FWD for pt in entry)
+            fwd_mbs = {pt.task.mubatch_idx for pt in entry if pt.exec_kind is TaskType.FWD}
+            bwd_mbs = {pt.task.mubatch_idx for pt in entry if pt.exec_kind is not TaskType.FWD}
+            # A fused entry may hold the forward and the backward of one microbatch (the last
+            # stage's, back to back): the backward reads what that forward leaves behind, so
+            # such members run one after the other; side by side only when the forward
+            # belongs to another microbatch than every backward of the entry.
+            beside = self.overlap and bool(fwd_mbs) and bool(bwd_mbs) and not (fwd_mbs & bwd_mbs)
             if beside:
                 self.fork.record(stream)
                 self.aux.wait(self.fork)

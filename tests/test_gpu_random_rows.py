@@ -1,0 +1,79 @@
+"""Seeded random draws of (layer family, schedule, microbatch count, rank, layers per chunk,
+stream / weight-gradient grouping mode): the rank's row on the GPU against the oracle's rank
+executor.  The fixed cases of test_gpu_stage.py name the combinations that matter; this sweep
+is for the ones nobody thought of (slot-ring corner cases, groups that never fill, ranks in the
+middle of a pipeline, a first stage whose backward is not split)."""
+import numpy as np
+import pytest
+
+import parity
+import test_gpu_stage as T
+
+from jaxpp_amd import runtime as rt
+from jaxpp_amd import schedules as S
+from jaxpp_amd.plan import make_rank_plan
+
+pytestmark = pytest.mark.gpu
+
+SPECS = [T.BERT, T.BERT_TANH, T.LLAMA, T.LLAMA_D64, T.DECODER, T.DECODER_D64]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    rt.require_gpu()
+
+
+def draw(seed):
+    """A valid (spec, schedule, n, rank, layers per chunk, mode) for this seed."""
+    rng = np.random.default_rng(1000 + seed)
+    while True:
+        spec = SPECS[rng.integers(len(SPECS))]
+        p = int(rng.integers(1, 5))                     # pipeline ranks
+        kind = rng.integers(6)
+        if kind == 0:
+            sched = S.Std1F1B(p)
+        elif kind == 1:
+            sched = S.GPipe(p)
+        elif kind == 2:
+            sched = S.Eager1F1B(p)
+        elif kind == 3:
+            sched = S.ZeroBubble(p)
+        elif kind == 4:
+            sched = S.Interleaved1F1B(p * int(rng.integers(2, 4)), p)
+        else:
+            sched = S.DualPipeV(2 * p, p)
+        n = int(rng.integers(1, 4)) * p if kind >= 4 else int(rng.integers(1, 8))
+        rank = int(rng.integers(p))
+        lpc = int(rng.integers(1, 3))
+        mode = ["two-streams", "one-stream", "group-2", "group-4"][rng.integers(4)]
+        try:
+            plan = make_rank_plan(sched, n, rank)
+        except Exception:                               # the schedule rejects the combination
+            continue
+        if len(plan.tasks) > 60:                        # keeps the oracle's share in seconds
+            continue
+        return spec, sched, n, rank, lpc, mode, plan
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_row_matches_oracle(seed):
+    spec, sched, n, rank, lpc, mode, plan = draw(seed)
+    print(f"seed {seed}: {spec.family} h{spec.hidden} {type(sched).__name__}"
+          f"{getattr(sched, 'num_stages', '')} n={n} rank={rank} lpc={lpc} {mode}: "
+          f"{len(plan.tasks)} tasks, {plan.n_chunks} chunk(s), max_live {plan.max_live}, "
+          f"split={plan.split_backward}", flush=True)
+    params = T.make_params(spec, plan.stages, lpc)
+    row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
+    ys_w, dxs_w, acc_w = T.run_on_oracle(spec, plan, params, row)
+    ys, dxs, grads = T.run_on_gpu(spec, plan, lpc, params, two_streams=mode == "two-streams",
+                                  wgrad_group={"group-2": 2, "group-4": 4}.get(mode, 0))
+    assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
+    for k in ys_w:
+        parity.close_stage(ys[k], ys_w[k], 2e-2, f"y{k}")
+    for k in dxs_w:
+        parity.close_stage(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
+    for s in plan.stages:
+        for li in range(lpc):
+            for pname, want in acc_w[s][li].items():
+                got = grads[s][li][pname]
+                parity.close_stage(got, want.reshape(got.shape), 2e-2, f"grad {s}/{li}/{pname}")

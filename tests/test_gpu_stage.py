@@ -118,6 +118,10 @@ CASES = [
     ("llama-dualpipev", LLAMA, S.DualPipeV(4, 2), 4, 1, 1),
     ("mixtral-1f1b", MIXTRAL, S.Std1F1B(2), 3, 1, 2),
     ("mixtral-dualpipev", MIXTRAL, S.DualPipeV(4, 2), 4, 0, 1),
+    # one rank holds all three stages: the table fuses the last stage's forward with its own
+    # backward, which must then run in order, not side by side
+    ("bert-interleaved-one-rank", BERT, S.Interleaved1F1B(3, 1), 2, 0, 2),
+    ("llama-interleaved-one-rank", LLAMA, S.Interleaved1F1B(2, 1), 3, 0, 1),
 ]
 
 
