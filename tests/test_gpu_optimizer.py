@@ -146,6 +146,47 @@ def test_stage_adam_after_loop(spec, two_streams):
     ex.close()
 
 
+def test_adam_step_runs_weight_gradients_that_are_still_held_back():
+    """With grouped weight gradients the last group of a row may be incomplete (3 microbatches
+    in pairs): the optimizer step must run what is pending before it reads the accumulators.
+    Same loop and step with and without grouping: the same weights (f32 reassociation aside)."""
+    spec, schedule, n_mb, lpc = LLAMA, S.Std1F1B(1), 3, 2
+    plan = make_rank_plan(schedule, n_mb, 0)
+    shape = (spec.tokens, spec.hidden)
+    results = []
+    for group in (0, 2):
+        ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True,
+                              False, wgrad_group=group)
+        for li in range(lpc):
+            ex.set_params(0, li, {k: L.bf16_round(v) for k, v in
+                                  init_layer_params(spec, 3, li, perturb=True).items()})
+        ex.optimizer_init()
+        bufs = {}
+
+        def io(pt, lane=0):
+            kind = "x" if pt.exec_kind is TaskType.FWD else "dy"
+            key = (kind, pt.task.stage_id, pt.task.mubatch_idx)
+            if key not in bufs:
+                bufs[key] = (rt.DeviceBuffer.from_f32_as_bf16(
+                    boundary_tensor(kind, pt.task.stage_id, pt.task.mubatch_idx, shape, 0)),
+                    rt.DeviceBuffer(spec.tokens * spec.hidden * 2))
+            return bufs[key][0].ptr, bufs[key][1].ptr
+
+        RankLoop(ex, plan).run(io)
+        if group:
+            assert ex.live_slots() == 1, "the third microbatch waits for a partner"
+        ex.adam_step(1, lr=1e-2, grad_scale=1.0 / n_mb)          # no join, no get_grads before it
+        rt.sync()
+        assert ex.live_slots() == 0
+        results.append([ex.get_opt_state(0, li) for li in range(lpc)])
+        ex.close()
+    for li in range(lpc):
+        for k in results[0][li]:
+            for what, a, b in zip(("weights", "m", "v"), results[0][li][k], results[1][li][k]):
+                assert np.abs(a).max() > 0
+                close(b, a, 1e-5, f"layer {li} {what}[{k}]")
+
+
 def test_stage_adam_needs_init():
     plan = make_rank_plan(S.Std1F1B(2), 2, 0)
     ex = rt.StageExecutor(BERT, plan.n_chunks, 1, plan.max_live, plan.split_backward, True, False)
