@@ -288,11 +288,12 @@ def test_lifetime_errors():
         rt.StageExecutor(LayerSpec("bert", 128, 4, 256, 128, 1), 1, 1, 1)
 
 
-@pytest.mark.parametrize("two_streams", [False, True], ids=["one-stream", "two-streams"])
+@pytest.mark.parametrize("two_streams,group", [(False, 0), (True, 0), (False, 2)],
+                         ids=["one-stream", "two-streams", "weight-gradients-in-pairs"])
 @pytest.mark.parametrize("spec,sched,n,rank", [(LLAMA, S.Interleaved1F1B(4, 2), 4, 0),
                                                (MIXTRAL, S.DualPipeV(4, 2), 4, 0)],
                          ids=["llama-interleaved", "mixtral-dualpipev"])
-def test_rank_row_replays_as_hip_graph(spec, sched, n, rank, two_streams):
+def test_rank_row_replays_as_hip_graph(spec, sched, n, rank, two_streams, group):
     """The entry points only enqueue, so a rank's row can be recorded into a HIP graph.  Every
     replay - with eager work and synchronisations between the replays - must reproduce the
     eager run bit for bit."""
@@ -301,7 +302,7 @@ def test_rank_row_replays_as_hip_graph(spec, sched, n, rank, two_streams):
     params = make_params(spec, plan.stages, lpc)
     shape = (spec.tokens, spec.hidden)
     ex = rt.StageExecutor(spec, plan.n_chunks, lpc, plan.max_live, plan.split_backward, True,
-                          two_streams)
+                          two_streams, wgrad_group=group)
     for c, stage in enumerate(plan.stages):
         ex.set_params(c, 0, params[stage][0])
     bufs = {}
