@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 import parity
+import test_gpu_full_size as F
 import test_gpu_stage as T
 
 from jaxpp_amd import runtime as rt
@@ -15,7 +16,7 @@ from jaxpp_amd.plan import make_rank_plan
 
 pytestmark = pytest.mark.gpu
 
-SPECS = [T.BERT, T.BERT_TANH, T.LLAMA, T.LLAMA_D64, T.DECODER, T.DECODER_D64]
+SPECS = [T.BERT, T.BERT_TANH, T.LLAMA, T.LLAMA_D64, T.DECODER, T.DECODER_D64, T.MIXTRAL]
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -55,13 +56,19 @@ def draw(seed):
         return spec, sched, n, rank, lpc, mode, plan
 
 
-@pytest.mark.parametrize("seed", range(64))
+@pytest.mark.parametrize("seed", range(80))
 def test_random_row_matches_oracle(seed):
     spec, sched, n, rank, lpc, mode, plan = draw(seed)
     print(f"seed {seed}: {spec.family} h{spec.hidden} {type(sched).__name__}"
           f"{getattr(sched, 'num_stages', '')} n={n} rank={rank} lpc={lpc} {mode}: "
           f"{len(plan.tasks)} tasks, {plan.n_chunks} chunk(s), max_live {plan.max_live}, "
           f"split={plan.split_backward}", flush=True)
+    if spec.family == "mixtral":
+        # top-2 routing is discontinuous: the oracle is held to the routing the device chose
+        # (checked to differ from its own only at near ties), one stream
+        F.check_rank_row(spec, sched, n, rank, lpc,
+                         wgrad_group={"group-2": 2, "group-4": 4}.get(mode, 0))
+        return
     params = T.make_params(spec, plan.stages, lpc)
     row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
     ys_w, dxs_w, acc_w = T.run_on_oracle(spec, plan, params, row)
@@ -72,8 +79,4 @@ def test_random_row_matches_oracle(seed):
         parity.close_stage(ys[k], ys_w[k], 2e-2, f"y{k}")
     for k in dxs_w:
         parity.close_stage(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
-    for s in plan.stages:
-        for li in range(lpc):
-            for pname, want in acc_w[s][li].items():
-                got = grads[s][li][pname]
-                parity.close_stage(got, want.reshape(got.shape), 2e-2, f"grad {s}/{li}/{pname}")
+    T.assert_grads_match(spec, plan, lpc, grads, acc_w)

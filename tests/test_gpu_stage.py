@@ -106,6 +106,33 @@ def make_params(spec, stages, layers_per_chunk):
                 for li in range(layers_per_chunk)] for s in stages}
 
 
+def assert_grads_match(spec, plan, lpc, grads, acc_w):
+    """The accumulated gradients of a rank against the oracle's, every parameter."""
+    bad = []
+    for s in plan.stages:
+        for li in range(lpc):
+            for pname, want in acc_w[s][li].items():
+                got = grads[s][li][pname]
+                want = want.reshape(got.shape)
+                err = float(np.abs(got - want).max()) / (float(np.abs(want).max()) + 1e-30)
+                fro = float(np.linalg.norm(got - want) / (np.linalg.norm(want) + 1e-30))
+                # Top-2 expert selection is discontinuous: a token whose second and third
+                # router logits are within bf16 rounding of each other may go to another
+                # expert than in the oracle (1-2 of 256 tokens flip between the oracle's own
+                # bf16 and f32 numerics).  One token's outer product then lands in another
+                # expert's gradient, so router and expert weights are held to 2e-2 in the
+                # Frobenius norm and 1e-1 in the max norm; all else to 2e-2 in the max norm.
+                routed = spec.family == "mixtral" and pname in ("Wr", "Wgu", "Wd")
+                n_bad, n_el, worst = parity.violations(got, want, 2e-2)
+                ok = (fro <= 2e-2 and err <= 1e-1) if routed else (
+                    err <= 2e-2 and n_bad <= parity.STAGE_BAD_FRAC * n_el and worst <= parity.MAX_EXCESS)
+                if not (np.isfinite(got).all() and ok):
+                    bad.append(f"grad {s}/{li}/{pname}: max err {err:.4g}, frobenius {fro:.4g}, "
+                               f"{n_bad} of {n_el} elements outside the elementwise bound "
+                               f"(worst {worst:.3g} x)")
+    assert not bad, "\n".join(bad)
+
+
 CASES = [
     ("bert-1f1b", BERT, S.Std1F1B(2), 4, 0, 2),
     ("bert-tanh-zb", BERT_TANH, S.ZeroBubble(2), 3, 1, 1),
@@ -139,29 +166,7 @@ def test_stage_matches_oracle(name, spec, sched, n, rank, lpc, two_streams):
         parity.close_stage(ys[k], ys_w[k], 2e-2, f"y{k}")
     for k in dxs_w:
         parity.close_stage(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
-    bad = []
-    for s in plan.stages:
-        for li in range(lpc):
-            for pname, want in acc_w[s][li].items():
-                got = grads[s][li][pname]
-                want = want.reshape(got.shape)
-                err = float(np.abs(got - want).max()) / (float(np.abs(want).max()) + 1e-30)
-                fro = float(np.linalg.norm(got - want) / (np.linalg.norm(want) + 1e-30))
-                # Top-2 expert selection is discontinuous: a token whose second and third
-                # router logits are within bf16 rounding of each other may go to another
-                # expert than in the oracle (1-2 of 256 tokens flip between the oracle's own
-                # bf16 and f32 numerics).  One token's outer product then lands in another
-                # expert's gradient, so router and expert weights are held to 2e-2 in the
-                # Frobenius norm and 1e-1 in the max norm; all else to 2e-2 in the max norm.
-                routed = spec.family == "mixtral" and pname in ("Wr", "Wgu", "Wd")
-                n_bad, n_el, worst = parity.violations(got, want, 2e-2)
-                ok = (fro <= 2e-2 and err <= 1e-1) if routed else (
-                    err <= 2e-2 and n_bad <= parity.STAGE_BAD_FRAC * n_el and worst <= parity.MAX_EXCESS)
-                if not (np.isfinite(got).all() and ok):
-                    bad.append(f"grad {s}/{li}/{pname}: max err {err:.4g}, frobenius {fro:.4g}, "
-                               f"{n_bad} of {n_el} elements outside the elementwise bound "
-                               f"(worst {worst:.3g} x)")
-    assert not bad, "\n".join(bad)
+    assert_grads_match(spec, plan, lpc, grads, acc_w)
 
 
 def test_task_order_does_not_change_gradients():
