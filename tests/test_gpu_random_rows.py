@@ -16,7 +16,11 @@ from jaxpp_amd.plan import make_rank_plan
 
 pytestmark = pytest.mark.gpu
 
-SPECS = [T.BERT, T.BERT_TANH, T.LLAMA, T.LLAMA_D64, T.DECODER, T.DECODER_D64, T.MIXTRAL]
+import test_gpu_f32 as F32  # noqa: E402
+
+# bf16 stages of every family, and float32 stages (held to 1e-4; wgrad grouping is a bf16 mode)
+SPECS = [T.BERT, T.BERT_TANH, T.LLAMA, T.LLAMA_D64, T.DECODER, T.DECODER_D64, T.MIXTRAL,
+         F32.BERT_D64_F32, F32.DECODER_F32, F32.LLAMA_F32, F32.LLAMA_D64_F32]
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -47,6 +51,8 @@ def draw(seed):
         rank = int(rng.integers(p))
         lpc = int(rng.integers(1, 3))
         mode = ["two-streams", "one-stream", "group-2", "group-4"][rng.integers(4)]
+        if spec.dtype == "f32" and mode.startswith("group"):
+            mode = "one-stream"
         try:
             plan = make_rank_plan(sched, n, rank)
         except Exception:                               # the schedule rejects the combination
@@ -56,7 +62,7 @@ def draw(seed):
         return spec, sched, n, rank, lpc, mode, plan
 
 
-@pytest.mark.parametrize("seed", range(80))
+@pytest.mark.parametrize("seed", range(96))
 def test_random_row_matches_oracle(seed):
     spec, sched, n, rank, lpc, mode, plan = draw(seed)
     print(f"seed {seed}: {spec.family} h{spec.hidden} {type(sched).__name__}"
@@ -68,6 +74,25 @@ def test_random_row_matches_oracle(seed):
         # (checked to differ from its own only at near ties), one stream
         F.check_rank_row(spec, sched, n, rank, lpc,
                          wgrad_group={"group-2": 2, "group-4": 4}.get(mode, 0))
+        return
+    if spec.dtype == "f32":
+        from jaxpp_amd.model import init_layer_params
+        params = {s: [init_layer_params(spec, 3, s * lpc + li, perturb=True) for li in range(lpc)]
+                  for s in plan.stages}
+        row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
+        ys_w, dxs_w, acc_w = T.run_on_oracle(spec, plan, params, row)
+        ys, dxs, grads = T.run_on_gpu(spec, plan, lpc, params, two_streams=mode == "two-streams")
+        assert set(ys) == set(ys_w) and set(dxs) == set(dxs_w)
+        for k in ys_w:
+            parity.close(ys[k], ys_w[k].astype(np.float64), 1e-4, f"y{k}")
+        for k in dxs_w:
+            parity.close(dxs[k], dxs_w[k].astype(np.float64), 1e-4, f"dx{k}")
+        for s in plan.stages:
+            for li in range(lpc):
+                for pname, want in acc_w[s][li].items():
+                    got = grads[s][li][pname]
+                    parity.close(got, want.reshape(got.shape).astype(np.float64), 1e-4,
+                                 f"grad {s}/{li}/{pname}")
         return
     params = T.make_params(spec, plan.stages, lpc)
     row = S.preprocess_schedule_tasks(sched.tasks(n), 0, False)[rank]
