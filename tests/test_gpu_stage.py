@@ -258,6 +258,38 @@ def test_grouped_weight_gradients_hold_their_slots():
         rt.StageExecutor(spec, 1, 1, 1, False, True, True, wgrad_group=2)
 
 
+def test_routing_readback():
+    """jpp_stage_routing: the experts and gate weights a forward chose, while the microbatch's
+    residuals are live; errors for stages without experts, unknown layers, dead microbatches."""
+    spec = MIXTRAL
+    ex = rt.StageExecutor(spec, 1, 2, 1, False, True, False)
+    for li in range(2):
+        ex.set_params(0, li, make_params(spec, [0], 2)[0][li])
+    buf = ex.upload_activation(boundary_tensor("x", 0, 0, (spec.tokens, spec.hidden), 0))
+    out = ex.new_activation()
+    with pytest.raises(rt.JppError, match="holds no residuals"):
+        ex.routing(0, 0, 0)
+    ex.run_task(TaskType.FWD, 0, 0, buf.ptr, out.ptr)
+    for li in range(2):
+        ids, gates = ex.routing(0, 0, li)
+        assert ids.min() >= 0 and ids.max() < spec.n_experts
+        assert (ids[:, 0] != ids[:, 1]).all(), "two different experts per token"
+        np.testing.assert_allclose(gates.sum(1), 1.0, rtol=0, atol=1e-5)
+        assert (gates[:, 0] >= gates[:, 1]).all(), "experts in descending order of their logits"
+    with pytest.raises(rt.JppError, match="out of range"):
+        ex.routing(0, 0, 2)
+    dy = ex.upload_activation(boundary_tensor("dy", 0, 0, (spec.tokens, spec.hidden), 0))
+    ex.run_task(TaskType.BWD, 0, 0, dy.ptr, out.ptr)
+    rt.sync()
+    with pytest.raises(rt.JppError, match="holds no residuals"):
+        ex.routing(0, 0, 0)
+    ex.close()
+    ex = rt.StageExecutor(LLAMA, 1, 1, 1, False, True, False)
+    with pytest.raises(rt.JppError, match="not a mixture-of-experts stage"):
+        ex.routing(0, 0, 0)
+    ex.close()
+
+
 def test_unfused_accumulate_path_is_close():
     spec, n = BERT, 2
     params = make_params(spec, [0], 1)
