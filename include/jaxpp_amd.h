@@ -106,12 +106,6 @@ int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, doub
  * moe_combine_fwd, moe_bwd_prepare, moe_combine_bwd, moe_router_wgrad. */
 int jpp_probe_class(int index, const char** name, int64_t* launches, double* total_ms,
                     double* total_flops, double* total_bytes);
-/* No counterpart in the reference: a measurement aid.  TFLOP/s this device sustains on
- * a register-only loop of bf16 MFMAs on every SIMD (shape 32: 32x32x16, 16: 16x16x32;
- * operands all zero, or random and different from one MFMA to the next as in a GEMM).
- * The clock under load depends on how many operand bits toggle, so the second figure is
- * the ceiling a real GEMM can approach.  Blocks the host (null stream; two runs of about 0.3 us per iteration, the second timed). */
-int jpp_mfma_rate(int shape, int random_operands, int64_t iters, double* tflops);
 
 /* ---- GEMM: stands in for the `dot_general`s of a stage task ----------------
  * C[M,N] = epilogue( sum_k Aop[m,k] * Bop[n,k] ), bf16 operands, fp32 MFMA

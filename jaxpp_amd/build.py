@@ -15,7 +15,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libjaxpp_amd.so")
 SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "attention_dkv.hip", "elementwise.hip",
-           "moe.hip", "optimizer.hip", "diagnostics.hip", "f32_ops.hip", "stage.hip"]
+           "moe.hip", "optimizer.hip", "f32_ops.hip", "stage.hip"]
+# measurement aids: a library of their own beside the product library
+DIAG_LIB = os.path.join(LIBDIR, "libjaxpp_amd_diag.so")
+DIAG_SOURCES = ["diagnostics.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          # packed fp32 ops are kept out of generated code on this hardware pool
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -67,10 +70,16 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(compile_one, SOURCES))
+        all_objs = list(ex.map(compile_one, SOURCES + DIAG_SOURCES))
+    objs, diag_objs = all_objs[:len(SOURCES)], all_objs[len(SOURCES):]
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
     if verbose:
         print(f"[jaxpp_amd.build] linked {LIB}", flush=True)
+    # resolves jpp_set_error from the product library next to it
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", DIAG_LIB, *diag_objs,
+          "-L" + LIBDIR, "-ljaxpp_amd", "-Wl,-rpath,$ORIGIN"])
+    if verbose:
+        print(f"[jaxpp_amd.build] linked {DIAG_LIB}", flush=True)
     return LIB
 
 

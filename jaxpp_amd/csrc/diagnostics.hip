@@ -4,6 +4,7 @@
 // to it is the device's (clock under load depends on how many operand bits toggle) and how
 // much is the kernels'.
 #include "common.h"
+#include "../../include/jaxpp_amd_diag.h"
 
 namespace {
 

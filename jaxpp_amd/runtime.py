@@ -107,7 +107,7 @@ EXPORTS = [
     "jpp_device_sync",
     "jpp_event_create", "jpp_event_destroy", "jpp_event_record", "jpp_event_sync",
     "jpp_event_elapsed_ms", "jpp_mem_info", "jpp_workspace_bytes", "jpp_graph_begin", "jpp_graph_end", "jpp_graph_launch",
-    "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_probe_class", "jpp_mfma_rate",
+    "jpp_graph_destroy", "jpp_probe_begin", "jpp_probe_end", "jpp_probe_class",
     "jpp_gemm_bf16", "jpp_gemm_bf16_multi", "jpp_attn_fwd", "jpp_attn_bwd",
     "jpp_gemm_f32", "jpp_attn_fwd_f32", "jpp_attn_bwd_f32", "jpp_norm_fwd_f32", "jpp_norm_bwd_f32",
     "jpp_colsum_accum_f32", "jpp_mse_loss_f32", "jpp_rope_f32",
@@ -126,6 +126,22 @@ EXPORTS = [
 
 def lib_path() -> str:
     return _LIB_PATH
+
+
+_diag = None
+
+
+def load_diag():
+    """The measurement aids (libjaxpp_amd_diag.so, next to the product library)."""
+    global _diag
+    if _diag is None:
+        load()                                        # its error reporting lives there
+        path = os.path.join(os.path.dirname(_LIB_PATH), "libjaxpp_amd_diag.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python -m jaxpp_amd.build`")
+        _diag = C.CDLL(path)
+        _diag.jpp_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int64, C.POINTER(C.c_double)]
+    return _diag
 
 
 def load():
@@ -232,7 +248,6 @@ def load():
     lib.jpp_stage_live_slots.argtypes = [C.c_void_p]
     lib.jpp_stage_routing.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                       C.c_void_p]
-    lib.jpp_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int64, C.POINTER(C.c_double)]
     lib.jpp_adam_step.argtypes = [C.c_void_p, C.POINTER(AdamArgs)]
     lib.jpp_stage_optimizer_init.argtypes = [C.c_void_p, C.c_void_p]
     lib.jpp_stage_opt_ptr.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
@@ -498,7 +513,7 @@ def gemm_multi(problems, stream=None):
 def mfma_rate(shape: int, random_operands: bool, iters: int = 100000) -> float:
     """TFLOP/s of a register-only MFMA loop on every SIMD (see jpp_mfma_rate)."""
     out = C.c_double(0.0)
-    check(load().jpp_mfma_rate(shape, int(random_operands), iters, C.byref(out)))
+    check(load_diag().jpp_mfma_rate(shape, int(random_operands), iters, C.byref(out)))
     return out.value
 
 

@@ -27,6 +27,17 @@ def test_library_exports_every_declared_symbol():
     assert sorted(rt.EXPORTS) == names, "runtime.EXPORTS and the header disagree"
 
 
+def test_diagnostics_live_in_a_library_of_their_own():
+    """jpp_mfma_rate (a measurement aid with no counterpart in the reference) is declared in
+    include/jaxpp_amd_diag.h and exported by libjaxpp_amd_diag.so, not by the product library."""
+    diag_header = os.path.join(ROOT, "include", "jaxpp_amd_diag.h")
+    names = sorted(set(re.findall(r"\b(jpp_[a-z0-9_]+)\s*\(", open(diag_header).read())))
+    assert names == ["jpp_mfma_rate"]
+    assert "jpp_mfma_rate" not in declared_symbols()
+    assert not hasattr(ctypes.CDLL(rt.lib_path()), "jpp_mfma_rate")
+    assert hasattr(rt.load_diag(), "jpp_mfma_rate")
+
+
 def test_error_convention_without_gpu():
     lib = rt.load()
     assert lib.jpp_version() == 100
