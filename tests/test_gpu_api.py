@@ -233,3 +233,18 @@ def test_treduce_i_with_an_explicit_length():
     for k, v in want_acc[0][0].items():
         close(grad[k], v.reshape(grad[k].shape), f"grad {k}")
     train_step.close()
+
+
+def test_the_example_script_runs_and_learns():
+    """examples/basic.py: Std1F1B against the microbatches in turn, bit for bit (checked inside
+    the script), Adam applied through the public API; the loss on its fixed batch goes down."""
+    import importlib.util
+    import os
+    rt.require_gpu()
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "examples", "basic.py")
+    spec = importlib.util.spec_from_file_location("example_basic", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for argv in (["--steps", "4"], ["--steps", "3", "--dtype", "f32", "--pp", "3", "--num-ubatches", "6"]):
+        history = mod.main(argv)
+        assert all(np.isfinite(history)) and history[-1] < history[0], history
