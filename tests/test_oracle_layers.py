@@ -294,3 +294,84 @@ def test_bf16_sensitivity_of_a_70b_shaped_layer():
         fracs.append(n_bad / n)
         assert worst <= parity.MAX_EXCESS
     assert fracs[0] <= 1e-5 and 5e-5 <= fracs[1] <= 1e-3 and 3e-4 <= fracs[2] <= 4e-3, fracs
+
+
+def test_attention_operand_rounding_is_what_it_says():
+    """`rt` of attention_fwd / attention_bwd: the probabilities (and, backward, the score
+    cotangents) are rounded where they become operands of the next product - after the row sum
+    (forward) and from the exact log-sum-exp (backward).  Against an independent per-row
+    computation on a tiny case, to 1e-12."""
+    rng = np.random.default_rng(8)
+    B, S, H, d = 1, 6, 2, 4
+    q, k, v, do = (rng.standard_normal((B, S, H, d)) for _ in range(4))
+    rt = L.bf16_round
+    for causal in (False, True):
+        o, lse = L.attention_fwd(q, k, v, causal, np.float64, rt)
+        o_exact, lse_exact = L.attention_fwd(q, k, v, causal, np.float64)
+        np.testing.assert_allclose(lse, lse_exact, rtol=1e-14)          # the sum is not rounded
+        assert np.abs(o - o_exact).max() < 2 ** -7 * np.abs(v).max()
+        assert np.abs(o - o_exact).max() > 0, "rounding the probabilities must show"
+        dq, dk, dv = L.attention_bwd(q, k, v, o_exact, do, lse_exact, causal, np.float64, rt)
+        for h in range(H):
+            for i in range(S):
+                hi = i + 1 if causal else S
+                sc = np.array([q[0, i, h] @ k[0, j, h] for j in range(hi)]) / math.sqrt(d)
+                w = np.exp(sc - sc.max())
+                want = sum(rt(w)[j].astype(np.float64) * v[0, j, h] for j in range(hi)) / w.sum()
+                np.testing.assert_allclose(o[0, i, h], want, rtol=1e-12)
+        # backward, row by row: p from the exact lse, dS rounded, P rounded for dV only
+        scale = 1 / math.sqrt(d)
+        dq_w, dk_w, dv_w = np.zeros_like(q[0]), np.zeros_like(k[0]), np.zeros_like(v[0])
+        for h in range(H):
+            for i in range(S):
+                hi = i + 1 if causal else S
+                p = np.array([math.exp(q[0, i, h] @ k[0, j, h] * scale - lse_exact[0, h, i]) for j in range(hi)])
+                dp = np.array([do[0, i, h] @ v[0, j, h] for j in range(hi)])
+                delta = do[0, i, h] @ o_exact[0, i, h]
+                ds = rt(p * (dp - delta) * scale).astype(np.float64)
+                pr = rt(p).astype(np.float64)
+                for j in range(hi):
+                    dq_w[i, h] += ds[j] * k[0, j, h]
+                    dk_w[j, h] += ds[j] * q[0, i, h]
+                    dv_w[j, h] += pr[j] * do[0, i, h]
+        np.testing.assert_allclose(dq[0], dq_w, rtol=1e-12, atol=1e-14)
+        np.testing.assert_allclose(dk[0], dk_w, rtol=1e-12, atol=1e-14)
+        np.testing.assert_allclose(dv[0], dv_w, rtol=1e-12, atol=1e-14)
+
+
+def test_forced_routing_of_the_mixture_layer():
+    """layer_fwd(forced_ids=...): forcing the layer's own choice changes nothing; forcing other
+    experts for a token gives that token the gated sum of exactly those experts, gates =
+    softmax over their two logits (computed by hand), and leaves every other token alone."""
+    spec = next(s for s in SPECS.values() if s.family == "mixtral")
+    cfg = cfg_of(spec)
+    rng = np.random.default_rng(4)
+    p = {k: v.astype(np.float64) for k, v in init_layer_params(spec, 1, 0, perturb=True).items()}
+    x = rng.standard_normal((spec.tokens, spec.hidden))
+    nm = L.Numerics.f64()
+    y0, st0 = L.layer_fwd(cfg, p, x, nm)
+    y1, st1 = L.layer_fwd(cfg, p, x, nm, forced_ids=st0["ids"])
+    np.testing.assert_array_equal(y1, y0)
+    np.testing.assert_array_equal(st1["own_ids"], st0["ids"])
+    t = 3
+    others = [e for e in range(cfg.n_experts) if e not in st0["ids"][t]][:cfg.top_k]
+    forced = st0["ids"].copy()
+    forced[t] = others
+    y2, st2 = L.layer_fwd(cfg, p, x, nm, forced_ids=forced)
+    same = np.ones(spec.tokens, bool)
+    same[t] = False
+    np.testing.assert_array_equal(y2[same], y0[same])
+    logits = st2["logits"][t]
+    sel = np.array([logits[e] for e in others])
+    g = np.exp(sel - sel.max())
+    g /= g.sum()
+    np.testing.assert_allclose(st2["gates"][t], g, rtol=1e-12)
+    # the token's expert outputs by hand: n2 -> gate/up -> SwiGLU -> down, per forced expert
+    # (y = h1 + sum_k gate_k * expert_k(n2); h1 is y0 minus the token's own expert sum)
+    own = sum(st0["gates"][t, kk] * st0["eo"][t, kk] for kk in range(cfg.top_k))
+    h1 = y0[t] - own
+    for kk, e in enumerate(others):
+        np.testing.assert_allclose(st2["eo"][t, kk],
+                                   L.swiglu(st2["gu"][t, kk][None], cfg.ffn)[0] @ p["Wd"][e], rtol=1e-10)
+    want = h1 + sum(g[kk] * st2["eo"][t, kk] for kk in range(cfg.top_k))
+    np.testing.assert_allclose(y2[t], want, rtol=1e-10)

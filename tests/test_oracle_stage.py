@@ -140,3 +140,34 @@ def test_adam_step_matches_torch():
         opt.step()
         p = O.adam_step(p, {"w": g}, m, v, step)
         np.testing.assert_allclose(p["w"], tp.detach().numpy(), rtol=2e-6, atol=1e-7)
+
+
+def test_rank_oracle_reports_router_margins_and_forced_changes():
+    """RankOracle.router_margin is the gap between the last selected router logit and the best
+    one left out (by hand from the stashed logits); forcing another routing is recorded per
+    layer in forced_changes, and only for the tokens whose set of experts changed."""
+    from jaxpp_amd.model import LayerSpec, init_layer_params
+    spec = LayerSpec("mixtral", 128, 1, 128, 64, 1, n_kv_heads=1, head_dim=128, causal=True,
+                     rope_theta=1e4, eps=1e-5, n_experts=4, top_k=2)
+    cfg = L.LayerCfg(**spec.as_dict())
+    params = {0: [init_layer_params(spec, 2, li, perturb=True) for li in range(2)]}
+    x = np.random.default_rng(0).standard_normal((spec.tokens, spec.hidden)).astype(np.float32)
+    ro = O.RankOracle(cfg, params, L.Numerics.f32())
+    ro.fwd(0, 0, x)
+    for li in range(2):
+        logits = ro.stash[0, 0][li]["logits"].astype(np.float64)
+        srt = np.sort(logits, -1)
+        np.testing.assert_array_equal(ro.router_margin[0, 0][li], srt[:, -2] - srt[:, -3])
+        assert (ro.router_margin[0, 0][li] >= 0).all()
+    own = [st["ids"].copy() for st in ro.stash[0, 0]]
+    # same experts in the other order: no change; token 5 of layer 1 to two other experts: one
+    forced = [own[0][:, ::-1].copy(), own[1].copy()]
+    forced[1][5] = [e for e in range(4) if e not in own[1][5]]
+    ro2 = O.RankOracle(cfg, params, L.Numerics.f32())
+    ro2.forced_ids[0, 0] = forced
+    ro2.fwd(0, 0, x)
+    assert not ro2.forced_changes[0, 0][0].any()
+    want = np.zeros(spec.tokens, bool)
+    want[5] = True
+    # layer 1 sees layer 0's output, which the reordering left unchanged
+    np.testing.assert_array_equal(ro2.forced_changes[0, 0][1], want)
