@@ -171,3 +171,48 @@ def test_rank_oracle_reports_router_margins_and_forced_changes():
     want[5] = True
     # layer 1 sees layer 0's output, which the reordering left unchanged
     np.testing.assert_array_equal(ro2.forced_changes[0, 0][1], want)
+
+
+def test_sequential_loop_with_targets_and_mixed_layer_families():
+    """treduce_sequential(targets=..., layer_cfgs=...): the loss is mean((out - target)^2) / n
+    against the given target (by hand from a forward pass), and the accumulated gradients are
+    the derivative of the summed losses - central finite differences in float64 on parameters
+    of both layers of a stage that holds a post-LN encoder layer and a pre-LN decoder block."""
+    bert = LayerSpec("bert", 32, 2, 64, 8, 1, eps=1e-12)
+    dec = LayerSpec("decoder", 32, 2, 64, 8, 1, causal=True, eps=1e-6, gelu_tanh=True)
+    cfgs = {0: [L.LayerCfg(**bert.as_dict()), L.LayerCfg(**dec.as_dict())]}
+    nm = L.Numerics.f64()
+    rng = np.random.default_rng(3)
+    params = [{k: v.astype(np.float64) for k, v in init_layer_params(bert, 5, 0, perturb=True).items()},
+              {k: v.astype(np.float64) for k, v in init_layer_params(dec, 5, 1, perturb=True).items()}]
+    xs = [rng.standard_normal((bert.tokens, bert.hidden)) for _ in range(3)]
+    ts = [rng.standard_normal((bert.tokens, bert.hidden)) for _ in range(3)]
+
+    def total(ps):                      # the summed losses in float64, from forward passes
+        out = 0.0
+        for x, t in zip(xs, ts):
+            a, _ = L.layer_fwd(cfgs[0][0], ps[0], x, nm)
+            a, _ = L.layer_fwd(cfgs[0][1], ps[1], a, nm)
+            out += ((a - t) ** 2).mean() / 3
+        return out
+
+    losses, acc = O.treduce_sequential(cfgs[0][0], [params], xs, nm, targets=ts, layer_cfgs=cfgs)
+    for m in range(3):
+        a, _ = L.layer_fwd(cfgs[0][0], params[0], xs[m], nm)
+        a, _ = L.layer_fwd(cfgs[0][1], params[1], a, nm)
+        np.testing.assert_allclose(losses[m], ((a - ts[m]) ** 2).mean() / 3, rtol=1e-6)
+        assert abs(losses[m] - ((a - xs[m]) ** 2).mean() / 3) > 1e-3 * losses[m], "not the input"
+    eps = 1e-6
+    for li, name, idx in [(0, "W1", (3, 5)), (0, "ln2_g", (7,)), (1, "Wqkv", (2, 11)), (1, "b2", (4,))]:
+        ps = [dict(p) for p in params]
+        w = ps[li][name].copy()
+        w[idx] += eps
+        ps[li][name] = w
+        up = total(ps)
+        w = w.copy()
+        w[idx] -= 2 * eps
+        ps[li][name] = w
+        down = total(ps)
+        got = acc[0][li][name].reshape(params[li][name].shape)[idx]
+        # the accumulators are f32: compare at their resolution
+        np.testing.assert_allclose(got, (up - down) / (2 * eps), rtol=2e-4, atol=1e-9)
