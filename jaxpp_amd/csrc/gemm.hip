@@ -387,12 +387,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
 #pragma unroll
         for (int i = 0; i < TMH; ++i) fx[0][i] = TileA::frag16(na, row_x + i * 16, 0, lane);
       }
-#ifdef JPP_SCHED_FENCE
-      // the fragment reads above are issued before this block's MFMAs and stay there: the
-      // compiler's scheduler would otherwise sink each read to just before its first use and
-      // expose the LDS latency in front of every few MFMAs
-      __builtin_amdgcn_sched_barrier(0);
-#endif
       // the refill of the retired stage is spread over this block's MFMAs: a wave that
       // issues its loads back to back waits on the memory pipeline with its MFMAs behind it
       constexpr int PARTS = TMH < IA && TMH < IB ? TMH : (IA < IB ? IA : IB);
@@ -430,9 +424,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
           }
         }
       }
-#ifdef JPP_SCHED_FENCE
-      __builtin_amdgcn_sched_barrier(0);
-#endif
     }
     if constexpr (EPI == JPP_EPI_ACC_F32) {
       if (stream_c && kt < NBT)
