@@ -392,8 +392,14 @@ def moe_setup(rng, T, h):
 
 
 def test_moe_routing_and_permutation():
-    rng = np.random.default_rng(11)
-    T, h, E = 1000, 256, 8
+    check_moe(11, 1000, 256)
+
+
+def check_moe(seed, T, h):
+    """Routing, the token permutation it implies, gather / combine and their backward, the
+    router's weight gradient: T tokens of width h over the 8 experts."""
+    rng = np.random.default_rng(seed)
+    E = 8
     lib, a, b, x, wr, cap = moe_setup(rng, T, h)
     rt.check(lib.jpp_moe_route(None, C.byref(a)))
     rt.sync()

@@ -119,3 +119,12 @@ def test_random_norm(seed):
     rows = int(rng.integers(1, 1500))
     cols = int(rng.integers(16, 1025)) * 8
     K.test_norm_fwd_bwd(ln, rows, cols)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_moe(seed):
+    rng = np.random.default_rng(6000 + seed)
+    T = int(rng.integers(1, 3000))                 # any count: groups are padded to 256 rows
+    h = int(rng.integers(2, 65)) * 8
+    print(f"seed {seed}: {T} tokens of width {h}", flush=True)
+    K.check_moe(seed, T, h)
