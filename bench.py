@@ -221,8 +221,8 @@ def main():
                          "of it (no host launch work in the timed region); the per-kernel probe "
                          "cannot see inside a replay, so `roofline` then comes from one more "
                          "eager step after the timed ones.  auto: for narrow layers (hidden < "
-                         "2048: thousands of small launches per step, +3 %), not for wide ones "
-                         "(the GPU is busy 99.8 % of an eager step)")
+                         "2048: thousands of small launches per step, +3 %%), not for wide ones "
+                         "(the GPU is busy 99.8 %% of an eager step)")
     ap.add_argument("--extra-fills", type=int, default=0,
                     help="diagnostic: after every step, clear a 6 GiB scratch buffer this many "
                          "times (about 2 ms each of memory-bound, low-power work).  The step "
