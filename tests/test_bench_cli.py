@@ -49,14 +49,8 @@ def test_unknown_workload_is_an_error():
 def test_without_a_gpu_the_run_fails_loudly():
     """No CPU path stands in for the HIP library: on a host without a device the script ends
     with an error and prints no result line."""
-    import ctypes
-    try:
-        hip = ctypes.CDLL("libamdhip64.so")
-        n = ctypes.c_int(0)
-        if hip.hipGetDeviceCount(ctypes.byref(n)) == 0 and n.value > 0:
-            pytest.skip("a GPU is visible")
-    except OSError:
-        pass
+    if os.path.exists("/dev/kfd"):      # asked of the file system: no HIP call in this process
+        pytest.skip("a GPU may be visible")
     r = run("--no-cpu-baseline", "--steps", "1", "--warmup", "0")
     assert r.returncode != 0
     assert "GPU" in r.stderr
