@@ -141,8 +141,11 @@ def measured_dominant_class(wb, wl) -> str:
     with rt.probe("*") as pr:
         wb.step()
         rt.sync()
-    acc = {k: v[1] for k, v in pr.classes.items() if k.startswith("gemm_tn_accf32")}
-    return max(acc, key=acc.get) if acc else dominant_gemm_class(wl)
+    for prefix in ("gemm_tn_accf32", "gemm_tn_", "gemm_"):   # (no fused accumulate: the bf16 form)
+        acc = {k: v[1] for k, v in pr.classes.items() if k.startswith(prefix)}
+        if acc:
+            return max(acc, key=acc.get)
+    return dominant_gemm_class(wl)
 
 
 def default_wgrad_group(wl, two_streams: bool) -> int:
