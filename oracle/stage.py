@@ -140,11 +140,12 @@ class RankOracle:
 # whole model: sequential loop and scheduled pipeline (cfg "CPU plumbing")
 # ---------------------------------------------------------------------------
 def treduce_sequential(cfg, stage_layers, xs, nm, round_wgrad=False, targets=None,
-                       layer_cfgs=None):
+                       layer_cfgs=None, preds=None):
     """The loop as ``treduce`` defines it: microbatches in order, every stage
     forward then backward; losses concatenated, gradients summed.  The loss
     compares the last stage's output with ``targets[m]`` (default: the
-    microbatch itself, as in the reference's examples)."""
+    microbatch itself, as in the reference's examples).  A list passed as
+    ``preds`` receives the last stage's output of every microbatch, in order."""
     n = len(xs)
     targets = xs if targets is None else targets
     ro = RankOracle(cfg, dict(enumerate(stage_layers)), nm, round_wgrad, layer_cfgs)
@@ -154,6 +155,8 @@ def treduce_sequential(cfg, stage_layers, xs, nm, round_wgrad=False, targets=Non
         a = xs[m]
         for s in range(S):
             a = ro.fwd(s, m, a)
+        if preds is not None:
+            preds.append(a)
         losses[m], d = L.mse_loss(a, targets[m], n, nm.acc)
         d = nm.rt(d.astype(np.float32))
         for s in reversed(range(S)):

@@ -58,8 +58,12 @@ def test_train_step_matches_oracle_pipeline(schedule, n_mb, mpmd):
 
     cfg = L.LayerCfg(**spec.as_dict())
     stages = [[p] for p in params["layers"]]
-    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16())
+    want_pred = []
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16(),
+                                               preds=want_pred)
     close(losses, want_loss, "losses")
+    for m in range(n_mb):                   # the returned activation: every microbatch's, stacked
+        close(pred[m], want_pred[m], f"prediction of microbatch {m}")
     for s in range(n_stages):
         for k, v in want_acc[s][0].items():
             close(grad["layers"][s][k], v.reshape(grad["layers"][s][k].shape), f"grad {s}/{k}")
@@ -99,8 +103,13 @@ def test_example_model_train_step():
     cfg = L.LayerCfg(**spec.as_dict())
     per = n_layers // pp
     stages = [params["layers"][s * per:(s + 1) * per] for s in range(pp)]
-    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16())
+    want_pred = []
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16(),
+                                               preds=want_pred)
     close(losses, want_loss, "losses")
+    assert pred.shape == batch.shape
+    for m in range(n_mb):
+        close(pred[m], want_pred[m], f"prediction of microbatch {m}")
     for s in range(pp):
         for li in range(per):
             for k, v in want_acc[s][li].items():

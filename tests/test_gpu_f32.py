@@ -377,9 +377,13 @@ def test_cfg1_train_step_through_the_public_api():
     cfg = L.LayerCfg(**CFG1.as_dict())
     per = n_layers // pp
     stages = [params["layers"][s * per:(s + 1) * per] for s in range(pp)]
-    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.f32())
+    want_pred = []
+    want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.f32(),
+                                               preds=want_pred)
     close(losses, want_loss.astype(np.float64), 1e-4, "losses")
     assert pred.shape == batch.shape and np.isfinite(pred).all()
+    for m in range(n_mb):
+        close(pred[m], want_pred[m].astype(np.float64), 1e-4, f"prediction of microbatch {m}")
     for s in range(pp):
         for li in range(per):
             for k, v in want_acc[s][li].items():

@@ -92,9 +92,14 @@ def test_random_train_step_matches_sequential_loop(seed):
     losses, pred, grad = train_step(params, {"hidden": batch, "target": targets})
     cfg = L.LayerCfg(**spec.as_dict())
     stages = [params["layers"][s * per:(s + 1) * per] for s in range(n_stages)]
+    want_pred = []
     want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16(),
-                                               targets=list(targets))
+                                               targets=list(targets), preds=want_pred)
     parity.close(np.asarray(losses, np.float32), np.asarray(want_loss), 2e-2, "losses")
+    assert pred.shape == batch.shape
+    for m in range(n_mb):
+        parity.close(np.asarray(pred[m], np.float32), want_pred[m], 2e-2,
+                     f"prediction of microbatch {m}", 1e-2)
     for s in range(n_stages):
         for li in range(per):
             for k, v in want_acc[s][li].items():

@@ -216,3 +216,23 @@ def test_sequential_loop_with_targets_and_mixed_layer_families():
         got = acc[0][li][name].reshape(params[li][name].shape)[idx]
         # the accumulators are f32: compare at their resolution
         np.testing.assert_allclose(got, (up - down) / (2 * eps), rtol=2e-4, atol=1e-9)
+
+
+def test_sequential_loop_hands_back_every_microbatch_output():
+    """treduce_sequential(preds=[...]): entry m is microbatch m through every layer of every
+    stage in turn (layer_fwd applied by hand here), and the loss is taken from exactly it."""
+    cfg = L.LayerCfg(**SPEC.as_dict())
+    nm = L.Numerics.f32()
+    stages = build(SPEC, 3)
+    xs = xs_for(SPEC, 4)
+    preds = []
+    losses, _ = O.treduce_sequential(cfg, stages, xs, nm, preds=preds)
+    assert len(preds) == len(xs)
+    for m, x in enumerate(xs):
+        a = x
+        for layers in stages:
+            for p in layers:
+                a = L.layer_fwd(cfg, p, a, nm)[0]
+        np.testing.assert_array_equal(preds[m], a)
+        want = np.mean((a.astype(np.float64) - x.astype(np.float64)) ** 2) / len(xs)
+        np.testing.assert_allclose(losses[m], want, rtol=1e-5)
