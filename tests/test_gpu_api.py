@@ -214,6 +214,48 @@ def test_loss_against_a_target_that_is_not_the_input(target_kind):
     train_step.close()
 
 
+def test_reductions_other_than_the_default_ones():
+    """operation=((Add, (Max, Concat(axis=1))), Add): the losses summed to the step's loss, the
+    element-wise maximum of the predictions over the microbatches, and the predictions stacked
+    along their second axis (reference: training.py:112-166)."""
+    rt.require_gpu()
+    spec = LayerSpec("bert", 256, 4, 512, 128, 1, eps=1e-12)
+    n_mb, pp = 3, 2
+    model = jaxpp.nn.TransformerStack(spec, n_layers=2, layers_per_stage=1)
+    params = model.init(seed=1, perturb=True)
+    params = {"layers": [{k: L.bf16_round(v) for k, v in p.items()} for p in params["layers"]]}
+    batch = L.bf16_round(np.random.default_rng(11).standard_normal(
+        (n_mb, spec.tokens, spec.hidden)).astype(np.float32))
+
+    def loss_fn(pars, mb):
+        res = model.apply(pars, mb)
+        return jaxpp.nn.mse_loss(res, mb) / n_mb, (res, res)
+
+    @partial(jaxpp.mpmd_jit_with_loop, mpmd_mesh=_mesh(pp))
+    def train_step(pars, xs):
+        fun = partial(jaxpp.value_and_grad(loss_fn, has_aux=True), pars)
+        return jaxpp.treduce(fun, xs, schedule=jaxpp.Std1F1B(pp),
+                             operation=((jaxpp.Add, (jaxpp.Max, jaxpp.Concat(axis=1))), jaxpp.Add))
+
+    (loss, (top, side_by_side)), grad = train_step(params, batch)
+    want_pred = []
+    want_loss, want_acc = O.treduce_sequential(L.LayerCfg(**spec.as_dict()),
+                                               [[p] for p in params["layers"]], list(batch),
+                                               L.Numerics.bf16(), preds=want_pred)
+    assert np.shape(loss) == ()
+    np.testing.assert_allclose(float(loss), float(want_loss.astype(np.float64).sum()), rtol=2e-2)
+    assert side_by_side.shape == (spec.tokens, n_mb, spec.hidden)
+    for m in range(n_mb):
+        close(side_by_side[:, m], want_pred[m], f"prediction of microbatch {m}")
+    # the maximum of the GPU's own predictions exactly, and of the oracle's to the bf16 bar
+    np.testing.assert_array_equal(top, np.max(np.asarray(side_by_side), axis=1))
+    close(top, np.maximum.reduce(want_pred), "maximum over the microbatches")
+    for s in range(pp):
+        for k, v in want_acc[s][0].items():
+            close(grad["layers"][s][k], v.reshape(grad["layers"][s][k].shape), f"grad {s}/{k}")
+    train_step.close()
+
+
 def test_treduce_i_with_an_explicit_length():
     """treduce_i(fun, length): the body picks its microbatch with take(x, i, axis) - here along
     axis 1 of an array laid out [tokens, microbatch, hidden] (reference: training.py:248-340)."""
