@@ -919,14 +919,17 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
   }
   s->total_bytes = n_layers * s->layer_elems * (4 + s->es) + s->scratch_bytes +
                    s->slot_bytes * s->slots.size();
-  hipMemset(s->params, 0, n_layers * s->layer_elems * s->es);
-  hipMemset(s->grads, 0, n_layers * s->layer_elems * 4);
+  // first failure of the set-up copies below; checked once behind them
+  hipError_t e_init = hipSuccess;
+  auto keep = [&](hipError_t e) { if (e_init == hipSuccess) e_init = e; };
+  keep(hipMemset(s->params, 0, n_layers * s->layer_elems * s->es));
+  keep(hipMemset(s->grads, 0, n_layers * s->layer_elems * 4));
 
   {
     int32_t split[3 * 16] = {};
     for (int k = 0; k < 3; ++k)
       for (int i = 0; i <= (2 << k); ++i) split[16 * k + i] = (int32_t)(T / (2 << k) * i);
-    hipMemcpy(s->S<>(s->s_split), split, sizeof(split), hipMemcpyHostToDevice);
+    keep(hipMemcpy(s->S<>(s->s_split), split, sizeof(split), hipMemcpyHostToDevice));
   }
   if (d->family == JPP_FAMILY_LLAMA || d->family == JPP_FAMILY_MIXTRAL) {
     // cos/sin of pos * theta^(-2i/d): evaluated in double, stored as f32
@@ -938,8 +941,13 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
         c[(size_t)pos * half + i] = (float)cos(ang);
         sn[(size_t)pos * half + i] = (float)sin(ang);
       }
-    hipMemcpy(s->S<>(s->s_cos), c.data(), c.size() * 4, hipMemcpyHostToDevice);
-    hipMemcpy(s->S<>(s->s_sin), sn.data(), sn.size() * 4, hipMemcpyHostToDevice);
+    keep(hipMemcpy(s->S<>(s->s_cos), c.data(), c.size() * 4, hipMemcpyHostToDevice));
+    keep(hipMemcpy(s->S<>(s->s_sin), sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
+  }
+  if (e_init != hipSuccess) {
+    jpp_stage_destroy(s);
+    return jpp_set_error(JPP_ERR_HIP, "stage_create: clearing or filling the stage's buffers "
+                         "failed: %s", hipGetErrorString(e_init));
   }
   hipError_t e5 = hipSuccess;
   if (d->two_streams) {
