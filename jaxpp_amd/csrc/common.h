@@ -88,10 +88,14 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 
 // -- LDS operand slabs ----------------------------------------------------------
 // A slab is [rows][64] bf16 (128 B per row, no padding).  The eight 16-byte
-// chunks of a row are XOR-swizzled with the row index so that both the MFMA
-// operand reads (32 consecutive rows, one chunk) and the transposing stores
-// (rows 8 apart, one chunk) spread over the LDS banks.
-__device__ __forceinline__ int slab_swz(int row) { return (row ^ (row >> 3)) & 7; }
+// chunks of a row are XOR-swizzled with the row index.  LDS serves 256 bytes a
+// cycle from 64 banks, so two consecutive rows span the banks once and a 16-byte
+// read wants the 16 lanes it is served with on 16 different (row parity, chunk)
+// pairs: the swizzle steps once per two rows.  Measured with a read-only loop of
+// 8 waves, in cycles per wave-level ds_read_b128 (4.00 when free of conflicts):
+// the 16-row fragments of the 16x16x32 MFMA 4.00 (6.00 with the row-wise swizzle
+// (row ^ row >> 3) & 7 used before), the 32-row fragments of the 32x32x16 MFMA 4.00.
+__device__ __forceinline__ int slab_swz(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int slab_off(int row, int chunk) {
   return row * 128 + ((chunk ^ slab_swz(row)) << 4);
 }
