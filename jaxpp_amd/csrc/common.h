@@ -89,13 +89,20 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 // -- LDS operand slabs ----------------------------------------------------------
 // A slab is [rows][64] bf16 (128 B per row, no padding).  The eight 16-byte
 // chunks of a row are XOR-swizzled with the row index.  LDS serves 256 bytes a
-// cycle from 64 banks, so two consecutive rows span the banks once and a 16-byte
-// read wants the 16 lanes it is served with on 16 different (row parity, chunk)
-// pairs: the swizzle steps once per two rows.  Measured with a read-only loop of
-// 8 waves, in cycles per wave-level ds_read_b128 (4.00 when free of conflicts):
-// the 16-row fragments of the 16x16x32 MFMA 4.00 (6.00 with the row-wise swizzle
-// (row ^ row >> 3) & 7 used before), the 32-row fragments of the 32x32x16 MFMA 4.00.
-__device__ __forceinline__ int slab_swz(int row) { return (row >> 1) & 7; }
+// cycle from 64 banks, so two consecutive rows span the banks once: the swizzle
+// steps once per two rows (16 rows x one chunk, the fragment of a 16x16x32 MFMA,
+// then lie on 16 different (row parity, chunk) pairs), and rows two apart also
+// differ in the upper half of the chunk index, which is what the transposing
+// reads need (16 lanes on 4 rows x 64 bytes).  Found with a read-only loop of 8
+// waves over XOR-linear maps of the row bits, in cycles per wave-level read:
+// ds_read_b128 4.00 (the floor) for the 16-row and the 32-row fragments - the
+// row-wise swizzle (row ^ row >> 3) & 7 used before took 6.00 for the former -
+// and ds_read_b64_tr_b16 2.3 for the transposed fragments (floor 2.06; 4.00 with
+// any swizzle whose upper bit is the same for rows two apart).
+__device__ __forceinline__ int slab_swz(int row) {
+  const int h = (row >> 1) & 7;
+  return h ^ ((h & 1) * 6);
+}
 __device__ __forceinline__ int slab_off(int row, int chunk) {
   return row * 128 + ((chunk ^ slab_swz(row)) << 4);
 }
