@@ -244,6 +244,11 @@ def main():
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="instead of the workload, print what the matrix cores sustain on a "
                          "register-only MFMA loop (zero and random operands, both tile shapes)")
+    ap.add_argument("--lds-read-rates", action="store_true",
+                    help="instead of the workload, print what the fragment reads of the GEMM "
+                         "and attention kernels cost in LDS cycles per wave-level read, address "
+                         "pattern by pattern (8 waves reading in a loop), with the operand "
+                         "slabs' chunk swizzle of the tree and with the one used before it")
     ap.add_argument("--after-loop", action="store_true",
                     help="also time the step behind the loop - Adam over the stage's f32 "
                          "gradient accumulators, rewriting the bf16 parameters - and report it "
@@ -262,6 +267,9 @@ def main():
             "16x16x32_zero_operands": rt.mfma_rate(16, False, 100000),
             "16x16x32_random_operands": rt.mfma_rate(16, True, 100000)},
             "published_peak_tflops": MFMA_BF16_PEAK / 1e12}))
+        return
+    if args.lds_read_rates:
+        print(json.dumps(lds_read_rates()))
         return
     wl = workloads()[args.workload]
     if args.n_mubatches:
@@ -374,6 +382,71 @@ def main():
         layers = int(round(1.2e13 / (3.0 * wl.layer.fwd_flops())))
         rec["cpu_baseline"] = cpu_baseline(wl, max(1, min(wl.layers_per_stage, layers)))
     print(json.dumps(rec))
+
+
+def lds_read_rates() -> dict:
+    """Cycles per wave-level LDS read for the address patterns of the kernels' fragment reads.
+    The patterns restate the address arithmetic of csrc/common.h (slab_off, DmaTile::frag16,
+    slab_frag, slab_frag_tr, mc_swz) for lane l of a wave; every pattern is measured at several
+    fragment positions and the worst is reported."""
+    def swz_tree(row):
+        h = (row >> 1) & 7
+        return h ^ ((h & 1) * 6)
+
+    def swz_before(row):
+        return (row ^ (row >> 3)) & 7
+
+    def mc_swz(k):
+        return ((k & 3) << 2) ^ (((k >> 3) & 1) << 1)
+
+    def worst(transposing, patterns):
+        return max(rt.lds_read_rate([f(l) for l in range(64)], transposing) for f in patterns)
+
+    out = {"unit": "shader clocks per wave-level read, 8 waves reading",
+           "ds_read_b128, lane l at 16 l (no conflicts: 256 B per clock)":
+               rt.lds_read_rate([16 * l for l in range(64)], False),
+           "ds_read_b64_tr_b16, lane l at 8 l":
+               rt.lds_read_rate([8 * l for l in range(64)], True)}
+    for name, swz in (("swizzle of the tree", swz_tree), ("swizzle before", swz_before),
+                      ("no swizzle", lambda row: 0)):
+        def slab_off(row, chunk, swz=swz):
+            return row * 128 + ((chunk ^ swz(row)) << 4)
+
+        def frag16(row0, k32):
+            return lambda l: slab_off(row0 + (l & 15), k32 * 4 + (l >> 4))
+
+        def frag32(row0, ks):
+            return lambda l: slab_off(row0 + (l & 31), ks * 2 + (l >> 5))
+
+        def frag_tr(col0, st, hi):
+            def f(l):
+                g, s = l >> 4, l & 15
+                n = col0 + ((g & 1) << 4) + ((s & 3) << 2)
+                k = st * 16 + ((g >> 1) << 2) + (s >> 2) + 8 * hi
+                return (n >> 6) * 8192 + ((n & 7) << 1) + slab_off(k, (n & 63) >> 3)
+            return f
+
+        out[name] = {
+            "GEMM, K-contiguous operand, 16-row fragment (ds_read_b128)":
+                worst(False, [frag16(r, k) for r in (0, 16, 48, 240) for k in (0, 1)]),
+            "attention, 32-row fragment (ds_read_b128)":
+                worst(False, [frag32(r, k) for r in (0, 32) for k in (0, 3)]),
+            "attention, transposed fragment (ds_read_b64_tr_b16)":
+                worst(True, [frag_tr(c, st, hi) for c in (0, 32, 96) for st in (0, 3)
+                             for hi in (0, 1)]),
+        }
+
+    def mc_frag(rows, row0, k32, hi):
+        def f(l):
+            g, s = l >> 4, l & 15
+            n = row0 + ((s & 3) << 2)
+            k = k32 * 32 + (g << 3) + (s >> 2) + 4 * hi
+            return k * (rows * 2) + (((n >> 3) ^ mc_swz(k)) << 4) + ((n & 7) << 1)
+        return f
+
+    out["GEMM, operand with the contraction index slow, 256 rows (ds_read_b64_tr_b16)"] = worst(
+        True, [mc_frag(256, r, k, hi) for r in (0, 16, 112, 240) for k in (0, 1) for hi in (0, 1)])
+    return out
 
 
 def kernel_table(wb, wl, steps: int, warmup: int, two: bool, group: int) -> dict:

@@ -97,7 +97,7 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 // waves over XOR-linear maps of the row bits, in cycles per wave-level read:
 // ds_read_b128 4.00 (the floor) for the 16-row and the 32-row fragments - the
 // row-wise swizzle (row ^ row >> 3) & 7 used before took 6.00 for the former -
-// and ds_read_b64_tr_b16 2.3 for the transposed fragments (floor 2.06; 4.00 with
+// and ds_read_b64_tr_b16 2.3 for the transposed fragments (the floor; 4.00 with
 // any swizzle whose upper bit is the same for rows two apart).
 __device__ __forceinline__ int slab_swz(int row) {
   const int h = (row >> 1) & 7;

@@ -141,6 +141,7 @@ def load_diag():
             raise RuntimeError(f"{path} is missing: build it with `python -m jaxpp_amd.build`")
         _diag = C.CDLL(path)
         _diag.jpp_mfma_rate.argtypes = [C.c_int, C.c_int, C.c_int64, C.POINTER(C.c_double)]
+        _diag.jpp_lds_read_rate.argtypes = [C.POINTER(C.c_uint32), C.c_int, C.POINTER(C.c_double)]
     return _diag
 
 
@@ -514,6 +515,17 @@ def mfma_rate(shape: int, random_operands: bool, iters: int = 100000) -> float:
     """TFLOP/s of a register-only MFMA loop on every SIMD (see jpp_mfma_rate)."""
     out = C.c_double(0.0)
     check(load_diag().jpp_mfma_rate(shape, int(random_operands), iters, C.byref(out)))
+    return out.value
+
+
+def lds_read_rate(lane_offsets, transposing: bool) -> float:
+    """Shader clocks per wave-level LDS read of 8 waves reading with these 64 per-lane byte
+    offsets (see jpp_lds_read_rate)."""
+    if len(lane_offsets) != 64:
+        raise ValueError("one byte offset per lane of a wave: 64 of them")
+    arr = (C.c_uint32 * 64)(*[int(o) for o in lane_offsets])
+    out = C.c_double(0.0)
+    check(load_diag().jpp_lds_read_rate(arr, int(transposing), C.byref(out)))
     return out.value
 
 

@@ -28,14 +28,26 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_diagnostics_live_in_a_library_of_their_own():
-    """jpp_mfma_rate (a measurement aid with no counterpart in the reference) is declared in
-    include/jaxpp_amd_diag.h and exported by libjaxpp_amd_diag.so, not by the product library."""
+    """The measurement aids (no counterpart in the reference) are declared in
+    include/jaxpp_amd_diag.h and exported by libjaxpp_amd_diag.so, not by the product library;
+    their argument checks run on the host."""
     diag_header = os.path.join(ROOT, "include", "jaxpp_amd_diag.h")
     names = sorted(set(re.findall(r"\b(jpp_[a-z0-9_]+)\s*\(", open(diag_header).read())))
-    assert names == ["jpp_mfma_rate"]
-    assert "jpp_mfma_rate" not in declared_symbols()
-    assert not hasattr(ctypes.CDLL(rt.lib_path()), "jpp_mfma_rate")
-    assert hasattr(rt.load_diag(), "jpp_mfma_rate")
+    assert names == ["jpp_lds_read_rate", "jpp_mfma_rate"]
+    product = ctypes.CDLL(rt.lib_path())
+    for name in names:
+        assert name not in declared_symbols()
+        assert not hasattr(product, name)
+        assert hasattr(rt.load_diag(), name)
+    diag = rt.load_diag()
+    out = ctypes.c_double(0.0)
+    assert diag.jpp_mfma_rate(7, 0, 1, ctypes.byref(out)) == -1
+    offsets = (ctypes.c_uint32 * 64)(*([0] * 63 + [65536]))        # lane 63 beyond the probe's LDS
+    assert diag.jpp_lds_read_rate(offsets, 0, ctypes.byref(out)) == -1
+    assert b"lane 63" in rt.load().jpp_last_error()
+    offsets[63] = 8                                                # not a multiple of 16
+    assert diag.jpp_lds_read_rate(offsets, 0, ctypes.byref(out)) == -1
+    assert diag.jpp_lds_read_rate(None, 0, ctypes.byref(out)) == -1
 
 
 def test_error_convention_without_gpu():
