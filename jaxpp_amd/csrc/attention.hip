@@ -124,7 +124,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run, mx);
+      // The reference point of the exponentials moves only when some row's maximum has grown
+      // by more than kLazy in the exponent: until then the probabilities of this block are
+      // taken against the older, smaller reference (they may reach 2^kLazy; sums and outputs
+      // are fp32 and the final division removes the common factor), and the 64 accumulator
+      // registers are not rescaled - with random scores some row of the 32 sets a new maximum
+      // in almost every block, by a small amount.
+      constexpr float kLazy = 8.0f;
+      const bool move = __any((mx - m_run) * sc > kLazy);
+      const float m_new = move ? fmaxf(m_run, mx) : m_run;
       const float neg = -m_new * sc;
       float rs = 0.f;
 #pragma unroll
@@ -135,7 +143,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
           s[t][r] = e;
           rs += e;
         }
-      if (__any(m_new != m_run)) {  // rescale only when some row's maximum moved
+      if (move) {
         const float alpha = fast_exp2((m_run - m_new) * sc);
         l_run *= alpha;
 #pragma unroll
