@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
   }
   const long stat = ((long)b * p.n_heads + h) * p.seq + qi;
   float lse2 = p.lse[stat] * kLog2e;
-  float dlt = p.delta[stat];
+  float dlt = p.delta[stat] * p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
   const float sc = p.scale * kLog2e;
   settle(qf);
   settle(dof);
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float pr = fast_exp2(fmaf(s[r], sc, -lse2));  // exp2(-inf) = 0 where masked
-          s[r] = pr * (dp[r] - dlt) * p.scale;
+          s[r] = pr * fmaf(dp[r], p.scale, -dlt);
         }
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
   };
   auto park = [&](int stage) {
     float* st = (float*)(smem + stage * STAGE + 2 * TILE);
-    if (tid < 128) st[tid] = tid < 64 ? rstat * kLog2e : rstat;
+    if (tid < 128) st[tid] = tid < 64 ? rstat * kLog2e : rstat * p.scale;  // delta parked scaled
   };
 
   fetch(0, 0);
@@ -459,7 +459,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
               float pr = fast_exp2(fmaf(s[u][r], sc, -ls[e]));
               if (diag && ki > q0 + ql + e) pr = 0.f;
               s[u][r] = pr;
-              dp[u][r] = pr * (dp[u][r] - dl[e]) * p.scale;
+              dp[u][r] = pr * fmaf(dp[u][r], p.scale, -dl[e]);
             }
           }
         }

@@ -97,7 +97,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
       dma_tile_pair<D>(p.d_o + (row0 + q0) * p.lddo + hh * D, offdo, dst + TILE, ksb);
     };
     auto park = [&](int stage) {
-      ((float*)(my + stage * STAGE + 2 * TILE))[ht] = ht < 64 ? rstat * kLog2e : rstat;
+      // lse in the exp2 domain; delta scaled, so that scale (dP - delta) is one fma per element
+      ((float*)(my + stage * STAGE + 2 * TILE))[ht] = ht < 64 ? rstat * kLog2e : rstat * p.scale;
     };
 
     // one 32-query tile against this wave's 32 keys
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_kernel(Att
           const int r = 4 * g + e;
           const float pr = fast_exp2(fmaf(s[r], sc, -ls[e]));  // exp2(-inf) = 0 where masked
           s[r] = pr;
-          dp[r] = pr * (dp[r] - dl[e]) * p.scale;
+          dp[r] = pr * fmaf(dp[r], p.scale, -dl[e]);
         }
       }
 #pragma unroll
