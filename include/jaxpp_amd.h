@@ -102,7 +102,7 @@ int jpp_probe_end(int64_t* launches, double* total_ms, double* total_flops, doub
 /* With jpp_probe_begin("*") every class is bracketed and jpp_probe_end returns the totals over
  * all of them; jpp_probe_class then reads class `index` (0, 1, ... until JPP_ERR_INVALID) of
  * the probe that has just ended: its name (valid until the next jpp_probe_begin) and its own
- * figures.  Further classes: attn_delta, sum_accum, mse, fill, cast, moe_route, moe_gather,
+ * figures.  Further classes: sum_accum, mse, fill, cast, moe_route, moe_gather,
  * moe_combine_fwd, moe_bwd_prepare, moe_combine_bwd, moe_router_wgrad. */
 int jpp_probe_class(int index, const char** name, int64_t* launches, double* total_ms,
                     double* total_flops, double* total_bytes);

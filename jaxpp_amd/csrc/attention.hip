@@ -182,37 +182,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// backward, step 0: delta[b,h,q] = sum_d dO * O
-// ---------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void attn_delta_kernel(AttnParams p) {
-  constexpr int LPH = D / 8;  // lanes per head
-  const long item = (long)blockIdx.x * 256 + threadIdx.x;
-  const long total = (long)p.batch * p.seq * p.n_heads * LPH;
-  float s = 0.f;
-  long row = 0;
-  int h = 0;
-  if (item < total) {
-    const int c = (int)(item % LPH);
-    const long rh = item / LPH;
-    h = (int)(rh % p.n_heads);
-    row = rh / p.n_heads;
-    const uint4 a = *(const uint4*)(p.o + row * p.ldo + h * D + c * 8);
-    const uint4 g = *(const uint4*)(p.d_o + row * p.lddo + h * D + c * 8);
-    s = bf16lo_to_f32(a.x) * bf16lo_to_f32(g.x) + bf16hi_to_f32(a.x) * bf16hi_to_f32(g.x) +
-        bf16lo_to_f32(a.y) * bf16lo_to_f32(g.y) + bf16hi_to_f32(a.y) * bf16hi_to_f32(g.y) +
-        bf16lo_to_f32(a.z) * bf16lo_to_f32(g.z) + bf16hi_to_f32(a.z) * bf16hi_to_f32(g.z) +
-        bf16lo_to_f32(a.w) * bf16lo_to_f32(g.w) + bf16hi_to_f32(a.w) * bf16hi_to_f32(g.w);
-  }
-#pragma unroll
-  for (int o = LPH / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
-  if (item < total && (item % LPH) == 0) {
-    const long b = row / p.seq, qpos = row % p.seq;
-    p.delta[(b * p.n_heads + h) * p.seq + qpos] = s;
-  }
-}
-
-// ---------------------------------------------------------------------------
 // backward, dQ: one workgroup per 128 queries of one head
 // ---------------------------------------------------------------------------
 template <int D, bool CAUSAL>
@@ -243,7 +212,25 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
   }
   const long stat = ((long)b * p.n_heads + h) * p.seq + qi;
   float lse2 = p.lse[stat] * kLog2e;
-  float dlt = p.delta[stat] * p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
+  // The row term delta = sum_d dO * O of this wave's 32 rows: a lane holds half of its row of
+  // dO already (the chunks the MFMA fragment gives it) and reads the same half of O; the other
+  // half is with lane ^ 32.  Written out for the dK/dV kernel, which runs behind this one.
+  float dlt = 0.f;
+  {
+    const bf16_t* obase = p.o + (row0 + q0) * p.ldo + h * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const uint4 ov = *(const uint4*)(obase + (long)(lane & 31) * p.ldo + ks * 16 + (lane >> 5) * 8);
+      float of[8], gf[8];
+      unpack8(ov, of);
+      unpack8(__builtin_bit_cast(uint4, dof[ks]), gf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dlt = fmaf(of[e], gf[e], dlt);
+    }
+    dlt += __shfl_xor(dlt, 32);
+    if (lane < 32) p.delta[stat] = dlt;
+  }
+  dlt *= p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
   const float sc = p.scale * kLog2e;
   settle(qf);
   settle(dof);
@@ -572,8 +559,6 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
   const bool fused_rope = a->rope_cos && a->causal;
   if (fused_rope) { p.rope_cos = a->rope_cos; p.rope_sin = a->rope_sin; }
   hipStream_t st = (hipStream_t)stream;
-  const long items = (long)a->batch * a->seq * a->n_heads * (a->head_dim / 8);
-  dim3 gdelta((unsigned)((items + 255) / 256));
   dim3 gq(a->seq / 128, a->n_heads, a->batch);
   // causal: 64-key blocks, a workgroup takes blocks x and n-1-x; else 128-key blocks
   dim3 gkv(a->seq / 128, a->n_kv_heads, a->batch);
@@ -581,10 +566,6 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
                     (a->causal ? 0.5 : 1.0);
 #define JPP_AB(D_, C_)                                                              \
   do {                                                                              \
-    {                                                                               \
-      ProbeScope probe(st, "attn_delta", 0, 4.0 * a->batch * a->seq * a->n_heads * D_); \
-      hipLaunchKernelGGL((attn_delta_kernel<D_>), gdelta, dim3(256), 0, st, p);     \
-    }                                                                               \
     if (int rc = set_smem(attn_bwd_dq_kernel<D_, C_>, 4 * D_ * 128)) return rc;     \
     {                                                                               \
       ProbeScope probe(st, "attn_bwd_dq", fl * 0.4, 0);                             \
