@@ -255,6 +255,48 @@ def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
     np.testing.assert_array_equal(dqkv_d.download_bf16((T, width)), want_r)
 
 
+@pytest.mark.parametrize("d,causal,slope", [(128, 1, 40.0), (128, 0, 40.0), (64, 1, 12.0),
+                                            (128, 1, -40.0), (64, 0, 300.0)])
+def test_attention_forward_with_drifting_row_maxima(d, causal, slope):
+    """Scores that grow (or fall) steadily along the key axis: the running maximum of every row
+    moves in every block of keys, by less than the forward kernel's threshold for moving its
+    reference point in most blocks and by more in some, so both of its paths - exponentials
+    against an older reference, and the rescale - carry weight in the result.  slope is the
+    growth of the scaled score over the whole sequence (300: a jump past the threshold in every
+    block; negative: the first block holds every maximum)."""
+    print(f"attention drift d={d} causal={causal} slope={slope}", flush=True)
+    rng = np.random.default_rng(int(abs(slope)) + d + causal)
+    batch, seq, hq, hkv = 1, 1024, 4, 2
+    T, width = batch * seq, (hq + 2 * hkv) * d
+    u = np.ones(d, np.float32) / np.sqrt(d)
+    ramp = (np.arange(seq, dtype=np.float32) / seq)[:, None]
+    q = 0.3 * rng.standard_normal((T, hq, d)).astype(np.float32) + np.sqrt(np.sqrt(d) * abs(slope)) * u
+    k = 0.3 * rng.standard_normal((T, hkv, d)).astype(np.float32) + \
+        (np.sign(slope) * np.sqrt(np.sqrt(d) * abs(slope)) * ramp * u)[:, None, :]
+    v = rng.standard_normal((T, hkv, d)).astype(np.float32)
+    qkv = L.bf16_round(np.concatenate([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], -1))
+    q4 = qkv[:, :hq * d].reshape(batch, seq, hq, d)
+    k4 = qkv[:, hq * d:(hq + hkv) * d].reshape(batch, seq, hkv, d)
+    v4 = qkv[:, (hq + hkv) * d:].reshape(batch, seq, hkv, d)
+    o_w, lse_w = L.attention_fwd(q4, k4, v4, bool(causal), rt=L.bf16_round)
+    # the case is what it claims: along the keys a row's scaled scores span about |slope|
+    s0 = (q4[0, -1, 0] @ k4[0, :, 0].T) / np.sqrt(d)
+    assert abs(float(s0[-1] - s0[0])) > 0.6 * abs(slope)
+    b_qkv, b_o = dev_bf16(qkv), rt.DeviceBuffer(T * hq * d * 2)
+    b_lse = rt.DeviceBuffer(batch * hq * seq * 4)
+    a = rt.AttnArgs(b_qkv.ptr, b_qkv.ptr + hq * d * 2, b_qkv.ptr + (hq + hkv) * d * 2, b_o.ptr,
+                    b_lse.ptr, None, None, None, None, None,
+                    width, width, width, hq * d, hq * d, width, width, width,
+                    batch, seq, hq, hkv, d, causal)
+    rt.check(rt.load().jpp_attn_fwd(None, C.byref(a)))
+    rt.sync()
+    got = b_o.download_bf16((T, hq * d))
+    assert np.isfinite(got).all()
+    close(got, o_w.reshape(T, -1), 2e-2, "attn out")
+    np.testing.assert_allclose(b_lse.download(np.float32, (batch, hq, seq)), lse_w, rtol=2e-3,
+                               atol=2e-2)
+
+
 @pytest.mark.parametrize("ln,rows,cols", [(True, 300, 256), (True, 1024, 1024), (False, 512, 4096),
                                           (False, 130, 8192), (False, 64, 128), (True, 261, 4096),
                                           (True, 1030, 8192), (True, 140, 6144), (False, 140, 5120)])
