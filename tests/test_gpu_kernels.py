@@ -259,11 +259,9 @@ def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
                                             (128, 1, -40.0), (64, 0, 300.0)])
 def test_attention_forward_with_drifting_row_maxima(d, causal, slope):
     """Scores that grow (or fall) steadily along the key axis: the running maximum of every row
-    moves in every block of keys, by less than the forward kernel's threshold for moving its
-    reference point in most blocks and by more in some, so both of its paths - exponentials
-    against an older reference, and the rescale - carry weight in the result.  slope is the
-    growth of the scaled score over the whole sequence (300: a jump past the threshold in every
-    block; negative: the first block holds every maximum)."""
+    moves in every block of keys, so the rescale of the running sums and outputs carries weight
+    in the result.  slope is the growth of the scaled score over the whole sequence (300: a jump
+    of 2^27 per block; negative: the first block holds every maximum)."""
     print(f"attention drift d={d} causal={causal} slope={slope}", flush=True)
     rng = np.random.default_rng(int(abs(slope)) + d + causal)
     batch, seq, hq, hkv = 1, 1024, 4, 2
