@@ -6,6 +6,8 @@ dimensions larger than the row)."""
 import ctypes as C
 import math
 
+import os
+
 import numpy as np
 import pytest
 
@@ -16,6 +18,9 @@ from jaxpp_amd import runtime as rt
 from oracle import layers as L
 
 pytestmark = pytest.mark.gpu
+
+# further draws on demand: JPP_SWEEP_OFFSET=100000 python -m pytest <this file> (the committed runs use 0)
+SWEEP_OFFSET = int(os.environ.get("JPP_SWEEP_OFFSET", "0"))
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -33,7 +38,7 @@ def pad_cols(a, ld):
 
 @pytest.mark.parametrize("seed", range(48))
 def test_random_gemm(seed):
-    rng = np.random.default_rng(3000 + seed)
+    rng = np.random.default_rng(3000 + SWEEP_OFFSET + seed)
     ta, tb, epi = K.GEMM_CASES[rng.integers(len(K.GEMM_CASES))]
     big = rng.integers(4) == 0                     # now and then: several rounds of 256x256 tiles
     m = int(rng.integers(1, 33 if big else 9)) * 128
@@ -101,7 +106,7 @@ def test_random_gemm(seed):
 
 @pytest.mark.parametrize("seed", range(24))
 def test_random_attention(seed):
-    rng = np.random.default_rng(4000 + seed)
+    rng = np.random.default_rng(4000 + SWEEP_OFFSET + seed)
     d = int(rng.choice([64, 128]))
     hkv = int(rng.integers(1, 4))
     hq = hkv * int(rng.choice([1, 2, 4]))
@@ -114,7 +119,7 @@ def test_random_attention(seed):
 
 @pytest.mark.parametrize("seed", range(24))
 def test_random_norm(seed):
-    rng = np.random.default_rng(5000 + seed)
+    rng = np.random.default_rng(5000 + SWEEP_OFFSET + seed)
     ln = bool(rng.integers(2))
     rows = int(rng.integers(1, 1500))
     cols = int(rng.integers(16, 1025)) * 8
@@ -123,7 +128,7 @@ def test_random_norm(seed):
 
 @pytest.mark.parametrize("seed", range(16))
 def test_random_moe(seed):
-    rng = np.random.default_rng(6000 + seed)
+    rng = np.random.default_rng(6000 + SWEEP_OFFSET + seed)
     T = int(rng.integers(1, 3000))                 # any count: groups are padded to 256 rows
     h = int(rng.integers(2, 65)) * 8
     print(f"seed {seed}: {T} tokens of width {h}", flush=True)

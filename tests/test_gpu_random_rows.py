@@ -3,6 +3,8 @@ stream / weight-gradient grouping mode): the rank's row on the GPU against the o
 executor.  The fixed cases of test_gpu_stage.py name the combinations that matter; this sweep
 is for the ones nobody thought of (slot-ring corner cases, groups that never fill, ranks in the
 middle of a pipeline, a first stage whose backward is not split)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -15,6 +17,9 @@ from jaxpp_amd import schedules as S
 from jaxpp_amd.plan import make_rank_plan
 
 pytestmark = pytest.mark.gpu
+
+# further draws on demand: JPP_SWEEP_OFFSET=100000 python -m pytest <this file> (the committed runs use 0)
+SWEEP_OFFSET = int(os.environ.get("JPP_SWEEP_OFFSET", "0"))
 
 import test_gpu_f32 as F32  # noqa: E402
 
@@ -30,7 +35,7 @@ def _gpu():
 
 def draw(seed):
     """A valid (spec, schedule, n, rank, layers per chunk, mode) for this seed."""
-    rng = np.random.default_rng(1000 + seed)
+    rng = np.random.default_rng(1000 + SWEEP_OFFSET + seed)
     while True:
         spec = SPECS[rng.integers(len(SPECS))]
         p = int(rng.integers(1, 5))                     # pipeline ranks
