@@ -178,6 +178,15 @@ typedef struct {
    * weight gradients of several microbatches, whose routing differs). */
   const int32_t* seg_more[3];
   const int32_t* seg_rows_more[3];
+  /* Rotary embedding in the epilogue (JPP_EPI_BF16, trans_a = 0, trans_b = 1, no bias, residual
+   * or groups; NULL: none): columns [0, rope_cols) of C are heads of rope_head_dim (64 or 128)
+   * elements, row r of C is position r % rope_seq, and the tables are f32
+   * [rope_seq, rope_head_dim / 2] as for jpp_rope.  The product is rounded to bf16, rotated and
+   * rounded again: the very values jpp_rope leaves when run over the plain result. */
+  const float* rope_cos;
+  const float* rope_sin;
+  int64_t rope_cols;
+  int rope_seq, rope_head_dim;
 } jpp_gemm_args;
 
 enum { JPP_GROUP_NONE = 0, JPP_GROUP_M = 1, JPP_GROUP_K = 2 };

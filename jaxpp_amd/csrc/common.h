@@ -86,6 +86,15 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
                     pack_bf16x2(f[6], f[7]));
 }
 
+// Rotary embedding of one pair: a and b are elements i and i + d/2 of a head, cs / sn the
+// table entries of (position, i).  One definition for the pass of its own and for the GEMM
+// epilogue that applies it, so that both round alike.
+__device__ __forceinline__ void rope_rotate(float a, float b, float cs, float sn, float& o1,
+                                            float& o2) {
+  o1 = a * cs - b * sn;
+  o2 = b * cs + a * sn;
+}
+
 // -- LDS operand slabs ----------------------------------------------------------
 // A slab is [rows][64] bf16 (128 B per row, no padding).  The eight 16-byte
 // chunks of a row are XOR-swizzled with the row index.  LDS serves 256 bytes a

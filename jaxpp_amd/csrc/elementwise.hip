@@ -524,7 +524,8 @@ __global__ __launch_bounds__(256) void rope_kernel(bf16_t* __restrict__ x, long 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float cs = ct[e], sn = inverse ? -st[e] : st[e];
-      const float o1 = a[e] * cs - b[e] * sn, o2 = b[e] * cs + a[e] * sn;
+      float o1, o2;
+      rope_rotate(a[e], b[e], cs, sn, o1, o2);
       a[e] = o1;
       b[e] = o2;
     }

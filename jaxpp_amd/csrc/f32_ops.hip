@@ -512,6 +512,8 @@ extern "C" {
 int jpp_gemm_f32(void* stream, const jpp_gemm_args* a) {
   JPP_REQUIRE(!a || a->k_parts <= 1, "gemm_f32: one operand pair per product");
   JPP_REQUIRE(a && a->a && a->b && a->c, "gemm_f32: null operand");
+  JPP_REQUIRE(!a->rope_cos && !a->rope_sin,
+              "gemm_f32: no rotary epilogue on f32 tensors (jpp_rope_f32 is the pass for them)");
   const bool group_k = a->group_mode == JPP_GROUP_K;
   JPP_REQUIRE(a->m > 0 && a->n > 0 && (a->k > 0 || group_k) && a->m % 64 == 0 && a->n % 64 == 0 &&
                   (a->k % 16 == 0 || group_k),

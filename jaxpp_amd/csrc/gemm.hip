@@ -58,6 +58,12 @@ struct GemmParams {
   int n_seg, group_mode;
   int64_t group_rows;
   long stride_b, stride_c;
+  // rotary embedding in the bf16 epilogue of the forward kernels (NULL: none): columns
+  // [0, rope_cols) are heads of rope_hd elements, row r is position (rope_row0 + r) % rope_seq
+  const float* rope_cos;
+  const float* rope_sin;
+  int rope_cols, rope_seq, rope_hd;
+  long rope_row0;
 };
 
 // One more problem of a launch that covers several independent products of one kind (same
@@ -581,6 +587,32 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
 #pragma unroll
               for (int e = 0; e < 8; ++e) v[e] += rv[e];
             }
+            if constexpr (!TA && TB) {
+              // rotary embedding of the query / key heads (forward projection): the partner
+              // of a column sits half a head away in the same staged row; both are rounded to
+              // bf16 first, as a pass of its own would read them back
+              if (p.rope_cos && n0 + c8 < p.rope_cols) {
+                const int hh = p.rope_hd >> 1, cin = (n0 + c8) & (p.rope_hd - 1);
+                const bool lo = cin < hh;
+                const uint8_t* prow = row + (lo ? hh : -hh) * 4;
+                const float4 b0 = *(const float4*)prow, b1 = *(const float4*)(prow + 16);
+                const float w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+                const long pos = (p.rope_row0 + mrow0 + r) % p.rope_seq;
+                const float* ct = p.rope_cos + pos * hh + (cin & (hh - 1));
+                const float* st = p.rope_sin + pos * hh + (cin & (hh - 1));
+                const float4 c0 = *(const float4*)ct, c1 = *(const float4*)(ct + 4);
+                const float4 s0 = *(const float4*)st, s1 = *(const float4*)(st + 4);
+                const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+                const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                  const float own = (float)(__bf16)v[e], other = (float)(__bf16)w[e];
+                  float o1, o2;
+                  rope_rotate(lo ? own : other, lo ? other : own, cs[e], sn[e], o1, o2);
+                  v[e] = lo ? o1 : o2;
+                }
+              }
+            }
           } else if constexpr (EPI == JPP_EPI_GELU) {
             float gl[8];
 #pragma unroll
@@ -762,6 +794,10 @@ void shift_origin(GemmParams& p, bool ta, bool tb, int epi, long m_off, long n_o
   if (p.c2)  // SwiGLU: s has one column per gate/up pair; GELU: as wide as C
     p.c2 = (bf16_t*)p.c2 + m_off * p.ldc2 + (epi == JPP_EPI_SWIGLU ? n_off / 2 : n_off);
   if (p.bias) p.bias += n_off;
+  if (p.rope_cos) {  // (n_off is a multiple of 256: whole heads)
+    p.rope_row0 += m_off;
+    p.rope_cols = (int)(p.rope_cols > n_off ? p.rope_cols - n_off : 0);
+  }
   if (p.resid) p.resid += m_off * p.ldresid + n_off;
   if (p.aux) p.aux += m_off * p.ldaux + c_cols;
 }
@@ -825,6 +861,23 @@ int prepare(const jpp_gemm_args* a, GemmParams& p) {
     p.b_more[i] = (const bf16_t*)a->b_more[i];
     p.seg_more[i] = a->seg_more[i];
     p.seg_rows_more[i] = a->seg_rows_more[i];
+  }
+  p.rope_cos = a->rope_cos; p.rope_sin = a->rope_sin;
+  p.rope_cols = (int)a->rope_cols; p.rope_seq = a->rope_seq; p.rope_hd = a->rope_head_dim;
+  p.rope_row0 = 0;
+  if (a->rope_cos || a->rope_sin) {
+    JPP_REQUIRE(a->rope_cos && a->rope_sin, "gemm: rope_cos and rope_sin go together");
+    JPP_REQUIRE(a->epilogue == JPP_EPI_BF16 && !a->trans_a && a->trans_b && !a->bias &&
+                    !a->resid && a->group_mode == JPP_GROUP_NONE,
+                "gemm: the rotary epilogue goes with JPP_EPI_BF16, trans_a = 0, trans_b = 1 and "
+                "no bias, residual or groups");
+    JPP_REQUIRE((a->rope_head_dim == 64 || a->rope_head_dim == 128) && a->rope_seq > 0 &&
+                    a->rope_cols >= 0 && a->rope_cols <= a->n &&
+                    a->rope_cols % a->rope_head_dim == 0,
+                "gemm: rotary epilogue: heads of 64 or 128 elements, rope_cols a multiple of the "
+                "head size and at most N, rope_seq positive");
+    JPP_REQUIRE(((uintptr_t)a->rope_cos | (uintptr_t)a->rope_sin) % 16 == 0,
+                "gemm: rotary tables must be 16-byte aligned");
   }
   if (a->k_parts > 1) {
     JPP_REQUIRE(a->k_parts <= 4 && a->group_mode != JPP_GROUP_M,

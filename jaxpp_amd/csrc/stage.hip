@@ -391,9 +391,24 @@ int layer_fwd(jpp_stage* s, hipStream_t st, int chunk, int li, uint8_t* slot, vo
   // llama
   RC(norm_f(s, st, at(L.x), s->P(chunk, li, L_rms1), nullptr, at(L.n1), nullptr,
             (float*)at(L.rstd1)));
-  RC(gemm(s, st, at(L.n1), h, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 1, at(L.qkv), s->qkvw, T, s->qkvw,
-          h, JPP_EPI_BF16));
-  RC(rope(s, st, at(L.qkv), 0));
+  if (s->f32()) {
+    RC(gemm(s, st, at(L.n1), h, 0, s->P(chunk, li, L_Wqkv), s->qkvw, 1, at(L.qkv), s->qkvw, T,
+            s->qkvw, h, JPP_EPI_BF16));
+    RC(rope(s, st, at(L.qkv), 0));
+  } else {
+    // the projection rotates the query and key heads in its epilogue (the same values a pass
+    // of jpp_rope over its plain result would leave)
+    jpp_gemm_args g;
+    memset(&g, 0, sizeof(g));
+    g.a = at(L.n1); g.b = s->P(chunk, li, L_Wqkv); g.c = at(L.qkv);
+    g.m = T; g.n = s->qkvw; g.k = h;
+    g.lda = h; g.ldb = s->qkvw; g.ldc = s->qkvw;
+    g.trans_a = 0; g.trans_b = 1; g.epilogue = JPP_EPI_BF16;
+    g.rope_cos = s->S<float>(s->s_cos); g.rope_sin = s->S<float>(s->s_sin);
+    g.rope_cols = (int64_t)(s->d.n_heads + s->d.n_kv_heads) * s->hd;
+    g.rope_seq = s->d.seq; g.rope_head_dim = (int)s->hd;
+    RC(jpp_gemm_bf16(st, &g));
+  }
   attn_args(s, aa, slot, L);
   RC(attn_f(s, st, &aa));
   RC(gemm(s, st, at(L.ctx), s->ctxw, 0, s->P(chunk, li, L_Wo), h, 1, at(L.h1), h, T, h, s->ctxw,

@@ -41,7 +41,9 @@ class GemmArgs(C.Structure):
                 ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("group_rows", C.c_int64),
                 ("seg_rows", C.c_void_p),
                 ("a_more", C.c_void_p * 3), ("b_more", C.c_void_p * 3), ("k_parts", C.c_int),
-                ("seg_more", C.c_void_p * 3), ("seg_rows_more", C.c_void_p * 3)]
+                ("seg_more", C.c_void_p * 3), ("seg_rows_more", C.c_void_p * 3),
+                ("rope_cos", C.c_void_p), ("rope_sin", C.c_void_p), ("rope_cols", C.c_int64),
+                ("rope_seq", C.c_int), ("rope_head_dim", C.c_int)]
 
 
 class AttnArgs(C.Structure):
@@ -477,9 +479,11 @@ class probe:
 def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, bias=None,
          resid=None, ldresid=0, aux=None, ldaux=0, c2=None, ldc2=0, gelu_tanh=0, tile=0,
          stream=None, seg=None, n_seg=0, group_mode=0, stride_b=0, stride_c=0, group_rows=0,
-         seg_rows=None, f32=False, more=(), more_seg=()):
+         seg_rows=None, f32=False, more=(), more_seg=(), rope=None):
     """`more`: further (a, b) operand pairs the contraction continues over (k elements each);
-    `more_seg`: for a grouped contraction, the (seg, seg_rows) row groups of those pairs."""
+    `more_seg`: for a grouped contraction, the (seg, seg_rows) row groups of those pairs;
+    `rope`: (cos, sin, cols, seq, head_dim) - rotary embedding of columns [0, cols) in the
+    epilogue of a forward product."""
     g = GemmArgs(a, b, c, c2, bias, resid, aux, m, n, k, lda, ldb, ldc, ldc2, ldresid, ldaux,
                  int(trans_a), int(trans_b), epilogue, gelu_tanh, tile, seg, n_seg, group_mode,
                  stride_b, stride_c, group_rows, seg_rows)
@@ -490,6 +494,8 @@ def gemm(a, b, c, m, n, k, lda, ldb, ldc, trans_a, trans_b, epilogue=EPI_BF16, b
     if more_seg:
         g.seg_more = (C.c_void_p * 3)(*([sg for sg, _ in more_seg] + [None] * (3 - len(more_seg))))
         g.seg_rows_more = (C.c_void_p * 3)(*([sr for _, sr in more_seg] + [None] * (3 - len(more_seg))))
+    if rope:
+        g.rope_cos, g.rope_sin, g.rope_cols, g.rope_seq, g.rope_head_dim = rope
     check((load().jpp_gemm_f32 if f32 else load().jpp_gemm_bf16)(stream, C.byref(g)))
 
 

@@ -78,7 +78,8 @@ def test_workspace_sizes():
 
 def test_struct_layouts_match_header_sizes():
     # 7 pointers + 9 int64 + 5 int (+ padding) ; guards against field drift
-    assert ctypes.sizeof(rt.GemmArgs) == 7 * 8 + 9 * 8 + 5 * 4 + 4 + 8 + 2 * 4 + 3 * 8 + 8 + 6 * 8 + 8 + 6 * 8
+    assert ctypes.sizeof(rt.GemmArgs) == (7 * 8 + 9 * 8 + 5 * 4 + 4 + 8 + 2 * 4 + 3 * 8 + 8 + 6 * 8 + 8 +
+                                          6 * 8 + 3 * 8 + 2 * 4)
     assert ctypes.sizeof(rt.AttnArgs) == 10 * 8 + 8 * 8 + 6 * 4 + 2 * 8
     assert ctypes.sizeof(rt.NormArgs) == 12 * 8 + 2 * 8 + 8
     assert ctypes.sizeof(rt.StageDesc) == 22 * 4

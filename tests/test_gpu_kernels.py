@@ -188,6 +188,47 @@ def test_gemm_rejects_bad_shapes():
         rt.gemm(None, d.ptr, d.ptr, 128, 128, 64, 64, 64, 128, 0, 0)
 
 
+@pytest.mark.parametrize("batch,seq,heads,rot_heads,d,k,tile", [
+    (2, 256, 8, 6, 128, 256, 0),        # 128 x 128 tiles
+    (2, 256, 12, 10, 128, 512, 4),      # 256 x 256 tiles
+    (1, 256, 8, 6, 64, 256, 0),         # heads of 64
+    (1, 512, 16, 12, 64, 128, 3),       # 128 x 256 tiles, four heads per tile
+    (1, 4096, 48, 40, 128, 256, 0),     # 384 tiles: a full round and a tail of 128 x 256 tiles
+                                        # over the last columns (the Llama-3-8B QKV projection)
+    (5, 1024, 32, 32, 128, 128, 0),     # 320 tiles: the tail over the last rows (positions
+                                        # continue behind the split)
+])
+def test_gemm_with_rotary_epilogue(batch, seq, heads, rot_heads, d, k, tile):
+    """The forward product that rotates its first rot_heads heads in the epilogue leaves the
+    very bits jpp_rope leaves when run over the plain product."""
+    print(f"gemm+rope b={batch} s={seq} heads={heads}/{rot_heads} d={d} k={k} tile={tile}", flush=True)
+    rng = np.random.default_rng(batch + seq + heads + d)
+    m, n = batch * seq, heads * d
+    a, w = rnd(rng, m, k), rnd(rng, k, n, scale=0.1)
+    cos, sin = L.rope_tables(seq, d, 5e5, np.float32)
+    ba, bw = dev_bf16(a), dev_bf16(w)
+    bc, bs = rt.DeviceBuffer.from_numpy(cos), rt.DeviceBuffer.from_numpy(sin)
+    plain, fused = rt.DeviceBuffer(m * n * 2), rt.DeviceBuffer(m * n * 2)
+    rt.gemm(ba.ptr, bw.ptr, plain.ptr, m, n, k, k, n, n, 0, 1, rt.EPI_BF16, tile=tile)
+    rt.check(rt.load().jpp_rope(None, plain.ptr, n, bc.ptr, bs.ptr, batch, seq, rot_heads, d, 0))
+    rt.gemm(ba.ptr, bw.ptr, fused.ptr, m, n, k, k, n, n, 0, 1, rt.EPI_BF16, tile=tile,
+            rope=(bc.ptr, bs.ptr, rot_heads * d, seq, d))
+    rt.sync()
+    want = plain.download_bf16((m, n))
+    got = fused.download_bf16((m, n))
+    np.testing.assert_array_equal(got, want)
+    # and the pass it replaces does what the oracle says (rotated heads only)
+    ref = L.bf16_round(a.astype(np.float64) @ w.astype(np.float64)).reshape(batch, seq, heads, d)
+    ref[:, :, :rot_heads] = L.rope_apply(ref[:, :, :rot_heads], cos, sin)
+    close(got, ref.reshape(m, n), 2e-2, "rotated product")
+    with pytest.raises(rt.JppError, match="rotary"):
+        rt.gemm(ba.ptr, bw.ptr, fused.ptr, m, n, k, k, n, n, 0, 1, rt.EPI_BF16,
+                rope=(bc.ptr, bs.ptr, rot_heads * d + 8, seq, d))
+    with pytest.raises(rt.JppError, match="rotary"):
+        rt.gemm(ba.ptr, bw.ptr, fused.ptr, m, n, k, k, n, n, 0, 1, rt.EPI_BF16, resid=ba.ptr,
+                ldresid=n, rope=(bc.ptr, bs.ptr, rot_heads * d, seq, d))
+
+
 @pytest.mark.parametrize("d,causal,hq,hkv,batch,seq", [
     (64, 0, 4, 4, 2, 256), (64, 1, 2, 2, 1, 384), (128, 1, 8, 2, 1, 512),
     (128, 0, 2, 1, 2, 128), (128, 1, 4, 4, 1, 256),
