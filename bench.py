@@ -117,8 +117,8 @@ class Workbench:
         return 3.0 * wl.layer.fwd_flops() * wl.layers_per_stage * self.plan.n_chunks * wl.n_mubatches
 
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/stage_cfg3_hbm_traffic.md: counters scaled by copy kernels of known size), keyed by
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# of this script (the counters scaled by what they read for copy kernels of known size), keyed by
 # (workload, kernel class, microbatches per weight-gradient launch): a launch over four
 # microbatches reads four operand pairs and the accumulator once
 MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8_multi", 4): 1.3344e10,  # a layer per launch
