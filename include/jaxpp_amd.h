@@ -216,7 +216,7 @@ typedef struct {
   float* lse;               /* fwd: out; bwd: in */
   const void* d_o;          /* bwd */
   void* dq; void* dk; void* dv;
-  float* delta;             /* bwd scratch, f32 [batch, n_heads, seq] */
+  float* delta;             /* bwd scratch, f32 [batch, n_heads, seq, 2] (JPP_WS_ATTN_DELTA) */
   int64_t ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv;
   int batch, seq, n_heads, n_kv_heads, head_dim, causal;
   /* Backward only, optional (NULL: off): f32 [seq, head_dim/2] tables of the half-split rotary

@@ -24,11 +24,8 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
-# Per-file additions.  The causal dK/dV attention kernel runs one wave per SIMD and depends on
-# the order of its own instructions; LLVM's iterative ILP scheduler orders it 4 % faster than
-# the default (measured on MI355X).  If a compiler does not know the option the file is built
-# without it.
-EXTRA_FLAGS = {"attention_dkv.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"]}
+# Per-file additions to FLAGS (none at present).
+EXTRA_FLAGS = {}
 
 
 def _hipcc() -> str:

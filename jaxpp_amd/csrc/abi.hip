@@ -318,7 +318,7 @@ size_t jpp_workspace_bytes(int op, int64_t d0, int64_t d1, int64_t d2) {
   switch (op) {
     case JPP_WS_NORM_BWD: return (size_t)2 * JPP_NORM_PARTIALS * d0 * 4;
     case JPP_WS_COLSUM: return (size_t)JPP_NORM_PARTIALS * d0 * 4;
-    case JPP_WS_ATTN_DELTA: return (size_t)d0 * d1 * d2 * 4;
+    case JPP_WS_ATTN_DELTA: return (size_t)2 * d0 * d1 * d2 * 4;
     case JPP_WS_MSE: return (size_t)JPP_NORM_PARTIALS * 4;
     case JPP_WS_MOE_WORK: return (size_t)2 * ((d0 + 255) / 256) * d1 * 4;
     case JPP_WS_MOE_ROUTER_WGRAD: return (size_t)64 * d0 * d1 * 4;

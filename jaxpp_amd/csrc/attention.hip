@@ -212,7 +212,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
   float lse2 = p.lse[stat] * kLog2e;
   // The row term delta = sum_d dO * O of this wave's 32 rows: a lane holds half of its row of
   // dO already (the chunks the MFMA fragment gives it) and reads the same half of O; the other
-  // half is with lane ^ 32.  Written out for the dK/dV kernel, which runs behind this one.
+  // half is with lane ^ 32.  Written out for the dK/dV kernel, which runs behind this one, in
+  // the form that kernel consumes: per row the pair {delta times the softmax scale, the
+  // log-sum-exp in the exp2 domain}.
   float dlt = 0.f;
   {
     const bf16_t* obase = p.o + (row0 + q0) * p.ldo + h * D;
@@ -226,9 +228,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
       for (int e = 0; e < 8; ++e) dlt = fmaf(of[e], gf[e], dlt);
     }
     dlt += __shfl_xor(dlt, 32);
-    if (lane < 32) p.delta[stat] = dlt;
+    dlt *= p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
+    if (lane < 32) *(float2*)(p.delta + 2 * stat) = make_float2(dlt, lse2);
   }
-  dlt *= p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
   const float sc = p.scale * kLog2e;
   settle(qf);
   settle(dof);
@@ -375,8 +377,9 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
   const uint32_t lds0 = lds_address(smem);
 
   // Q / dO tiles go HBM -> LDS directly; the 64 lse and 64 delta values of a
-  // block travel through one register per thread and are parked in LDS at the
-  // end of the previous iteration, so waiting for them never stalls the tiles.
+  // block (as the dQ kernel left them: exp2 domain, delta scaled) travel through
+  // one register per thread and are parked in LDS at the end of the previous
+  // iteration, so waiting for them never stalls the tiles.
   float rstat = 0.f;
   auto fetch = [&](int it, int stage) {
     const int hh = hk * grp + it / nqb;
@@ -384,14 +387,14 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
     const long stat = ((long)b * p.n_heads + hh) * p.seq + q0;
     // one unconditional load, consumed only in park(): nothing in between waits for it
     const int st = tid & 127;
-    rstat = *(st < 64 ? p.lse + stat + st : p.delta + stat + (st - 64));
+    rstat = p.delta[2 * (stat + (st & 63)) + (st < 64 ? 1 : 0)];
     const uint32_t dst = lds0 + stage * STAGE;
     dma_tile<D>(p.q + (row0 + q0) * p.ldq + hh * D, offq, dst, wave);
     dma_tile<D>(p.d_o + (row0 + q0) * p.lddo + hh * D, offdo, dst + TILE, wave);
   };
   auto park = [&](int stage) {
     float* st = (float*)(smem + stage * STAGE + 2 * TILE);
-    if (tid < 128) st[tid] = tid < 64 ? rstat * kLog2e : rstat * p.scale;  // delta parked scaled
+    if (tid < 128) st[tid] = rstat;
   };
 
   fetch(0, 0);

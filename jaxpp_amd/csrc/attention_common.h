@@ -75,6 +75,34 @@ __device__ __forceinline__ bf16x8 slabs_frag(const uint8_t* slabs, int row0, int
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// MFMAs as volatile asm statements, for the kernels that run one wave per SIMD and order
+// their own instructions: such statements are emitted where they are written, in the order
+// they are written, and LDS reads do not cross them.  The first letter names where the
+// accumulator lives, the other two the operands: `a` the accumulation registers (reached by
+// MFMAs and loads only), `v` the ordinary ones (where elementwise code can read a result).
+// The compiler does not know these statements are MFMAs: a kernel that uses them keeps every
+// other access to their results 11 issue slots behind them itself.
+#define JPP_MFMA(NAME, ACC, A, B)                                                          \
+  __device__ __forceinline__ void NAME(f32x16& acc, const bf16x8& a, const bf16x8& b) {    \
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"                                 \
+                 : "+" ACC(acc) : A(a), B(b) : "memory");                                  \
+  }
+JPP_MFMA(mfma_avv, "a", "v", "v")
+JPP_MFMA(mfma_vva, "v", "v", "a")
+JPP_MFMA(mfma_vvv, "v", "v", "v")
+#undef JPP_MFMA
+// the first product of a chain: the accumulator starts from zero
+__device__ __forceinline__ void mfma_vva_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b) : "memory");
+}
+// two floats -> one register of two bf16 (round to nearest even), one instruction
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
 // Makes the compiler wait here for the loads that produce these registers.  Without it the
 // wait lands at their first use inside the main loop as a vmcnt count, and there it also
 // waits for the HBM -> LDS copies of the next tile, which the wave has just issued (vmcnt
@@ -124,8 +152,7 @@ int set_smem(K kern, int bytes) {
   return JPP_OK;
 }
 
-// dK/dV under a causal mask (attention_dkv.hip, a translation unit of its own: it is built
-// with another instruction scheduler than the other kernels); grid (seq/128, kv heads, batch)
+// dK/dV under a causal mask (attention_dkv.hip); grid (seq/128, kv heads, batch)
 int launch_dkv_causal(hipStream_t stream, const AttnParams& p, int head_dim, dim3 grid);
 
 }  // namespace jpp_attn

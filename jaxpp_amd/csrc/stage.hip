@@ -899,7 +899,7 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
                                    (size_t)64 * h * 8 * 4,
                                    (size_t)JPP_NORM_PARTIALS * (size_t)(5 * h + f) * 4}));
   s->s_partial_side = sc.take(d->two_streams ? (size_t)64 * h * 8 * 4 : 256);
-  s->s_delta = sc.take((size_t)d->batch * d->n_heads * d->seq * 4);
+  s->s_delta = sc.take((size_t)2 * d->batch * d->n_heads * d->seq * 4);
   size_t max_w = 0;
   for (auto& p : s->pinfo) max_w = std::max(max_w, (size_t)(p.rows * p.cols));
   // unfused path: a bf16 weight gradient; fused path: partial products of a split contraction

@@ -68,7 +68,7 @@ def test_workspace_sizes():
     lib = rt.load()
     assert lib.jpp_workspace_bytes(0, 8192, 0, 0) == 2 * rt.NORM_PARTIALS * 8192 * 4     # norm backward
     assert lib.jpp_workspace_bytes(1, 1024 + 4096, 0, 0) == rt.NORM_PARTIALS * 5120 * 4  # column sums
-    assert lib.jpp_workspace_bytes(2, 2, 32, 4096) == 2 * 32 * 4096 * 4                  # attention delta
+    assert lib.jpp_workspace_bytes(2, 2, 32, 4096) == 2 * 2 * 32 * 4096 * 4                  # attention delta
     assert lib.jpp_workspace_bytes(3, 0, 0, 0) == rt.NORM_PARTIALS * 4
     assert lib.jpp_workspace_bytes(4, 8192, 8, 0) == 2 * 32 * 8 * 4
     assert lib.jpp_workspace_bytes(5, 4096, 8, 0) == 64 * 4096 * 8 * 4

@@ -241,7 +241,7 @@ def test_attention_f32(B, S, Hq, Hkv, d, causal):
                                        lse_w, causal, np.float64)
     b_qkv, b_do = dev(qkv), dev(do)
     o, lse = rt.DeviceBuffer(B * S * Hq * d * 4), rt.DeviceBuffer(B * Hq * S * 4)
-    dqkv, delta = rt.DeviceBuffer(B * S * w * 4), rt.DeviceBuffer(B * Hq * S * 4)
+    dqkv, delta = rt.DeviceBuffer(B * S * w * 4), rt.DeviceBuffer(2 * B * Hq * S * 4)
     a = rt.AttnArgs(b_qkv.ptr, b_qkv.ptr + Hq * d * 4, b_qkv.ptr + (Hq + Hkv) * d * 4, o.ptr, lse.ptr,
                     b_do.ptr, dqkv.ptr, dqkv.ptr + Hq * d * 4, dqkv.ptr + (Hq + Hkv) * d * 4, delta.ptr,
                     w, w, w, Hq * d, Hq * d, w, w, w, B, S, Hq, Hkv, d, int(causal))

@@ -260,7 +260,7 @@ def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
     dqkv_d.zero()
     b_qkv, b_o, b_do = dev_bf16(qkv), rt.DeviceBuffer(T * hq * d * 2), dev_bf16(do)
     b_lse = rt.DeviceBuffer(batch * hq * seq * 4)
-    b_delta = rt.DeviceBuffer(batch * hq * seq * 4)
+    b_delta = rt.DeviceBuffer(2 * batch * hq * seq * 4)
     a = rt.AttnArgs(b_qkv.ptr, b_qkv.ptr + hq * d * 2, b_qkv.ptr + (hq + hkv) * d * 2, b_o.ptr,
                     b_lse.ptr, b_do.ptr, dqkv_d.ptr, dqkv_d.ptr + hq * d * 2,
                     dqkv_d.ptr + (hq + hkv) * d * 2, b_delta.ptr,
