@@ -168,7 +168,10 @@ typedef struct {
    * (a, b), then (a_more[0], b_more[0]), ... - k elements each, same shapes and leading
    * dimensions - as if the pairs were concatenated along the contraction index.  The
    * weight gradients of several microbatches accumulate this way with one read and one write
-   * of the fp32 accumulator instead of one per microbatch.  0 or 1: one pair. */
+   * of the fp32 accumulator instead of one per microbatch.  0 or 1: one pair.  Built for
+   * trans_a = trans_b = 1 with JPP_EPI_ACC_F32 on the 256-wide tiles: N a multiple of 256,
+   * `tile` 0 (the library then takes 256x256, or 128x256 when M is not a multiple of 256),
+   * 3 or 4; anything else is JPP_ERR_INVALID. */
   const void* a_more[3];
   const void* b_more[3];
   int k_parts;
@@ -443,9 +446,14 @@ typedef struct {
                             chunk beyond max_live, and jpp_stage_live_slots counts them);
                             jpp_stage_join runs what is still held back, so call it (or
                             jpp_stage_zero_grads / jpp_stage_adam_step, which do) before reading
-                            the accumulators.  Groups are fixed by microbatch index, so the
-                            accumulators do not depend on the order of tasks.  One stream,
-                            bf16, fused_wgrad_accum only. */
+                            the accumulators.  Groups are fixed by microbatch index and a
+                            group's operand pairs enter its product in microbatch order, so
+                            the accumulators do not depend on the order in which the members
+                            of a group arrive; a member of another group of the same chunk
+                            arriving in between sends what is pending ahead as a shorter
+                            product (same sums, other rounding).  If a grouped launch fails
+                            the stage is unusable: every later task and join returns
+                            JPP_ERR_STATE.  One stream, bf16, fused_wgrad_accum only. */
 } jpp_stage_desc;
 
 

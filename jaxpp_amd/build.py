@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libjaxpp_amd.so")
-SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "attention_dkv.hip", "elementwise.hip",
+SOURCES = ["abi.hip", "gemm.hip", "attention.hip", "attention_dq.hip", "attention_dkv.hip", "elementwise.hip",
            "moe.hip", "optimizer.hip", "f32_ops.hip", "stage.hip"]
 # measurement aids: a library of their own beside the product library
 DIAG_LIB = os.path.join(LIBDIR, "libjaxpp_amd_diag.so")

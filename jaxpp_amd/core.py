@@ -26,7 +26,7 @@ import numpy as np
 from jaxpp_amd import tracing
 from jaxpp_amd.mesh import MpmdMesh
 from jaxpp_amd.schedules import (BaseSchedule, FusedTask, Task, mk_task_name,
-                                 preprocess_schedule_tasks)
+                                 preprocess_schedule_tasks, schedule_task_fusion_disabled)
 from jaxpp_amd.types import TaskType
 
 # ---------------------------------------------------------------------------
@@ -243,9 +243,11 @@ def order_tasks(rows: list, num_stages: int) -> list:
 
 
 def validate_schedule(schedule: BaseSchedule, n_mubatches: int,
-                      unpack_fused_tasks: bool = False) -> list:
+                      unpack_fused_tasks: bool | None = None) -> list:
     """Preprocess the table and check it against the task graph; returns the
-    global order."""
+    global order.  `unpack_fused_tasks` None: as JAXPP_DISABLE_SCHEDULE_TASK_FUSION says."""
+    if unpack_fused_tasks is None:
+        unpack_fused_tasks = schedule_task_fusion_disabled()
     rows = preprocess_schedule_tasks(schedule.tasks(n_mubatches), 0, unpack_fused_tasks)
     seen = set()
     for row in rows:
@@ -371,7 +373,8 @@ def run_loop(tr, outputs, ops, n: int, schedule: BaseSchedule):
     mesh = fn.mpmd_mesh
     body = cluster_ops(tr, schedule.num_stages)
     S = schedule.num_stages
-    rows = preprocess_schedule_tasks(schedule.tasks(n), 0, False)
+    # (src/jaxpp/core.py:2559-2563: the environment decides whether fused entries stay fused)
+    rows = preprocess_schedule_tasks(schedule.tasks(n), 0, schedule_task_fusion_disabled())
     if len(rows) != mesh.mpmd_dim:
         raise AssertionError(f"schedule places tasks on {len(rows)} MPMD groups, the mesh has "
                              f"{mesh.mpmd_dim}")

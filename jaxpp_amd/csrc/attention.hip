@@ -1,5 +1,6 @@
 // Fused attention for gfx950: forward with online softmax, and a two-kernel
-// deterministic backward (dQ per query block, dK/dV per key block; no atomics).
+// deterministic backward (dQ per query block, attention_dq.hip; dK/dV per key block, here
+// without a mask and in attention_dkv.hip under one; no atomics).
 //
 // Everything runs on v_mfma_f32_32x32x16_bf16.  Scores are computed transposed
 // where that lets the probabilities feed the next MFMA straight from the
@@ -180,7 +181,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// backward, dQ: one workgroup per 128 queries of one head
+// backward, dQ without a causal mask (short sequences; under a mask: attention_dq.hip):
+// one workgroup per 128 queries of one head, 32 per wave, two workgroups per CU
 // ---------------------------------------------------------------------------
 template <int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
@@ -555,6 +557,8 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
                   ((uintptr_t)a->d_o | (uintptr_t)a->dq | (uintptr_t)a->dk | (uintptr_t)a->dv) % 16 == 0,
               "attn_bwd: operands must keep 16-byte alignment");
   JPP_REQUIRE(!a->rope_cos == !a->rope_sin, "attn_bwd: rope_cos and rope_sin go together");
+  JPP_REQUIRE(((uintptr_t)a->rope_cos | (uintptr_t)a->rope_sin) % 16 == 0,
+              "attn_bwd: rotary tables must be 16-byte aligned");
   AttnParams p = make_params(a);
   // the causal kernels rotate dq / dk back themselves; without a mask a pass of its own does
   const bool fused_rope = a->rope_cos && a->causal;
@@ -567,10 +571,14 @@ extern "C" int jpp_attn_bwd(void* stream, const jpp_attn_args* a) {
                     (a->causal ? 0.5 : 1.0);
 #define JPP_AB(D_, C_)                                                              \
   do {                                                                              \
-    if (int rc = set_smem(attn_bwd_dq_kernel<D_, C_>, 4 * D_ * 128)) return rc;     \
     {                                                                               \
       ProbeScope probe(st, "attn_bwd_dq", fl * 0.4, 0);                             \
-      hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, C_>), gq, dim3(256), 4 * D_ * 128, st, p); \
+      if (C_) {                                                                     \
+        if (int rc = launch_dq(st, p, D_, true)) return rc;                         \
+      } else {                                                                      \
+        if (int rc = set_smem(attn_bwd_dq_kernel<D_, false>, 4 * D_ * 128)) return rc; \
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, false>), gq, dim3(256), 4 * D_ * 128, st, p); \
+      }                                                                             \
     }                                                                               \
     ProbeScope probe(st, "attn_bwd_dkv", fl * 0.6, 0);                              \
     if (C_) {                                                                       \

@@ -152,6 +152,8 @@ int set_smem(K kern, int bytes) {
   return JPP_OK;
 }
 
+// dQ and the row statistics the dK/dV kernels read (attention_dq.hip)
+int launch_dq(hipStream_t stream, const AttnParams& p, int head_dim, bool causal);
 // dK/dV under a causal mask (attention_dkv.hip); grid (seq/128, kv heads, batch)
 int launch_dkv_causal(hipStream_t stream, const AttnParams& p, int head_dim, dim3 grid);
 

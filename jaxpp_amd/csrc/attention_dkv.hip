@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     int f_h = 0, f_left = total;
     // part j of an item's loads (NLOAD of them per wave: the Q tile's, the dO tile's, the row
     // statistics); the last part moves the cursor on
-    auto fetch_part = [&](int slot, int j) {
+    auto fetch_part = [&](int slot, int j) __attribute__((always_inline)) {
       const uint32_t dst = lds0 + slot * SLOT;
       constexpr int PER = Tile64::INSTS;  // loads per wave and 64-column slab
       if (j < NLOAD - 1) {
@@ -109,13 +109,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
       f_do += wrap ? -(head_back + 64 * p.lddo) : (go ? D : 0);
       f_st += wrap ? -2 * ((long)(grp - 1) * p.seq + 64) : (go ? 2 * (long)p.seq : 0);
     };
-    auto fetch = [&](int slot) {
+    auto fetch = [&](int slot) __attribute__((always_inline)) {
 #pragma unroll
       for (int j = 0; j < NLOAD; ++j) fetch_part(slot, j);
     };
 
     // S and dP of an item (its tiles in `slot`) against this wave's keys
-    auto scores = [&](const uint8_t* slot, f32x16& s, f32x16& dp) {
+    auto scores = [&](const uint8_t* slot, f32x16& s, f32x16& dp) __attribute__((always_inline)) {
       bf16x8 qfr[KS], dofr[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     // Items of the key block's own query block are masked: the query half behind the keys
     // sees all of them, the half in front none, the one on the diagonal what lies at or
     // before each query.  Items past the end (an odd count is rounded up) count as unseen.
-    auto mask = [&](f32x16& s, int item) {
+    auto mask = [&](f32x16& s, int item) __attribute__((always_inline)) {
       if (item >= total - grp) {  // wave-uniform
         if (item >= total || qh < ksb) {
 #pragma unroll
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < DT; ++i) { dotr[h2][i] = pf[h2]; qtr[h2][i] = pf[h2]; }
     }
-    auto grads = [&]() {
+    auto grads = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     // the instruction stream.  The MFMAs of a trip are volatile asm statements (they keep
     // their order, and LDS reads do not cross them); the elementwise work is tied to its place
     // by empty asm statements on its inputs and results.
-    auto trip = [&](auto tail, int i, f32x16& s_c, f32x16& dp_c, f32x16& s_n, f32x16& dp_n) {
+    auto trip = [&](auto tail, int i, f32x16& s_c, f32x16& dp_c, f32x16& s_n, f32x16& dp_n) __attribute__((always_inline)) {
       constexpr bool TAIL = decltype(tail)::value;
       const uint8_t* sl_c = smem + (i & 3) * SLOT;
       const uint8_t* sl_n = smem + ((i + 1) & 3) * SLOT;
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
       }
       // row statistics of item i: {scaled delta, lse} pairs, two rows per 16-byte read
       const float* st = (const float*)(sl_c + 2 * TILE) + 2 * ql0;
-      auto stats = [&](int r) { return *(const float4*)(st + 2 * ((r >> 2) * 8 + (r & 3))); };
+      auto stats = [&](int r) __attribute__((always_inline)) { return *(const float4*)(st + 2 * ((r >> 2) * 8 + (r & 3))); };
       float4 st_q[3] = {stats(0), stats(2), stats(4)};  // read two pairs of rows ahead of their use
       // dV / dK products of item i - 1 from registers (the reads above arrive under them);
       // behind each pair, the transposed fragments of item i take over its registers

@@ -929,6 +929,10 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
   int tile = a->tile ? a->tile : choose_tile(a->m, a->n);
   // row groups come in 256-row segments; a contraction split into groups takes any tile
   if (a->group_mode == JPP_GROUP_M || (a->group_mode == JPP_GROUP_K && !a->tile)) tile = 4;
+  // several operand pairs exist on the 256-wide tiles only: a tile left to the library goes
+  // there whatever the problem's size (N not a multiple of 256 is refused below, with the
+  // kernel's message)
+  if (a->k_parts > 1 && !a->tile) tile = 4;
   JPP_REQUIRE(tile >= 1 && tile <= 4, "gemm: unknown tile %d", tile);
   if ((tile == 2 || tile == 4) && a->m % 256) tile = a->n % 256 ? 1 : 3;
   if ((tile == 3 || tile == 4) && a->n % 256) tile = a->m % 256 ? 1 : 2;

@@ -109,6 +109,7 @@ struct jpp_stage {
   // gradient half is done and whose weight-gradient half waits for the rest of its group.
   int wg = 1;
   std::vector<std::vector<std::pair<int, int>>> pend;
+  bool broken = false;   // a grouped weight-gradient launch failed half way: accumulators unusable
 
   bool f32() const { return d.dtype == JPP_DTYPE_F32; }
   void* P(int chunk, int layer, int i) {
@@ -684,15 +685,21 @@ int layer_bwd_w_group(jpp_stage* s, hipStream_t st, int chunk, int li, int n, ui
 }
 
 // Runs the pending weight-gradient halves of a chunk (a whole group, or what a flush finds)
-// and releases their slots.
+// and releases their slots.  The operand pairs go into the product in microbatch order,
+// whatever order the tasks arrived in.  If a launch fails, gradients of the layers above it
+// have already been accumulated and nothing can take them back: the stage is marked broken
+// (every later task and join reports JPP_ERR_STATE) instead of leaving entries pending that
+// a later flush would accumulate a second time.
 int run_pending_w(jpp_stage* s, hipStream_t st, int chunk) {
   auto& pend = s->pend[chunk];
   if (pend.empty()) return JPP_OK;
+  std::sort(pend.begin(), pend.end());
   uint8_t* slots[4];
   const int n = (int)pend.size();
   for (int i = 0; i < n; ++i) slots[i] = s->slots[pend[i].second];
-  for (int li = s->d.layers_per_chunk - 1; li >= 0; --li)
-    RC(layer_bwd_w_group(s, st, chunk, li, n, slots));
+  int rc = JPP_OK;
+  for (int li = s->d.layers_per_chunk - 1; li >= 0 && rc == JPP_OK; --li)
+    rc = layer_bwd_w_group(s, st, chunk, li, n, slots);
   for (auto& e : pend) {
     const auto key = std::make_pair(chunk, e.first);
     s->free_slots.push_back(e.second);
@@ -700,16 +707,18 @@ int run_pending_w(jpp_stage* s, hipStream_t st, int chunk) {
     s->phase.erase(key);
   }
   pend.clear();
-  return JPP_OK;
+  if (rc != JPP_OK) s->broken = true;
+  return rc;
 }
 
 // The input-gradient half of (chunk, mb) is done: its weight-gradient half runs now if it
-// completes its group (microbatches mb / G * G .. + G - 1), else it waits.
+// completes its group (microbatches mb / G * G .. + G - 1, in any order), else it waits; a
+// microbatch of another group arriving first sends what is pending ahead as it is.
 int defer_or_run_w(jpp_stage* s, hipStream_t st, int chunk, int mb, int slot_i) {
   auto& pend = s->pend[chunk];
   if (!pend.empty() && pend.front().first / s->wg != mb / s->wg) RC(run_pending_w(s, st, chunk));
   pend.emplace_back(mb, slot_i);
-  if (mb % s->wg == s->wg - 1 || (int)pend.size() == s->wg) RC(run_pending_w(s, st, chunk));
+  if ((int)pend.size() == s->wg) RC(run_pending_w(s, st, chunk));
   return JPP_OK;
 }
 
@@ -1042,6 +1051,9 @@ int jpp_stage_grad_ptr(jpp_stage* s, int chunk, int layer, int i, float** ptr) {
 
 int jpp_stage_join(jpp_stage* s, void* stream) {
   JPP_REQUIRE(s, "stage: null");
+  if (s->broken)
+    return jpp_set_error(JPP_ERR_STATE, "stage_join: a grouped weight-gradient launch of this "
+                         "stage failed earlier; its accumulators are incomplete");
   RC(flush_pending_w(s, (hipStream_t)stream));   // weight gradients held back for their group
   if (s->tail_pending) JPP_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, s->ev_tail, 0));
   return JPP_OK;
@@ -1144,6 +1156,9 @@ int jpp_stage_live_slots(const jpp_stage* s) { return s ? (int)s->live.size() : 
 int jpp_stage_run_task(jpp_stage* s, int kind, int chunk, int mb, const void* in, void* out,
                        void* stream) {
   JPP_REQUIRE(s, "run_task: null stage");
+  if (s->broken)
+    return jpp_set_error(JPP_ERR_STATE, "run_task: a grouped weight-gradient launch of this stage "
+                         "failed earlier; its accumulators are incomplete");
   JPP_REQUIRE(chunk >= 0 && chunk < s->d.n_chunks, "run_task: chunk %d out of range", chunk);
   hipStream_t st = (hipStream_t)stream;
   const int nl = s->d.layers_per_chunk;

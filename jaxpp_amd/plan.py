@@ -13,7 +13,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
-from jaxpp_amd.schedules import BaseSchedule, FusedTask, Task, preprocess_schedule_tasks
+from jaxpp_amd.schedules import (BaseSchedule, FusedTask, Task, preprocess_schedule_tasks,
+                                 schedule_task_fusion_disabled)
 from jaxpp_amd.types import TaskType
 
 
@@ -43,7 +44,11 @@ def stages_of_rank(schedule: BaseSchedule, rank: int) -> list:
 
 
 def make_rank_plan(schedule: BaseSchedule, n_mubatches: int, rank: int,
-                   unpack_fused_tasks: bool = False, first_stage_id: int = 0) -> RankPlan:
+                   unpack_fused_tasks: bool | None = None, first_stage_id: int = 0) -> RankPlan:
+    """`unpack_fused_tasks` None: as the environment says (JAXPP_DISABLE_SCHEDULE_TASK_FUSION,
+    the reference's switch, read where it unrolls the loop: src/jaxpp/core.py:2559-2563)."""
+    if unpack_fused_tasks is None:
+        unpack_fused_tasks = schedule_task_fusion_disabled()
     rows = preprocess_schedule_tasks(schedule.tasks(n_mubatches), first_stage_id,
                                      unpack_fused_tasks)
     if not 0 <= rank < len(rows):

@@ -13,6 +13,7 @@ rank, whose entries are executed in order by that rank.
 from __future__ import annotations
 
 import dataclasses
+import os
 from abc import ABCMeta, abstractmethod
 from collections import defaultdict
 from dataclasses import dataclass, field
@@ -24,7 +25,8 @@ __all__ = [
     "Task", "FusedTask", "ScheduleTasks", "BaseSchedule",
     "InterleavedBaseSchedule", "Std1F1B", "Eager1F1B", "GPipe", "ZeroBubble",
     "Interleaved1F1B", "KimiK2", "DualPipeV", "dualpipev_tasks",
-    "preprocess_schedule_tasks", "check_and_strip_adjecent_bwd_a_bwd_w",
+    "preprocess_schedule_tasks", "schedule_task_fusion_disabled",
+    "check_and_strip_adjecent_bwd_a_bwd_w",
     "strip_nones", "unpack_fused_tasks_fn", "mk_task_name",
 ]
 
@@ -467,6 +469,21 @@ def check_and_strip_adjecent_bwd_a_bwd_w(tasks: Sequence, first_stage_id: Any) -
             out.append(t)
         i += 1
     return out
+
+
+def schedule_task_fusion_disabled() -> bool:
+    """The reference's ``JAXPP_DISABLE_SCHEDULE_TASK_FUSION`` switch (src/jaxpp/env_vars.py:10-12,
+    read where the loop is unrolled, src/jaxpp/core.py:2559-2563): when set, fused entries of a
+    schedule's table are run as their members, one after the other.  Same spellings as the
+    reference's ``parse_bool`` (src/jaxpp/utils.py:87-92); anything else is an error."""
+    v = os.environ.get("JAXPP_DISABLE_SCHEDULE_TASK_FUSION")
+    if v is None:
+        return False
+    if v.lower() in ("true", "1", "t", "y", "yes"):
+        return True
+    if v.lower() in ("false", "0", "f", "n", "no"):
+        return False
+    raise ValueError(f"Unsupported value JAXPP_DISABLE_SCHEDULE_TASK_FUSION={v}")
 
 
 def preprocess_schedule_tasks(schedule: ScheduleTasks, first_stage_id,

@@ -13,6 +13,11 @@ fp32 1e-4 of it.  The number of elements that break the bound is reported and mu
 unless the caller grants a fraction (tensors whose elements are long sums of rounded
 intermediates; the cap is written at the call).  The older, weaker bound on the largest error
 against the largest magnitude is kept as a second assertion.
+
+The bf16 oracle rounds where the kernels round, so agreement with it says that the device
+follows the same arithmetic, not how good that arithmetic is.  `close_to_truth` is the anchor
+for that: the device result may be no farther from the unrounded computation (the oracle in
+float32 on the same bf16 inputs) than the bf16 oracle itself is, by a stated factor.
 """
 from __future__ import annotations
 
@@ -81,3 +86,35 @@ def close(got, want, rtol: float, what: str = "", max_bad_frac: float = 0.0,
         f"rtol {rtol:g} * (|want| + rms); worst at {worst:.3g} x the bound "
         f"(allowed fraction {max_bad_frac:g}){where_bad(got, want, rtol)}")
     assert worst <= max_excess, f"{what}: an element is {worst:.3g} x outside the elementwise bound"
+
+
+# How much farther from the unrounded result than the bf16 oracle the device may be: in the
+# Frobenius norm (an average over the tensor: tight), and in the largest error (one element:
+# noisier, so looser).
+TRUTH_FRO = 1.5
+TRUTH_MAX = 2.5
+
+
+def close_to_truth(got, want_bf16, want_f32, what: str = "", fro: float = TRUTH_FRO,
+                   mx: float = TRUTH_MAX):
+    """`got`: the device's bf16-path result; `want_bf16`: the oracle with bf16 storage rounding;
+    `want_f32`: the oracle in float32 on the same (bf16-valued) inputs.  Asserts
+        ||got - want_f32||_F <= fro * ||want_bf16 - want_f32||_F   and
+        max|got - want_f32|  <= mx  * max|want_bf16 - want_f32|,
+    each with a floor of one bf16 ulp (2^-8) of the tensor's rms / largest value per element,
+    below which a bf16 result cannot be told from the truth."""
+    got = np.asarray(got, np.float64)
+    b = np.asarray(want_bf16, np.float64).reshape(got.shape)
+    t = np.asarray(want_f32, np.float64).reshape(got.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite"
+    ulp = 2.0 ** -8
+    e_got, e_ref = np.linalg.norm(got - t), np.linalg.norm(b - t)
+    floor_f = ulp * np.linalg.norm(t)
+    assert e_got <= fro * max(e_ref, floor_f), (
+        f"{what}: distance to the float32 result {e_got:.4g} (Frobenius) against the bf16 "
+        f"oracle's own {e_ref:.4g}: {e_got / max(e_ref, 1e-300):.2f} x, allowed {fro} x")
+    m_got, m_ref = float(np.abs(got - t).max()), float(np.abs(b - t).max())
+    floor_m = ulp * float(np.abs(t).max())
+    assert m_got <= mx * max(m_ref, floor_m), (
+        f"{what}: largest distance to the float32 result {m_got:.4g} against the bf16 oracle's "
+        f"own {m_ref:.4g}: {m_got / max(m_ref, 1e-300):.2f} x, allowed {mx} x")

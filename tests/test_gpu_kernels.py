@@ -164,9 +164,8 @@ def test_gemm_several_weight_gradients_in_one_launch(parts, k, shapes):
         close(g, w, 1e-4 * math.sqrt(k * parts), f"multi {shp}")
     for (dA, dB, dc), prev, (m, n), g in zip(keep, prevs, shapes, got):
         dc.upload(prev)
-        # (several operand pairs: only the 256-wide tiles are built for that)
+        # (several operand pairs: the library takes the 256-wide tiles built for that itself)
         rt.gemm(dA[0].ptr, dB[0].ptr, dc.ptr, m, n, k, m, n, n, 1, 1, rt.EPI_ACC_F32,
-                tile=4 if parts > 1 and (m // 256) * (n // 256) < 192 else 0,
                 more=[(a.ptr, b.ptr) for a, b in zip(dA[1:], dB[1:])])
         rt.sync()
         np.testing.assert_array_equal(dc.download(np.float32, (m, n)), g)
@@ -294,6 +293,13 @@ def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
     rt.check(rt.load().jpp_attn_bwd(None, C.byref(a)))
     rt.sync()
     np.testing.assert_array_equal(dqkv_d.download_bf16((T, width)), want_r)
+    # the kernels read the tables 16 bytes at a time: a table that is not aligned so is refused
+    a.rope_cos = bc.ptr + 4
+    with pytest.raises(rt.JppError, match="rotary tables must be 16-byte aligned"):
+        rt.check(rt.load().jpp_attn_bwd(None, C.byref(a)))
+    a.rope_cos, a.rope_sin = bc.ptr, None
+    with pytest.raises(rt.JppError, match="rope_cos and rope_sin go together"):
+        rt.check(rt.load().jpp_attn_bwd(None, C.byref(a)))
 
 
 @pytest.mark.parametrize("d,causal,slope", [(128, 1, 40.0), (128, 0, 40.0), (64, 1, 12.0),

@@ -287,3 +287,34 @@ def test_stage_lifetimes_per_stage():
     rows = S.preprocess_schedule_tasks(S.Interleaved1F1B(4, 2).tasks(4), 0, False)
     peak, split = core._stage_lifetimes(rows, 4)
     assert split == [False] * 4 and all(1 <= p <= 4 for p in peak)
+
+
+def test_schedule_task_fusion_switch(monkeypatch):
+    """JAXPP_DISABLE_SCHEDULE_TASK_FUSION (src/jaxpp/env_vars.py:10-12, read at
+    src/jaxpp/core.py:2559-2563): with it set, a rank's plan and the global order run the
+    members of a fused table entry one after the other; spellings as the reference's
+    parse_bool, anything else an error."""
+    sched, n = S.Interleaved1F1B(num_stages=4, mpmd_dim=2, fuse_steady_state=True), 8
+    monkeypatch.delenv("JAXPP_DISABLE_SCHEDULE_TASK_FUSION", raising=False)
+    fused = make_rank_plan(sched, n, 0)
+    groups = [pt.group for pt in fused.tasks]
+    assert len(set(groups)) < len(groups)                  # some entries hold two tasks
+    for spelling in ("1", "true", "T", "yes", "Y"):
+        monkeypatch.setenv("JAXPP_DISABLE_SCHEDULE_TASK_FUSION", spelling)
+        assert S.schedule_task_fusion_disabled()
+        flat = make_rank_plan(sched, n, 0)
+        assert len({pt.group for pt in flat.tasks}) == len(flat.tasks)
+        assert [pt.task for pt in flat.tasks] == [pt.task for pt in fused.tasks]
+        assert flat.max_live == fused.max_live
+        order = core.validate_schedule(sched, n)
+        assert all(not isinstance(e.entry, S.FusedTask) for e in order)
+    for spelling in ("0", "false", "no"):
+        monkeypatch.setenv("JAXPP_DISABLE_SCHEDULE_TASK_FUSION", spelling)
+        assert not S.schedule_task_fusion_disabled()
+        assert [pt.group for pt in make_rank_plan(sched, n, 0).tasks] == groups
+    # an explicit argument wins over the environment
+    monkeypatch.setenv("JAXPP_DISABLE_SCHEDULE_TASK_FUSION", "1")
+    assert [pt.group for pt in make_rank_plan(sched, n, 0, unpack_fused_tasks=False).tasks] == groups
+    monkeypatch.setenv("JAXPP_DISABLE_SCHEDULE_TASK_FUSION", "maybe")
+    with pytest.raises(ValueError, match="Unsupported value JAXPP_DISABLE_SCHEDULE_TASK_FUSION=maybe"):
+        make_rank_plan(sched, n, 0)

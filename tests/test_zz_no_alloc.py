@@ -2,7 +2,10 @@
 the library's own static device buffer - against jpp_norm_bwd with a caller-provided
 workspace: same kernels, so dx and the accumulated scale / shift gradients must be
 bit-identical.  Two calls in a row share the buffer, the second on a smaller input (fewer
-rows and columns than the first left behind); a call beyond the buffer's width is refused."""
+rows and columns than the first left behind); a call beyond the buffer's width is refused.
+What the entry point is for - callers that cannot allocate - is checked directly: after a first
+call it runs under stream capture and replays bit for bit, and the device's free memory is the
+same after the calls as before."""
 import ctypes as C
 
 import numpy as np
@@ -76,3 +79,45 @@ def test_static_scratch_entry_point_rejects_rows_wider_than_its_buffer():
                     1, 8192 + 8, 1e-5)
     assert lib.jpp_norm_bwd_static(None, C.byref(a)) == -1
     assert b"exceed" in lib.jpp_last_error()
+
+
+def test_static_scratch_entry_point_allocates_nothing_and_runs_under_capture():
+    rt.require_gpu()
+    lib = rt.load()
+    rng = np.random.default_rng(12)
+    c = _case(rng, False, 200, 2048)
+    want = _run(c, static=False)
+    rows, cols = c["rows"], c["cols"]
+    up = rt.DeviceBuffer.from_f32_as_bf16
+    bx, bg, bdy, br = up(c["x"]), up(c["g"]), up(c["dy"]), up(c["resid"])
+    by, bdx = rt.DeviceBuffer(rows * cols * 2), rt.DeviceBuffer(rows * cols * 2)
+    brstd = rt.DeviceBuffer(rows * 4)
+    bdg = rt.DeviceBuffer.from_numpy(c["acc_g"])
+    a = rt.NormArgs(bx.ptr, bg.ptr, None, by.ptr, None, brstd.ptr, bdy.ptr, br.ptr, bdx.ptr,
+                    bdg.ptr, None, None, rows, cols, 1e-5)
+    rt.check(lib.jpp_norm_fwd(None, C.byref(a)))
+    rt.check(lib.jpp_norm_bwd_static(None, C.byref(a)))      # first call on this device: the
+    rt.sync()                                                # address lookup happens here
+    stream = rt.Stream()
+    graph = rt.Graph(stream)
+    with graph:                                              # an allocation or a symbol lookup
+        rt.check(lib.jpp_norm_bwd_static(stream.ptr, C.byref(a)))   # here would fail the capture
+    graph.launch()                                           # (the runtime's own set-up of a
+    stream.sync()                                            # first replay is not counted)
+    free0, total = C.c_size_t(), C.c_size_t()
+    rt.check(lib.jpp_mem_info(C.byref(free0), C.byref(total)))
+    for replay in range(3):
+        bdg.upload(c["acc_g"])
+        bdx.zero()
+        rt.sync()
+        graph.launch()
+        stream.sync()
+        np.testing.assert_array_equal(bdx.download(np.uint16, (rows, cols)), want[0],
+                                      err_msg=f"dx, replay {replay}")
+        np.testing.assert_array_equal(bdg.download(np.float32, (cols,)), want[1],
+                                      err_msg=f"dgamma, replay {replay}")
+        rt.check(lib.jpp_norm_bwd_static(None, C.byref(a)))  # eager work between the replays
+        rt.sync()
+    free1 = C.c_size_t()
+    rt.check(lib.jpp_mem_info(C.byref(free1), C.byref(total)))
+    assert free1.value == free0.value, "the static entry point (or its replays) allocated device memory"
