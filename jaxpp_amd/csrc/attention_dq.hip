@@ -50,62 +50,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   const float sc = p.scale * kLog2e;
   const uint32_t lds0 = lds_address(smem);
 
-  // this wave's Q and dO as MFMA operands (accumulation registers), and per query tile the
-  // row's log-sum-exp (exp2 domain) and delta (times the softmax scale); delta = sum_d dO * O:
-  // a lane holds half of its row of dO (the chunks the fragments give it) and reads the same
-  // half of O, the other half is with lane ^ 32
-  bf16x8 qf[2][KS], dof[2][KS];
-  float lse2[2] = {0.f, 0.f}, dlt[2] = {0.f, 0.f};
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
-    if (active) {
-      const long r = row0 + q0 + qt * 32;
-      const bf16_t* qbase = p.q + r * p.ldq + h * D;
-      const bf16_t* dobase = p.d_o + r * p.lddo + h * D;
-      const bf16_t* obase = p.o + r * p.ldo + h * D;
-      const long stat = ((long)b * p.n_heads + h) * p.seq + q0 + qt * 32 + (lane & 31);
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        qf[qt][ks] = global_frag(qbase, p.ldq, ks, lane);
-        dof[qt][ks] = global_frag(dobase, p.lddo, ks, lane);
-      }
-      lse2[qt] = p.lse[stat] * kLog2e;
-      float acc = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const uint4 ov = *(const uint4*)(obase + (long)(lane & 31) * p.ldo + ks * 16 + (lane >> 5) * 8);
-        float of[8], gf[8];
-        unpack8(ov, of);
-        unpack8(__builtin_bit_cast(uint4, dof[qt][ks]), gf);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc = fmaf(of[e], gf[e], acc);
-      }
-      acc += __shfl_xor(acc, 32);
-      dlt[qt] = acc * p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
-      // for the dK/dV kernel, in the form it consumes: {scaled delta, lse} per row
-      if (lane < 32) *(float2*)(p.delta + 2 * stat) = make_float2(dlt[qt], lse2[qt]);
-    } else {
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { qf[qt][ks][e] = (__bf16)0.f; dof[qt][ks][e] = (__bf16)0.f; }
-    }
-  }
-  // (waits for the loads here, and names where the fragments live)
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qf[qt][ks]), "+a"(dof[qt][ks]));
-  settle(lse2[0]); settle(lse2[1]); settle(dlt[0]); settle(dlt[1]);
-
-  f32x16 dqacc[2][DT];
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-    for (int i = 0; i < DT; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) dqacc[qt][i][r] = 0.f;
-
   const bf16_t* kbase = p.k + row0 * p.ldk + hk * D;
   const bf16_t* vbase = p.v + row0 * p.ldv + hk * D;
   Tile64::Offsets offk, offv;
@@ -127,6 +71,74 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
     for (int j = 0; j < NLOAD; ++j) fetch_part(block, j);
   };
+  // the first three key blocks are on their way while this wave's own operands arrive
+  fetch(0);
+  fetch(1);
+  fetch(2);
+
+  // This wave's Q and dO as MFMA operands (accumulation registers), and per query tile the
+  // row's log-sum-exp (exp2 domain) and delta (times the softmax scale); delta = sum_d dO * O:
+  // a lane holds half of its row of dO (the chunks the fragments give it) and reads the same
+  // half of O, the other half is with lane ^ 32.  All loads are issued before the first of
+  // them is waited for.
+  bf16x8 qf[2][KS], dof[2][KS];
+  uint4 ov[2][KS];
+  float lse2[2] = {0.f, 0.f}, dlt[2] = {0.f, 0.f};
+  if (active) {
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      const long r = row0 + q0 + qt * 32;
+      const bf16_t* qbase = p.q + r * p.ldq + h * D;
+      const bf16_t* dobase = p.d_o + r * p.lddo + h * D;
+      const bf16_t* obase = p.o + r * p.ldo + h * D;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        qf[qt][ks] = global_frag(qbase, p.ldq, ks, lane);
+        dof[qt][ks] = global_frag(dobase, p.lddo, ks, lane);
+        ov[qt][ks] = *(const uint4*)(obase + (long)(lane & 31) * p.ldo + ks * 16 + (lane >> 5) * 8);
+      }
+      lse2[qt] = p.lse[((long)b * p.n_heads + h) * p.seq + q0 + qt * 32 + (lane & 31)];
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      const long stat = ((long)b * p.n_heads + h) * p.seq + q0 + qt * 32 + (lane & 31);
+      lse2[qt] *= kLog2e;
+      float acc = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        float of[8], gf[8];
+        unpack8(ov[qt][ks], of);
+        unpack8(__builtin_bit_cast(uint4, dof[qt][ks]), gf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = fmaf(of[e], gf[e], acc);
+      }
+      acc += __shfl_xor(acc, 32);
+      dlt[qt] = acc * p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
+      // for the dK/dV kernel, in the form it consumes: {scaled delta, lse} per row
+      if (lane < 32) *(float2*)(p.delta + 2 * stat) = make_float2(dlt[qt], lse2[qt]);
+    }
+  } else {
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { qf[qt][ks][e] = (__bf16)0.f; dof[qt][ks][e] = (__bf16)0.f; }
+  }
+  // (names where the fragments live from here on)
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qf[qt][ks]), "+a"(dof[qt][ks]));
+  settle(lse2[0]); settle(lse2[1]); settle(dlt[0]); settle(dlt[1]);
+
+  f32x16 dqacc[2][DT];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dqacc[qt][i][r] = 0.f;
 
   // state of the pipeline between trips
   bf16x8 kfr[KS], vfr[KS];   // K / V rows of the 32-key tile whose scores come next
@@ -246,10 +258,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     if (TAIL) mask(s_a, j + 1, 0, 0);
   };
 
-  fetch(0);
-  fetch(1);
-  fetch(2);
-  dma_wait<NLOAD>();
+  dma_wait<NLOAD>();   // blocks 0 and 1 are in (block 2 may be on its way)
   __syncthreads();
   if (active) {
 #pragma unroll
@@ -316,10 +325,14 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
     for (int i = 0; i < DT; ++i) asm volatile("s_nop 15" : "+a"(dqacc[qt][i]));
+  if (p.rope_cos) {
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+      rope_back<D, DT>(dqacc[qt], p.rope_cos, p.rope_sin, q0 + qt * 32 + (lane & 31), lane);
+  }
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
     const int qi = q0 + qt * 32 + (lane & 31);
-    if (p.rope_cos) rope_back<D, DT>(dqacc[qt], p.rope_cos, p.rope_sin, qi, lane);
     bf16_t* drow = p.dq + (row0 + qi) * p.lddq + h * D;
 #pragma unroll
     for (int i = 0; i < DT; ++i)
