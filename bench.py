@@ -100,6 +100,11 @@ class Workbench:
         rt.sync()
         self._keep = (wpool, ones, bpool)
 
+    def close(self):
+        """Frees the executor and every buffer (the next workload needs the memory)."""
+        self.ex.close()
+        self.x_in, self.dy_in, self.out, self._keep, self.loop = {}, {}, [], (), None
+
     def step(self, stream=None):
         ex = self.ex
         ex.zero_grads(stream)                 # `Add.state`: accumulators start from zero
@@ -204,6 +209,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg3", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-side-runs", action="store_true",
+                    help="leave out the short extra measurements the default line carries: the "
+                         "same row with one weight-gradient product per microbatch "
+                         "(`ungrouped`) and, for the default workload, three steps each of "
+                         "cfg2 / cfg4 / cfg5 (`other_workloads`)")
     ap.add_argument("--n-mubatches", type=int, default=None,
                     help="override the workload's microbatch count (shorter runs under "
                          "rocprofv3 --pmc, which serialises every dispatch; not the headline)")
@@ -226,12 +236,6 @@ def main():
                          "eager step after the timed ones.  auto: for narrow layers (hidden < "
                          "2048: thousands of small launches per step, +3 %%), not for wide ones "
                          "(the GPU is busy 99.8 %% of an eager step)")
-    ap.add_argument("--extra-fills", type=int, default=0,
-                    help="diagnostic: after every step, clear a 6 GiB scratch buffer this many "
-                         "times (about 2 ms each of memory-bound, low-power work).  The step "
-                         "grows by less than the fills take alone: the device holds an average "
-                         "power, and what the matrix-core kernels lose to it they partly get "
-                         "back while something cheaper runs.  Not a valid headline run.")
     ap.add_argument("--kernel-table", action="store_true",
                     help="instead of the one-line result, time every kernel class of the step "
                          "with HIP events (jpp_probe_begin(\"*\")) over the timed steps and print "
@@ -279,63 +283,14 @@ def main():
     group = args.wgrad_group if args.wgrad_group is not None else default_wgrad_group(wl, two)
     if args.unfused_accumulate or two:
         group = 1
-    args.graph = args.graph == "on" or (args.graph == "auto" and wl.layer.hidden < 2048)
+    use_graph = args.graph == "on" or (args.graph == "auto" and wl.layer.hidden < 2048)
     wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two, wgrad_group=group)
     if args.kernel_table:
         print(json.dumps(kernel_table(wb, wl, args.steps, args.warmup, two, group)))
         return
 
-    # The host enqueues a step in a fraction of the time the GPU takes to run it.  It is kept at
-    # most two steps ahead (the queue never drains, so the timing is unaffected): tools that
-    # keep a record per dispatch in flight, rocprofv3 among them, do not survive a backlog of
-    # 100 000 launches.
-    ends = []
-
-    filler = rt.DeviceBuffer(6 << 30) if args.extra_fills else None
-
-    def paced_step():
-        if len(ends) >= 2:
-            ends.pop(0).sync()
-        wb.step()
-        for _ in range(args.extra_fills):
-            filler.zero()
-        ev = rt.Event()
-        ev.record()
-        ends.append(ev)
-
     cls = args.probe or measured_dominant_class(wb, wl)
-    for _ in range(args.warmup):
-        paced_step()
-    rt.sync()
-    start, stop = rt.Event(), rt.Event()
-    if args.graph:
-        stream = rt.Stream()
-        if not args.warmup:
-            wb.step(stream.ptr)               # first launches configure their kernels
-            stream.sync()
-        wb.ex.quiesce()
-        graph = rt.Graph(stream)
-        with graph:
-            wb.step(stream.ptr)
-        graph.launch()                        # one untimed replay
-        stream.sync()
-        start.record(stream.ptr)
-        for _ in range(args.steps):
-            graph.launch()
-        stop.record(stream.ptr)
-        stop.sync()
-        with rt.probe(cls) as pr:
-            wb.step()
-            rt.sync()
-    else:
-        with rt.probe(cls) as pr:
-            start.record()
-            for _ in range(args.steps):
-                paced_step()
-            stop.record()
-            stop.sync()
-    rt.sync()
-    ms = start.elapsed_ms(stop) / args.steps
+    ms, pr = timed_steps(wb, args.steps, args.warmup, use_graph, cls)
     tokens = wl.tokens_per_step
     flops = wb.step_flops()
     spec = wl.layer
@@ -349,13 +304,28 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {
             "workload": (f"{wl.name}: {spec.family} stage, rank {wl.rank} of {wl.schedule}"
-                         f"{wl.schedule_kwargs}, {self_desc(wl, wb)}"),
+                         f"{wl.schedule_kwargs}, {self_desc(wl, wb)}; every parameter and "
+                         "boundary tensor is a buffer of its own filled from windows, at "
+                         "per-tensor offsets, of one N(0, 0.02^2) pool (weights) and one "
+                         "N(0, 1) pool (activations, cotangents) of 2^26 values"),
             "tokens_per_step": tokens, "n_mubatches": wl.n_mubatches,
             "layers": wl.layers_per_stage * wb.plan.n_chunks,
+            # the schedule's own figure: forwards whose backward has not run
             "peak_live_microbatches": wb.plan.max_live,
+            # what the run holds: with weight gradients in groups, a microbatch whose weight
+            # gradients wait for its group keeps its residual slot beyond the schedule's
+            # release point (n_chunks * (wgrad_group - 1) slots more)
+            "residual_slots": wb.plan.max_live + wb.plan.n_chunks * (max(group, 1) - 1),
             "fused_wgrad_accumulate": not args.unfused_accumulate,
-            "two_streams": two, "hip_graph": bool(args.graph), "wgrad_group": group,
-            **({"extra_fills": args.extra_fills} if args.extra_fills else {}),
+            "two_streams": two, "hip_graph": bool(use_graph),
+            "wgrad_group": group,
+            "wgrad_group_meaning": ("weight gradients of this many consecutive microbatches run "
+                                    "as one product per weight: the fp32 accumulator is read "
+                                    "and written once per group and the additions inside an "
+                                    "element are reassociated (equal to the per-microbatch "
+                                    "run to fp32 rounding, not bit for bit); 1 = the "
+                                    "reference's one accumulate per microbatch"),
+            "schedule_task_fusion": not S.schedule_task_fusion_disabled(),
             "device_bytes": wb.ex.nbytes,
         },
         "algorithmic_flops_per_step": flops,
@@ -377,11 +347,93 @@ def main():
         }
     if args.after_loop:
         rec["after_loop"] = after_loop(wb, wl, args.steps)
+    wb.close()
+    del wb
+    if group > 1 and not args.no_side_runs:
+        # the same row with one weight-gradient product per microbatch (the reference's
+        # lifetimes and accumulate order), a few steps
+        rec["ungrouped"] = side_run(wl, args.workload, wgrad_group=1)
+    if not args.no_side_runs and args.workload == "cfg3" and not args.n_mubatches:
+        # the other single-GPU configurations, a few steps each, so that one run records them
+        rec["other_workloads"] = {name: side_run(workloads()[name], name)
+                                  for name in ("cfg2", "cfg4", "cfg5")}
     if not args.no_cpu_baseline:
         # a sample of 10-20 s on the host: about 1.2e13 FLOP at the ~1 TFLOP/s its BLAS reaches
         layers = int(round(1.2e13 / (3.0 * wl.layer.fwd_flops())))
         rec["cpu_baseline"] = cpu_baseline(wl, max(1, min(wl.layers_per_stage, layers)))
     print(json.dumps(rec))
+
+
+def timed_steps(wb, steps: int, warmup: int, use_graph: bool, cls: str | None):
+    """`warmup` untimed steps, then `steps` timed ones between two HIP events; returns
+    (ms per step, the probe of kernel class `cls`).
+
+    The host enqueues a step in a fraction of the time the GPU takes to run it.  It is kept at
+    most two steps ahead (the queue never drains, so the timing is unaffected): tools that
+    keep a record per dispatch in flight, rocprofv3 among them, do not survive a backlog of
+    100 000 launches."""
+    ends = []
+
+    def paced_step():
+        if len(ends) >= 2:
+            ends.pop(0).sync()
+        wb.step()
+        ev = rt.Event()
+        ev.record()
+        ends.append(ev)
+
+    for _ in range(warmup):
+        paced_step()
+    rt.sync()
+    start, stop = rt.Event(), rt.Event()
+    if use_graph:
+        stream = rt.Stream()
+        if not warmup:
+            wb.step(stream.ptr)               # first launches configure their kernels
+            stream.sync()
+        wb.ex.quiesce()
+        graph = rt.Graph(stream)
+        with graph:
+            wb.step(stream.ptr)
+        graph.launch()                        # one untimed replay
+        stream.sync()
+        start.record(stream.ptr)
+        for _ in range(steps):
+            graph.launch()
+        stop.record(stream.ptr)
+        stop.sync()
+        with rt.probe(cls or "-") as pr:
+            wb.step()
+            rt.sync()
+    else:
+        with rt.probe(cls or "-") as pr:
+            start.record()
+            for _ in range(steps):
+                paced_step()
+            stop.record()
+            stop.sync()
+    rt.sync()
+    return start.elapsed_ms(stop) / steps, pr
+
+
+def side_run(wl, name: str, wgrad_group: int | None = None, steps: int = 3, warmup: int = 1) -> dict:
+    """A short measurement of another workload (or of this one in another mode) with the
+    settings the bench would choose for it; the executor is freed afterwards."""
+    import gc
+    gc.collect()
+    two = wl.layer.hidden < 2048
+    group = 1 if two else (wgrad_group if wgrad_group is not None else default_wgrad_group(wl, two))
+    wb = Workbench(wl, fused=True, two_streams=two, wgrad_group=group)
+    ms, _ = timed_steps(wb, steps, warmup, use_graph=wl.layer.hidden < 2048, cls=None)
+    flops = wb.step_flops()
+    out = {"ms_per_step": ms, "tokens_per_s": wl.tokens_per_step / (ms * 1e-3),
+           "mfma_peak_frac": flops / (ms * 1e-3) / MFMA_BF16_PEAK, "steps": steps,
+           "wgrad_group": group, "two_streams": two, "hip_graph": wl.layer.hidden < 2048,
+           "device_bytes": wb.ex.nbytes}
+    wb.close()
+    del wb
+    gc.collect()
+    return out
 
 
 def lds_read_rates() -> dict:
