@@ -81,7 +81,10 @@ def close(got, want, rtol: float, what: str = "", max_bad_frac: float = 0.0,
     err = float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max()) if want.size else 0.0
     assert err <= rtol * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g} (rtol {rtol:g})"
     n_bad, n, worst = violations(got, want, rtol)
-    assert n_bad <= max_bad_frac * n, (
+    # (where a fraction is granted at all, one element of a tensor too small for the fraction
+    # to amount to one - a bias of 768 elements - is granted as well)
+    allowed = max(max_bad_frac * n, 1.0) if max_bad_frac > 0 else 0.0
+    assert n_bad <= allowed, (
         f"{what}: {n_bad} of {n} elements ({n_bad / max(n, 1):.3g}) outside "
         f"rtol {rtol:g} * (|want| + rms); worst at {worst:.3g} x the bound "
         f"(allowed fraction {max_bad_frac:g}){where_bad(got, want, rtol)}")

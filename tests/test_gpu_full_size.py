@@ -24,7 +24,7 @@ from jaxpp_amd.model import LayerSpec
 from jaxpp_amd.plan import make_rank_plan
 from oracle import layers as L
 
-from test_gpu_stage import close, make_params, run_on_gpu, run_on_oracle
+from test_gpu_stage import assert_close_to_truth, close, make_params, run_on_gpu, run_on_oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -185,6 +185,8 @@ def test_llama_8b_layer_matches_oracle():
     for pname, want in acc_w[0][0].items():
         got = grads[0][0][pname]
         parity.close_stage(got, want.reshape(got.shape), 2e-2, f"grad {pname}")
+    print("full-size layer: oracle in float32", flush=True)
+    assert_close_to_truth(spec, plan1, lpc, params, row, (ys, dxs, grads), (ys_w, dxs_w, acc_w))
     # the same microbatch twice (boundary tensors depend on the microbatch index, so the
     # second pass is a second run of microbatch 0 into the same accumulators)
     shape = (spec.tokens, spec.hidden)
@@ -228,6 +230,8 @@ def test_bert_large_layers_match_oracle(two_streams):
             for pname, want in acc_w[s_][li].items():
                 got = grads[s_][li][pname]
                 parity.close_stage(got, want.reshape(got.shape), 2e-2, f"grad {s_}/{li}/{pname}")
+    if two_streams:
+        assert_close_to_truth(spec, plan, lpc, params, row, (ys, dxs, grads), (ys_w, dxs_w, acc_w))
 
 
 # ---------------------------------------------------------------------------
@@ -491,3 +495,102 @@ def test_bench_row_equals_sequential_order(name, peak):
                 # sums of 32 x 4096 products in another order: a few fp32 ulps of the terms
                 parity.close(grads_grp[i][pname], v, 3e-5, f"grouped: grad {i}/{pname}")
         ex.close()
+
+
+@pytest.mark.parametrize("name", ["cfg4", "cfg5"])
+def test_deep_bench_rows_equal_sequential_order(name):
+    """The two other rows bench.py times, at their real depth in microbatches and at the full
+    layer widths, on bench's own device state and with its own weight-gradient grouping:
+    cfg4 = ZeroBubble(8) rank 1, 24 microbatches, split backward with the BWD_W tasks in the
+    table's bubble slots, Llama-70B-shaped layers; cfg5 = DualPipeV(8, 4) rank 0, 16
+    microbatches, both V-chunks on the rank, Mixtral-8x7B-shaped layers.  Two layers per stage
+    instead of ten / four (memory and time; the slot ring, the held-back weight gradients and
+    the order of tasks - what depth in microbatches exercises - do not depend on the layer
+    count).  As for cfg3 there is no oracle at this size; the scheduled row must give
+    bit-identical results to the same work in sequential order (the reference's own invariant,
+    tests/test_transformations.py:187-191): every task's output and every accumulator, the
+    latter kept on the device (a copy per parameter) and compared one parameter at a time."""
+    import dataclasses
+
+    import bench
+    from jaxpp_amd.model import workloads
+    from jaxpp_amd.types import TaskType
+    wl = dataclasses.replace(workloads()[name], layers_per_stage=2)
+    group = bench.default_wgrad_group(wl, False)
+    assert group == 2
+    print(f"bench row {name}: {wl.schedule}{wl.schedule_kwargs} rank {wl.rank}, "
+          f"{wl.n_mubatches} microbatches, weight gradients in groups of {group}", flush=True)
+    wb = bench.Workbench(wl, fused=True, two_streams=False, wgrad_group=group)
+    ex, plan = wb.ex, wb.plan
+    lib = rt.load()
+    act = wl.layer.tokens * wl.layer.hidden
+    keys = [(pt.exec_kind, pt.chunk, pt.task.mubatch_idx) for pt in plan.tasks
+            if pt.exec_kind is not TaskType.BWD_W]
+    outs = [{k: rt.DeviceBuffer(act * 2) for k in keys} for _ in range(2)]
+
+    def io_into(which):
+        def io(pt, lane=0):
+            m = pt.task.mubatch_idx
+            src = wb.x_in if pt.exec_kind is TaskType.FWD else wb.dy_in
+            return src[pt.chunk, m].ptr, outs[which][pt.exec_kind, pt.chunk, m].ptr
+        return io
+
+    def grad_ptrs():
+        for c in range(plan.n_chunks):
+            for li in range(wl.layers_per_stage):
+                for pname, rows, cols in ex.params:
+                    yield (c, li, pname), ex._ptr(lib.jpp_stage_grad_ptr, c, li, pname), rows * cols * 4
+
+    # the schedule's order, one task at a time so that the peak of live slots is seen
+    ex.zero_grads()
+    live_peak, io = 0, io_into(0)
+    for pt in plan.tasks:
+        if pt.exec_kind is TaskType.BWD_W:
+            ex.run_task(pt.exec_kind, pt.chunk, pt.task.mubatch_idx)
+        else:
+            ex.run_task(pt.exec_kind, pt.chunk, pt.task.mubatch_idx, *io(pt))
+        live_peak = max(live_peak, ex.live_slots())
+    ex.join()
+    rt.sync()
+    assert ex.live_slots() == 0
+    assert plan.max_live <= live_peak <= plan.max_live + plan.n_chunks * (group - 1), (
+        f"live slots peaked at {live_peak}; the plan says {plan.max_live}, a group holds "
+        f"{plan.n_chunks * (group - 1)} more")
+    print(f"  live slots peaked at {live_peak} (plan {plan.max_live})", flush=True)
+    kept = {}
+    for key, ptr, nbytes in grad_ptrs():
+        kept[key] = rt.DeviceBuffer(nbytes)
+        rt.check(lib.jpp_memcpy_d2d_async(kept[key].ptr, ptr, nbytes, None))
+    rt.sync()
+
+    # sequential order: microbatch by microbatch, forward then backward of every chunk
+    ex.zero_grads()
+    io = io_into(1)
+    bwd_kinds = {}
+    for pt in plan.tasks:
+        if pt.exec_kind is not TaskType.FWD:
+            bwd_kinds.setdefault((pt.chunk, pt.task.mubatch_idx), []).append(pt)
+    for m in range(wl.n_mubatches):
+        for c in range(plan.n_chunks):
+            ex.run_task(TaskType.FWD, c, m, wb.x_in[c, m].ptr, outs[1][TaskType.FWD, c, m].ptr)
+        for c in reversed(range(plan.n_chunks)):
+            for pt in bwd_kinds[c, m]:
+                if pt.exec_kind is TaskType.BWD_W:
+                    ex.run_task(pt.exec_kind, c, m)
+                else:
+                    ex.run_task(pt.exec_kind, c, m, *io(pt))
+    ex.join()
+    rt.sync()
+    assert ex.live_slots() == 0
+
+    for k in keys:
+        a, b = outs[0][k].download(np.uint16, (act,)), outs[1][k].download(np.uint16, (act,))
+        assert b.any(), f"output of {k} was never written"
+        np.testing.assert_array_equal(a, b, err_msg=f"output of {k}")
+    for key, ptr, nbytes in grad_ptrs():
+        a = kept[key].download(np.float32, (nbytes // 4,))
+        b = rt.download_ptr(ptr, np.float32, (nbytes // 4,))
+        assert np.isfinite(b).all() and (b.any() or key[2].startswith("b")), f"accumulator {key}"
+        np.testing.assert_array_equal(a, b, err_msg=f"accumulator {key}")
+        kept[key].free()
+    wb.close()

@@ -7,12 +7,16 @@ target, as in the README's autoencoder step, a pre-LN residual stack is ill-cond
 cotangent 2 (pred - x) / N is the difference of two nearly equal bf16 tensors, and a one-ulp
 difference in pred is a few per cent of it.  That is a property of that loss, not of the
 executor, and the fixed cases of test_gpu_api.py cover that step.)  A whole pipeline of up to
-eight layers compounds the rounding of every layer behind it, so the elementwise bound is
-granted 1e-2 of a tensor's elements here, ten times the stage-level figure, and the worst of
-them 8 x the bound instead of 4 x (seen: 4.1 x on one QKV weight gradient of a six-layer BERT
-pipeline in four hundred further draws); the sweep is for dataflow errors - a wrong slot, a
-microbatch counted twice, a stage out of order - which put whole tensors off by their own
-magnitude and fail the bound on the largest error."""
+eight layers compounds the rounding of every layer behind it: pipelines of more than four
+layers are granted 4e-3 of a tensor's elements outside the elementwise bound instead of the
+stage-level 1e-3 (the worst of them 4 x the bound, as everywhere).  That is what the oracle's own
+arithmetic does at this depth: evaluated twice on the sweep's six-layer BERT pipeline, with
+float32 and with float64 accumulation, it disagrees with itself on 2.5e-3 of the first layer's
+QKV weight gradient, by up to 2.5 x (tests/test_oracle_stage.py,
+test_bf16_sensitivity_of_a_six_layer_pipeline).  How good the bf16 results are is held
+separately: no farther from the float32 computation than the bf16 oracle's own
+(parity.close_to_truth).  The sweep is for dataflow errors - a wrong slot, a microbatch counted
+twice, a stage out of order - which put whole tensors off by their own magnitude."""
 import os
 from functools import partial
 
@@ -70,6 +74,11 @@ def draw(seed):
         return spec, sched, p, n_mb, per
 
 
+# fraction of a tensor's elements granted outside the elementwise bound: the stage-level
+# figure, and what pipelines of more than four layers get (see the module's text)
+DEEP_BAD_FRAC = 4e-3
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_random_train_step_matches_sequential_loop(seed):
     rt.require_gpu()
@@ -101,14 +110,26 @@ def test_random_train_step_matches_sequential_loop(seed):
     want_pred = []
     want_loss, want_acc = O.treduce_sequential(cfg, stages, list(batch), L.Numerics.bf16(),
                                                targets=list(targets), preds=want_pred)
+    # the unrounded computation (float32 on the same bf16-valued inputs): the device may be no
+    # farther from it than the bf16 oracle is (expert layers aside: the float32 run may route
+    # a token to another expert)
+    BAD_FRAC = DEEP_BAD_FRAC if n_stages * per > 4 else parity.STAGE_BAD_FRAC
+    EXCESS = parity.MAX_EXCESS
+    truth_pred = []
+    truth = None if spec.family == "mixtral" else O.treduce_sequential(
+        cfg, stages, list(batch), L.Numerics.f32(), targets=list(targets), preds=truth_pred)
     parity.close(np.asarray(losses, np.float32), np.asarray(want_loss), 2e-2, "losses")
     assert pred.shape == batch.shape
     for m in range(n_mb):
-        parity.close(np.asarray(pred[m], np.float32), want_pred[m], 2e-2,
-                     f"prediction of microbatch {m}", 1e-2, 8.0)
+        got = np.asarray(pred[m], np.float32)
+        parity.close(got, want_pred[m], 2e-2, f"prediction of microbatch {m}", BAD_FRAC, EXCESS)
+        if truth:
+            parity.close_to_truth(got, want_pred[m], truth_pred[m], f"prediction of microbatch {m}")
     for s in range(n_stages):
         for li in range(per):
             for k, v in want_acc[s][li].items():
                 got = np.asarray(grad["layers"][s * per + li][k], np.float32)
-                parity.close(got, v.reshape(got.shape), 2e-2, f"grad {s}/{li}/{k}", 1e-2, 8.0)
+                parity.close(got, v.reshape(got.shape), 2e-2, f"grad {s}/{li}/{k}", BAD_FRAC, EXCESS)
+                if truth:
+                    parity.close_to_truth(got, v, truth[1][s][li][k], f"grad {s}/{li}/{k}")
     train_step.close()

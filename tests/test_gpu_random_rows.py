@@ -133,6 +133,8 @@ def test_random_row_of_wide_layers_matches_oracle(seed):
     for k in dxs_w:
         parity.close_stage(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
     T.assert_grads_match(spec, plan, lpc, grads, acc_w, WIDE_BAD_FRAC)
+    if seed % 3 == 0:      # (the float32 oracle run doubles a case's host time: every third)
+        T.assert_close_to_truth(spec, plan, lpc, params, row, (ys, dxs, grads), (ys_w, dxs_w, acc_w))
 
 
 @pytest.mark.parametrize("seed", range(96))
@@ -178,3 +180,4 @@ def test_random_row_matches_oracle(seed):
     for k in dxs_w:
         parity.close_stage(dxs[k], dxs_w[k], 2e-2, f"dx{k}")
     T.assert_grads_match(spec, plan, lpc, grads, acc_w)
+    T.assert_close_to_truth(spec, plan, lpc, params, row, (ys, dxs, grads), (ys_w, dxs_w, acc_w))
