@@ -215,8 +215,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
   // The row term delta = sum_d dO * O of this wave's 32 rows: a lane holds half of its row of
   // dO already (the chunks the MFMA fragment gives it) and reads the same half of O; the other
   // half is with lane ^ 32.  Written out for the dK/dV kernel, which runs behind this one, in
-  // the form that kernel consumes: per row the pair {delta times the softmax scale, the
-  // log-sum-exp in the exp2 domain}.
+  // the form that kernel consumes: per 64 rows, -delta[64] and then the log-sum-exp[64] in
+  // the exp2 domain.
   float dlt = 0.f;
   {
     const bf16_t* obase = p.o + (row0 + q0) * p.ldo + h * D;
@@ -230,8 +230,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
       for (int e = 0; e < 8; ++e) dlt = fmaf(of[e], gf[e], dlt);
     }
     dlt += __shfl_xor(dlt, 32);
-    dlt *= p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
-    if (lane < 32) *(float2*)(p.delta + 2 * stat) = make_float2(dlt, lse2);
+    if (lane < 32) {
+      float* st = p.delta + 2 * (stat & ~63L) + (stat & 63);  // (seq is a multiple of 64)
+      st[0] = -dlt;
+      st[64] = lse2;
+    }
   }
   const float sc = p.scale * kLog2e;
   settle(qf);
@@ -304,7 +307,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float pr = fast_exp2(fmaf(s[r], sc, -lse2));  // exp2(-inf) = 0 where masked
-          s[r] = pr * fmaf(dp[r], p.scale, -dlt);
+          s[r] = pr * (dp[r] - dlt);  // (the softmax scale is applied to dQ at the end)
         }
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
@@ -319,6 +322,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
     __syncthreads();
   }
 
+#pragma unroll
+  for (int i = 0; i < DT; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dqacc[i][r] *= p.scale;
   if (p.rope_cos) rope_back<D, DT>(dqacc, p.rope_cos, p.rope_sin, qi, lane);
   bf16_t* drow = p.dq + (row0 + qi) * p.lddq + h * D;
 #pragma unroll
@@ -379,7 +386,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
   const uint32_t lds0 = lds_address(smem);
 
   // Q / dO tiles go HBM -> LDS directly; the 64 lse and 64 delta values of a
-  // block (as the dQ kernel left them: exp2 domain, delta scaled) travel through
+  // block (as the dQ kernel left them: exp2 domain, -delta) travel through
   // one register per thread and are parked in LDS at the end of the previous
   // iteration, so waiting for them never stalls the tiles.
   float rstat = 0.f;
@@ -389,7 +396,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
     const long stat = ((long)b * p.n_heads + hh) * p.seq + q0;
     // one unconditional load, consumed only in park(): nothing in between waits for it
     const int st = tid & 127;
-    rstat = p.delta[2 * (stat + (st & 63)) + (st < 64 ? 1 : 0)];
+    rstat = p.delta[2 * stat + (st ^ 64)];  // lse[64], then -delta[64]
     const uint32_t dst = lds0 + stage * STAGE;
     dma_tile<D>(p.q + (row0 + q0) * p.ldq + hh * D, offq, dst, wave);
     dma_tile<D>(p.d_o + (row0 + q0) * p.lddo + hh * D, offdo, dst + TILE, wave);
@@ -449,7 +456,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
               float pr = fast_exp2(fmaf(s[u][r], sc, -ls[e]));
               if (diag && ki > q0 + ql + e) pr = 0.f;
               s[u][r] = pr;
-              dp[u][r] = pr * fmaf(dp[u][r], p.scale, -dl[e]);
+              dp[u][r] = pr * (dp[u][r] + dl[e]);  // (the softmax scale is applied to dK at the end)
             }
           }
         }
@@ -483,8 +490,9 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const int d = i * 32 + g * 8 + (lane >> 5) * 4;
-      *(uint2*)(dkrow + d) = make_uint2(pack_bf16x2(dkacc[i][4 * g], dkacc[i][4 * g + 1]),
-                                        pack_bf16x2(dkacc[i][4 * g + 2], dkacc[i][4 * g + 3]));
+      *(uint2*)(dkrow + d) =
+          make_uint2(pack_bf16x2(dkacc[i][4 * g] * p.scale, dkacc[i][4 * g + 1] * p.scale),
+                     pack_bf16x2(dkacc[i][4 * g + 2] * p.scale, dkacc[i][4 * g + 3] * p.scale));
       *(uint2*)(dvrow + d) = make_uint2(pack_bf16x2(dvacc[i][4 * g], dvacc[i][4 * g + 1]),
                                         pack_bf16x2(dvacc[i][4 * g + 2], dvacc[i][4 * g + 3]));
     }

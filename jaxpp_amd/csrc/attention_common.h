@@ -88,12 +88,16 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
                  : "+" ACC(acc) : A(a), B(b) : "memory");                                  \
   }
 JPP_MFMA(mfma_avv, "a", "v", "v")
+JPP_MFMA(mfma_vaa, "v", "a", "a")
 JPP_MFMA(mfma_vva, "v", "v", "a")
 JPP_MFMA(mfma_vvv, "v", "v", "v")
 #undef JPP_MFMA
 // the first product of a chain: the accumulator starts from zero
 __device__ __forceinline__ void mfma_vva_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b) : "memory");
+}
+__device__ __forceinline__ void mfma_vaa_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "a"(a), "a"(b) : "memory");
 }
 // two floats -> one register of two bf16 (round to nearest even), one instruction
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {

@@ -18,13 +18,20 @@ namespace {
 // Under the mask a key block sees only the queries behind it, so a workgroup takes block x
 // and then block n-1-x: every workgroup of the launch carries the same amount of work.
 //
-// Items travel HBM -> LDS through a ring of four slots (Q tile, dO tile, the rows' scaled
-// delta and log-sum-exp), fetched three items ahead.  Per item a wave runs
-//   1. S = Q K^T, dP = dO V^T                         (16 MFMAs at head 128)
-//   2. P = exp2(S - lse), dS = P (dP - delta)          (elementwise)
+// Items travel HBM -> LDS through a ring of four slots (Q tile, dO tile, the rows' -delta
+// and log-sum-exp), fetched three items ahead.  Per item a wave runs
+//   1. S = Q K^T, dP - delta = dO V^T - delta          (16 MFMAs at head 128; the accumulator
+//                                                       of the second starts from -delta, read
+//                                                       from LDS straight into its registers)
+//   2. P = exp2(S - lse), dS = P (dP - delta)          (elementwise; the softmax scale that
+//                                                       belongs on dS is applied to dK at the end)
 //   3. dV += P^T dO, dK += dS^T Q                      (16 MFMAs)
 // and one trip of the loop issues 3 of the item before, then 1 of the item after with 2 of
 // the item in the middle between its MFMAs; two sets of score registers alternate.
+//
+// With one wave per SIMD the kernel is bound by the number of instructions a trip issues, so
+// the LDS addresses of a trip are a handful of per-lane constants plus the slot's offset, and
+// every read is one of those registers plus an immediate.
 // ---------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
@@ -48,16 +55,33 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
   Tile64::Offsets offq, offdo;
   Tile64::offsets(offq, p.ldq, wave, lane);
   Tile64::offsets(offdo, p.lddo, wave, lane);
-  // one 16-byte load per lane brings an item's row statistics, 64 {scaled delta, lse} pairs
-  // as the dQ kernel left them; the upper half of the wave repeats the lower one into the
-  // unused part of the slot
+  // one 16-byte load per lane brings an item's row statistics, -delta[64] then lse[64] as the
+  // dQ kernel left them; the upper half of the wave repeats the lower one into the unused
+  // part of the slot
   const uint32_t offst = (uint32_t)((lane & 31) * 16);
-  const int ql0 = qh * 32 + (lane >> 5) * 4;  // first of this lane's rows within a 64-query block
+
+  // Per-lane parts of the LDS addresses, in bytes from the start of a slot.
+  // Row fragment (tile t, step ks) of this wave's 32 queries:
+  //   t TILE + (ks >> 2) 8192 + (a_row ^ (ks & 3) << 5)
+  // (the chunk 2 (ks & 3) + lane / 32 enters the swizzle by XOR, and 2 (ks & 3) has bit 0 clear)
+  const uint32_t a_row = (uint32_t)slab_off(qh * 32 + (lane & 31), lane >> 5);
+  // Transposed fragment (tile t, columns 32 ii.., steps 2 qh + h2, half hi) - slab_frag_tr()
+  // with its address split into the lane's part and the rest:
+  //   t TILE + (ii >> 1) 8192 + h2 2048 + hi 1024 + (a_tr ^ ((ii & 1) ^ hi) << 6)
+  uint32_t a_tr;
+  {
+    const int g = lane >> 4, s = lane & 15;
+    const int k0 = qh * 32 + ((g >> 1) << 2) + (s >> 2);
+    const int c0 = ((g & 1) << 1) + ((s & 3) >> 1);
+    a_tr = (uint32_t)(((s & 1) << 3) + slab_off(k0, c0));
+  }
+  // Row statistics: the lane's rows 8 g + 4 (lane / 32) + 0..3 of its query half, four floats
+  // per read:  2 TILE + [256 for lse] + 32 g + a_st
+  const uint32_t a_st = (uint32_t)(2 * TILE + (qh * 32 + (lane >> 5) * 4) * 4);
 
   for (int seg = 0; seg < 2; ++seg) {
     const int kb = seg == 0 ? w.x : nkb - 1 - w.x;
     const int k0 = kb * 64 + ksb * 32;
-    const int ki = k0 + (lane & 31);
 
     bf16x8 kf[KS], vf[KS];
     {
@@ -123,12 +147,19 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
         dofr[ks] = slabs_frag<D>(slot + TILE, qh * 32, ks, lane);
       }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int g = 0; g < 4; ++g) {
+        const float4 nd = *(const float4*)(slot + a_st + 32 * g);
+        dp[4 * g] = nd.x; dp[4 * g + 1] = nd.y; dp[4 * g + 2] = nd.z; dp[4 * g + 3] = nd.w;
+      }
+      // (the same statements as in the trips: compiler-chosen MFMAs would leave their results
+      // in the accumulation registers, and the loop would copy its scores there and back)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[ks], kf[ks], s, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dofr[ks], vf[ks], dp, 0, 0, 0);
+        if (ks == 0) mfma_vaa_first(s, qfr[0], kf[0]);
+        else mfma_vaa(s, qfr[ks], kf[ks]);
+        mfma_vaa(dp, dofr[ks], vf[ks]);
       }
+      asm volatile("s_nop 15" : "+v"(s), "+v"(dp));
     };
     // Items of the key block's own query block are masked: the query half behind the keys
     // sees all of them, the half in front none, the one on the diagonal what lies at or
@@ -165,75 +196,113 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     };
 
     // One trip: item i is in the middle (its scores in s_c / dp_c), i - 1 before, i + 1 after.
-    // A wave issues in order: an MFMA that finds the matrix core busy holds back whatever
-    // follows it, so the elementwise work and the LDS reads have to sit between the MFMAs in
-    // the instruction stream.  The MFMAs of a trip are volatile asm statements (they keep
-    // their order, and LDS reads do not cross them); the elementwise work is tied to its place
-    // by empty asm statements on its inputs and results.
+    // A wave issues in order, and an MFMA that finds the matrix core busy (32 cycles per
+    // MFMA) holds back whatever follows it.  So the MFMAs go out one at a time, each followed
+    // by its share of the trip's other instructions - about as much as issues in those 32
+    // cycles - and never two in a row, where the second would hold up the wave while nothing
+    // else issues.  MFMAs and elementwise instructions are volatile asm statements (they
+    // keep their order, and LDS reads do not cross the MFMAs).
     auto trip = [&](auto tail, int i, f32x16& s_c, f32x16& dp_c, f32x16& s_n, f32x16& dp_n) __attribute__((always_inline)) {
       constexpr bool TAIL = decltype(tail)::value;
-      const uint8_t* sl_c = smem + (i & 3) * SLOT;
-      const uint8_t* sl_n = smem + ((i + 1) & 3) * SLOT;
-      // Q / dO fragments of item i + 1: the first half now, the second while the first is used
-      bf16x8 qfr[KS], dofr[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS / 2; ++ks) {
-        qfr[ks] = slabs_frag<D>(sl_n, qh * 32, ks, lane);
-        dofr[ks] = slabs_frag<D>(sl_n + TILE, qh * 32, ks, lane);
-      }
-      // row statistics of item i: {scaled delta, lse} pairs, two rows per 16-byte read
-      const float* st = (const float*)(sl_c + 2 * TILE) + 2 * ql0;
-      auto stats = [&](int r) __attribute__((always_inline)) { return *(const float4*)(st + 2 * ((r >> 2) * 8 + (r & 3))); };
-      float4 st_q[3] = {stats(0), stats(2), stats(4)};  // read two pairs of rows ahead of their use
-      // dV / dK products of item i - 1 from registers (the reads above arrive under them);
-      // behind each pair, the transposed fragments of item i take over its registers
-#pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2)
-#pragma unroll
-        for (int ii = 0; ii < DT; ++ii) {
-          mfma_avv(dvacc[ii], dotr[h2][ii], pf[h2]);
-          mfma_avv(dkacc[ii], qtr[h2][ii], dsf[h2]);
-          dotr[h2][ii] = slab_frag_tr(sl_c + TILE, 64, ii * 32, 2 * qh + h2, lane);
-          qtr[h2][ii] = slab_frag_tr(sl_c, 64, ii * 32, 2 * qh + h2, lane);
-          // item i + 3 into the slot item i - 1 has left (its scalar address work runs under
-          // the MFMAs)
-          // (a load or two behind every pair of MFMAs rather than all at once)
-          {
-            constexpr int GROUPS = 2 * DT, EACH = (NLOAD + GROUPS - 1) / GROUPS;
-            const int g = h2 * DT + ii;
-#pragma unroll
-            for (int j = g * EACH; j < (g + 1) * EACH && j < NLOAD; ++j) fetch_part((i + 3) & 3, j);
-          }
+      constexpr int NB = 4 * DT;    // MFMAs of step 3
+      constexpr int NR = KS + 8;    // reads for steps 1 and 2: KS/2 Q and KS/2 dO row fragments, 4 x -delta, 4 x lse
+      constexpr int EPG = 16 / KS;  // elements of step 2 per MFMA pair of step 1
+      uint32_t b_row[4], b_tr[2], b_stc, b_stn;  // this trip's address registers
+      bf16x8 qfr[KS], dofr[KS];     // Q / dO fragments of item i + 1
+      float4 lse_r[4];              // lse of item i's rows
+      auto row_frag = [&](int t, int ks) __attribute__((always_inline)) {
+        return *(const bf16x8*)(smem + b_row[ks & 3] + (t * TILE + (ks >> 2) * 8192));
+      };
+      auto tr_frag = [&](int t, int ii, int h2) __attribute__((always_inline)) {
+        typedef __attribute__((address_space(3))) s16x4* lds_s16x4;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)JPP_LDS_PTR(
+            smem + b_tr[ii & 1] + (t * TILE + (ii >> 1) * 8192 + h2 * 2048)));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)JPP_LDS_PTR(
+            smem + b_tr[(ii & 1) ^ 1] + (t * TILE + (ii >> 1) * 8192 + h2 * 2048 + 1024)));
+        const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, v);
+      };
+      auto early_read = [&](int n) __attribute__((always_inline)) {
+        if (n < KS) {  // first half of the row fragments (the second follows while the first is used)
+          if (n & 1) dofr[n >> 1] = row_frag(1, n >> 1);
+          else qfr[n >> 1] = row_frag(0, n >> 1);
+        } else if (n < KS + 4) {  // -delta of item i + 1's rows: where its dP products start from
+          const int g = n - KS;
+          const float4 nd = *(const float4*)(smem + b_stn + 32 * g);
+          dp_n[4 * g] = nd.x; dp_n[4 * g + 1] = nd.y; dp_n[4 * g + 2] = nd.z; dp_n[4 * g + 3] = nd.w;
+        } else {
+          const int g = n - KS - 4;
+          lse_r[g] = *(const float4*)(smem + b_stc + (256 + 32 * g));
         }
-      // S and dP of item i + 1, two MFMAs at a time, with P and dS of EPG elements of item i
-      // behind each pair
-      constexpr int EPG = 16 / KS;
+      };
+      // dV / dK products of item i - 1 from registers; behind each, the transposed fragments
+      // of item i take over its operand's registers, and a share of: the reads for steps 1
+      // and 2, the loads of item i + 3 into the slot item i - 1 has left
+#pragma unroll
+      for (int m = 0; m < NB; ++m) {
+        const int h2 = m / (2 * DT), ii = (m >> 1) % DT;
+        if (m & 1) mfma_avv(dkacc[ii], qtr[h2][ii], dsf[h2]);
+        else mfma_avv(dvacc[ii], dotr[h2][ii], pf[h2]);
+        if (m == 0) {
+          // (slot offsets are multiples of 1024: adding them commutes with the XORs; the
+          // offsets pass through an asm statement so that this work stays behind the MFMA)
+          uint32_t o_c = (uint32_t)(i & 3) * SLOT, o_n = (uint32_t)((i + 1) & 3) * SLOT;
+          asm volatile("" : "+s"(o_c), "+s"(o_n));
+          b_stc = a_st + o_c;
+          b_stn = a_st + o_n;
+          b_row[0] = a_row + o_n;
+#pragma unroll
+          for (int j = 1; j < 4; ++j) b_row[j] = b_row[0] ^ (j << 5);
+          b_tr[0] = a_tr + o_c;
+          b_tr[1] = b_tr[0] ^ 64;
+          asm volatile("" : "+v"(b_row[0]), "+v"(b_row[1]), "+v"(b_row[2]), "+v"(b_row[3]),
+                            "+v"(b_tr[0]), "+v"(b_tr[1]), "+v"(b_stc), "+v"(b_stn));
+        }
+        if (m & 1) qtr[h2][ii] = tr_frag(0, ii, h2);
+        else dotr[h2][ii] = tr_frag(1, ii, h2);
+#pragma unroll
+        for (int n = m * NR / NB; n < (m + 1) * NR / NB; ++n) early_read(n);
+#pragma unroll
+        for (int j = m * NLOAD / NB; j < (m + 1) * NLOAD / NB; ++j) fetch_part((i + 3) & 3, j);
+      }
+      // S and dP of item i + 1, with P and dS of EPG elements of item i behind each pair:
+      // behind the first MFMA the exponentials (and the arguments of the next pair's), behind
+      // the second the products and the packing to bf16.  No instruction reads the result of
+      // the one before it.
+      auto lse_of = [&](int r) __attribute__((always_inline)) {
+        const float4 l4 = lse_r[r >> 2];
+        return (r & 3) == 0 ? l4.x : (r & 3) == 1 ? l4.y : (r & 3) == 2 ? l4.z : l4.w;
+      };
+      float t[EPG], tn[EPG], pe[EPG], de[EPG];
       uint32_t pw[8], dw[8];  // P and dS as bf16 pairs
+#define JPP_EXP_ARGS(KS_, DST)                                                              \
+  _Pragma("unroll") for (int e = 0; e < EPG; ++e) {                                         \
+    const float l = lse_of((KS_) * EPG + e);                                                \
+    asm volatile("v_fma_f32 %0, %1, %2, -%3"                                                \
+                 : "=v"(DST[e]) : "v"(s_c[(KS_) * EPG + e]), "s"(sc), "v"(l));              \
+  }
+      JPP_EXP_ARGS(0, t)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        if (ks == 0) {
-          mfma_vva_first(s_n, qfr[0], kf[0]);
-          mfma_vva_first(dp_n, dofr[0], vf[0]);
-        } else {
-          mfma_vva(s_n, qfr[ks], kf[ks]);
-          mfma_vva(dp_n, dofr[ks], vf[ks]);
-        }
-        if (ks < KS / 2) {
-          qfr[ks + KS / 2] = slabs_frag<D>(sl_n, qh * 32, ks + KS / 2, lane);
-          dofr[ks + KS / 2] = slabs_frag<D>(sl_n + TILE, qh * 32, ks + KS / 2, lane);
-        }
+        if (ks == 0) mfma_vaa_first(s_n, qfr[0], kf[0]);
+        else mfma_vaa(s_n, qfr[ks], kf[ks]);
 #pragma unroll
-        for (int r = ks * EPG; r < ks * EPG + EPG; r += 2) {
-          const float4 x = st_q[(r >> 1) % 3];
-          if (r + 6 < 16) st_q[(r >> 1) % 3] = stats(r + 6);
-          float s0 = s_c[r], s1 = s_c[r + 1], g0 = dp_c[r], g1 = dp_c[r + 1];
-          asm volatile("" : "+v"(s0), "+v"(s1), "+v"(g0), "+v"(g1));
-          const float p0 = fast_exp2(fmaf(s0, sc, -x.y));  // exp2(-inf) = 0 where masked
-          const float p1 = fast_exp2(fmaf(s1, sc, -x.w));
-          pw[r >> 1] = pack2(p0, p1);
-          dw[r >> 1] = pack2(p0 * fmaf(g0, p.scale, -x.x), p1 * fmaf(g1, p.scale, -x.z));
-          asm volatile("" : "+v"(pw[r >> 1]), "+v"(dw[r >> 1]));
+        for (int e = 0; e < EPG; ++e)  // exp2(-inf) = 0 where masked
+          asm volatile("v_exp_f32 %0, %1" : "=v"(pe[e]) : "v"(t[e]));
+        if (ks + 1 < KS) { JPP_EXP_ARGS(ks + 1, tn) }
+        if (ks < KS / 2) qfr[ks + KS / 2] = row_frag(0, ks + KS / 2);
+        mfma_vaa(dp_n, dofr[ks], vf[ks]);
+#pragma unroll
+        for (int e = 0; e < EPG; ++e)
+          asm volatile("v_mul_f32 %0, %1, %2" : "=v"(de[e]) : "v"(pe[e]), "v"(dp_c[ks * EPG + e]));
+#pragma unroll
+        for (int e = 0; e < EPG; e += 2) {
+          asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(pw[(ks * EPG + e) >> 1]) : "v"(pe[e]), "v"(pe[e + 1]));
+          asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dw[(ks * EPG + e) >> 1]) : "v"(de[e]), "v"(de[e + 1]));
         }
+        if (ks < KS / 2) dofr[ks + KS / 2] = row_frag(1, ks + KS / 2);
+#pragma unroll
+        for (int e = 0; e < EPG; ++e) t[e] = tn[e];
       }
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
@@ -245,9 +314,10 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
       }
       // The compiler does not know that the asm statements above are MFMAs, whose results
       // take 11 issue slots to land: whatever it does with the new scores (copies included)
-      // has to wait behind this statement, which the elementwise work of the last MFMA pair
-      // (ten instructions and more, tied in front of it) and four idle slots keep clear.
-      asm volatile("s_nop 3" : "+v"(s_n), "+v"(dp_n));
+      // has to wait behind this statement, which the elementwise work behind the last MFMA
+      // (four instructions or more) and eight idle slots keep clear.
+#undef JPP_EXP_ARGS
+      asm volatile("s_nop 7" : "+v"(s_n), "+v"(dp_n));
       if constexpr (TAIL) mask(s_n, i + 1);
       lds_wait_all();       // this wave has read all it needs of item i's slot ...
       dma_wait<NLOAD>();    // ... and its share of item i + 2 has landed (i + 3 may be on its way)
@@ -275,9 +345,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     dma_wait_all();  // the cursor's repeated fetches of the last item
     __syncthreads();
 
+    // (what follows is computed from a lane index the compiler cannot trace back: addresses
+    // worked out ahead of the loop would sit in registers through all of it)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
     // the upper query half hands its partial sums to the lower one through LDS:
     // [ksb][register][lane] floats
-    float* xch = (float*)smem + ksb * (2 * DT * 16 * 64) + lane;
+    float* xch = (float*)smem + ksb * (2 * DT * 16 * 64) + lane_e;
     if (qh == 1) {
 #pragma unroll
       for (int i = 0; i < DT; ++i)
@@ -289,21 +363,22 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     }
     __syncthreads();
     if (qh == 0) {
+      const int ki = k0 + (lane_e & 31);
       bf16_t* dkrow = p.dk + (row0 + ki) * p.lddk + hk * D;
       bf16_t* dvrow = p.dv + (row0 + ki) * p.lddv + hk * D;
 #pragma unroll
       for (int i = 0; i < DT; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          dkacc[i][r] += xch[(i * 16 + r) * 64];
+          dkacc[i][r] = (dkacc[i][r] + xch[(i * 16 + r) * 64]) * p.scale;
           dvacc[i][r] += xch[((DT + i) * 16 + r) * 64];
         }
-      if (p.rope_cos) rope_back<D, DT>(dkacc, p.rope_cos, p.rope_sin, ki, lane);
+      if (p.rope_cos) rope_back<D, DT>(dkacc, p.rope_cos, p.rope_sin, ki, lane_e);
 #pragma unroll
       for (int i = 0; i < DT; ++i) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const int d = i * 32 + g * 8 + (lane >> 5) * 4;
+          const int d = i * 32 + g * 8 + (lane_e >> 5) * 4;
           *(uint2*)(dkrow + d) = make_uint2(pack_bf16x2(dkacc[i][4 * g], dkacc[i][4 * g + 1]),
                                             pack_bf16x2(dkacc[i][4 * g + 2], dkacc[i][4 * g + 3]));
           *(uint2*)(dvrow + d) = make_uint2(pack_bf16x2(dvacc[i][4 * g], dvacc[i][4 * g + 1]),

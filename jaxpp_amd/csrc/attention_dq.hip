@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   fetch(2);
 
   // This wave's Q and dO as MFMA operands (accumulation registers), and per query tile the
-  // row's log-sum-exp (exp2 domain) and delta (times the softmax scale); delta = sum_d dO * O:
+  // row's log-sum-exp (exp2 domain) and delta = sum_d dO * O:
   // a lane holds half of its row of dO (the chunks the fragments give it) and reads the same
   // half of O, the other half is with lane ^ 32.  All loads are issued before the first of
   // them is waited for.
@@ -113,9 +113,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
         for (int e = 0; e < 8; ++e) acc = fmaf(of[e], gf[e], acc);
       }
       acc += __shfl_xor(acc, 32);
-      dlt[qt] = acc * p.scale;  // scale (dP - delta) = fma(dP, scale, -scale delta)
-      // for the dK/dV kernel, in the form it consumes: {scaled delta, lse} per row
-      if (lane < 32) *(float2*)(p.delta + 2 * stat) = make_float2(dlt[qt], lse2[qt]);
+      dlt[qt] = acc;
+      // for the dK/dV kernel, in the form it consumes: per 64 rows, -delta[64] then lse[64]
+      if (lane < 32) {
+        float* st = p.delta + 2 * (stat & ~63L) + (stat & 63);  // (seq is a multiple of 64)
+        st[0] = -acc;
+        st[64] = lse2[qt];
+      }
     }
   } else {
 #pragma unroll
@@ -213,7 +217,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
         asm volatile("" : "+v"(s0), "+v"(s1), "+v"(g0), "+v"(g1));
         const float p0 = fast_exp2(fmaf(s0, sc, -lse2[QC]));  // exp2(-inf) = 0 where masked
         const float p1 = fast_exp2(fmaf(s1, sc, -lse2[QC]));
-        dw[r >> 1] = pack2(p0 * fmaf(g0, p.scale, -dlt[QC]), p1 * fmaf(g1, p.scale, -dlt[QC]));
+        dw[r >> 1] = pack2(p0 * (g0 - dlt[QC]), p1 * (g1 - dlt[QC]));
         asm volatile("" : "+v"(dw[r >> 1]));
       }
     }
@@ -325,6 +329,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
     for (int i = 0; i < DT; ++i) asm volatile("s_nop 15" : "+a"(dqacc[qt][i]));
+  // the softmax scale that belongs on dS
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dqacc[qt][i][r] *= p.scale;
   if (p.rope_cos) {
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt)

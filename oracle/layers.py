@@ -242,7 +242,9 @@ def attention_fwd(q, k, v, causal, acc=np.float32, rt=identity):
 
 def attention_bwd(q, k, v, o, do, lse, causal, acc=np.float32, rt=identity):
     """``rt`` rounds the recomputed probabilities and the score cotangents where
-    they become operands of the three gradient products."""
+    they become operands of the three gradient products; the softmax scale that
+    belongs on the score cotangents is applied to the finished dq and dk (a
+    blocked attention backward carries it out of the inner loop this way)."""
     B, S, Hq, d = q.shape
     Hkv = k.shape[2]
     grp = Hq // Hkv
@@ -259,10 +261,10 @@ def attention_bwd(q, k, v, o, do, lse, causal, acc=np.float32, rt=identity):
     dv = np.matmul(rt(p).astype(acc).transpose(0, 1, 3, 2), doa)
     dp = np.matmul(doa, va.transpose(0, 1, 3, 2))
     delta = (doa * oa).sum(-1, keepdims=True)
-    ds = rt(p * (dp - delta) * scale).astype(acc)
-    dq = np.matmul(ds, ka)
+    ds = rt(p * (dp - delta)).astype(acc)
+    dq = np.matmul(ds, ka) * acc(scale)
     dk = np.matmul(ds.transpose(0, 1, 3, 2), qa)
-    dk = dk.reshape(B, Hkv, grp, S, d).sum(2)
+    dk = dk.reshape(B, Hkv, grp, S, d).sum(2) * acc(scale)
     dv = dv.reshape(B, Hkv, grp, S, d).sum(2)
     return (dq.transpose(0, 2, 1, 3), dk.transpose(0, 2, 1, 3), dv.transpose(0, 2, 1, 3))
 
