@@ -5,6 +5,8 @@
 
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace jpp_attn {
@@ -105,6 +107,33 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
   const f32x2 v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+// f(integral_constant<int, I>) for I = FROM .. TO - 1
+template <int FROM, int TO, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (FROM < TO) {
+    f(std::integral_constant<int, FROM>{});
+    static_for<FROM + 1, TO>(f);
+  }
+}
+
+// One wave-level HBM -> LDS load whose LDS address is `lds_base` + IMM (both wave-uniform;
+// the add writes M0 itself) and whose source is the wave-uniform address `src` + OFF bytes +
+// the lane's `off`.  (The instruction's offset field moves the source and the LDS address
+// alike, so M0 is set OFF short of the target.)
+template <int IMM, int OFF>
+__device__ __forceinline__ void dma_load16_at(uint64_t src, uint32_t off, uint32_t lds_base) {
+  static_assert(OFF >= 0 && OFF < 4096 && IMM >= OFF, "offset field of a global load");
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4"
+               :
+               : "s"(lds_base), "v"(off), "s"(src), "n"(IMM - OFF), "n"(OFF)
+               : "memory", "scc");
+}
+__device__ __forceinline__ uint64_t uniform_u64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
 }
 
 // Makes the compiler wait here for the loads that produce these registers.  Without it the

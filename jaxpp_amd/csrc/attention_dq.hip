@@ -19,10 +19,14 @@ namespace {
 //   1. S^T = K Q^T, dP^T = V dO^T                         (16 MFMAs at head 128)
 //   2. dS^T = exp2(S^T - lse) (dP^T - delta)              (elementwise)
 //   3. dQ^T += K^T dS^T                                   (8 MFMAs)
-// and one trip issues 3 of the tile before, then 1 of the tile after with 2 of the tile in
-// the middle between its MFMAs.  The K / V row fragments of a 32-key tile stay in registers
-// for its two query tiles, and so do its transposed K fragments; they are replaced, register
-// by register, behind the last MFMAs that read them.
+// and one trip issues the MFMAs of 3 of the tile before and of 1 of the tile after, one at a
+// time, with a share of 2 of the tile in the middle and of the trip's loads behind each: a
+// wave issues in order, and an MFMA that finds the matrix core busy (32 cycles per MFMA)
+// holds back whatever follows it, so two MFMAs in a row would stall the wave while nothing
+// else issues.  The K / V row fragments of a 32-key tile stay in registers for its two query
+// tiles, and so do its transposed K fragments; they are replaced, register by register,
+// behind the MFMAs that read them last.  The softmax scale that belongs on dS is applied to
+// the finished dQ.
 //
 // Under the mask a wave's last block is the one on its diagonal (tile c unseen, a and d
 // masked elementwise); it then only helps to fetch for the waves behind it.
@@ -56,20 +60,46 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   Tile64::offsets(offk, p.ldk, wave, lane);
   Tile64::offsets(offv, p.ldv, wave, lane);
 
-  // part j of the loads of `block` (clamped to the last one, so that every trip of the loop
-  // issues the same number of loads: the waits below count them)
-  auto fetch_part = [&](int block, int j) __attribute__((always_inline)) {
-    const long kn = (long)min(block, nblk - 1) * 64;
-    const uint32_t dst = lds0 + (block & 3) * SLOT;
+  // Per-lane parts of the LDS addresses, in bytes from the start of a slot (a block's K tile,
+  // then its V tile).  Row fragment (tile t, key tile kt, step ks):
+  //   t TILE + (ks >> 2) 8192 + kt 4096 + (a_row ^ (ks & 3) << 5)
+  // (the chunk 2 (ks & 3) + lane / 32 enters the swizzle by XOR, and 2 (ks & 3) has bit 0 clear).
+  // Transposed K fragment (columns 32 i.., key tile kt, steps 2 kt + h2, half hi) - what
+  // slab_frag_tr() reads, the address split into the lane's part and the rest:
+  //   (i >> 1) 8192 + kt 4096 + h2 2048 + hi 1024 + (a_tr ^ ((i & 1) ^ hi) << 6)
+  const uint32_t a_row = lds0 + (uint32_t)slab_off(lane & 31, lane >> 5);
+  uint32_t a_tr;
+  {
+    const int g = lane >> 4, s = lane & 15;
+    a_tr = lds0 + (uint32_t)(((s & 1) << 3) + slab_off(((g >> 1) << 2) + (s >> 2), ((g & 1) << 1) + ((s & 3) >> 1)));
+  }
+  typedef __attribute__((address_space(3))) const bf16x8* lds_frag;
+  typedef __attribute__((address_space(3))) s16x4* lds_s16x4;
+
+  // The fetch cursor: the K / V rows of the block that is fetched next, advanced block by block
+  // and left on the last one (every trip of the loop issues the same number of loads: the
+  // waits below count them).  Part j of a block's loads goes to `dst` + its place in the slot;
+  // the source of a tile's second 64-column slab is an immediate offset.
+  uint64_t f_k = uniform_u64((uint64_t)kbase), f_v = uniform_u64((uint64_t)vbase);
+  const uint64_t f_dk = (uint64_t)p.ldk * 128, f_dv = (uint64_t)p.ldv * 128;  // bytes per 64 rows
+  int f_left = nblk - 1;
+  const uint32_t lds_w = lds0 + wave * (Tile64::INSTS * 1024);
+  auto fetch_part = [&](uint32_t dst, auto j_c) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
     constexpr int PER = Tile64::INSTS;  // loads per wave and 64-column slab
-    const int t = j / (PER * (D / 64)), c = (j / PER) % (D / 64), k = j % PER;
-    const bf16_t* src = t ? vbase + kn * p.ldv : kbase + kn * p.ldk;
-    dma_load16(uniform_ptr(src + c * 64), (t ? offv : offk)[k],
-               dst + t * TILE + c * 8192 + (wave * PER + k) * 1024);
+    constexpr int t = J / (PER * (D / 64)), c = (J / PER) % (D / 64), k = J % PER;
+    dma_load16_at<t * TILE + c * 8192 + k * 1024, c * 128>(t ? f_v : f_k, (t ? offv : offk)[k], dst);
   };
-  auto fetch = [&](int block) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < NLOAD; ++j) fetch_part(block, j);
+  auto fetch_advance = [&]() __attribute__((always_inline)) {
+    const bool go = f_left > 0;
+    f_left -= go ? 1 : 0;
+    f_k += go ? f_dk : 0;
+    f_v += go ? f_dv : 0;
+  };
+  auto fetch = [&](int slot) __attribute__((always_inline)) {
+    const uint32_t dst = lds_w + (uint32_t)slot * SLOT;
+    static_for<0, NLOAD>([&](auto j_c) __attribute__((always_inline)) { fetch_part(dst, j_c); });
+    fetch_advance();
   };
   // the first three key blocks are on their way while this wave's own operands arrive
   fetch(0);
@@ -147,14 +177,14 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   // state of the pipeline between trips
   bf16x8 kfr[KS], vfr[KS];   // K / V rows of the 32-key tile whose scores come next
   bf16x8 ktr[2][DT];         // transposed K of the 32-key tile whose dQ products come next
-  bf16x8 dsf[2];             // dS^T of the tile whose dQ products come next
+  bf16x8 dsf_x[2], dsf_y[2]; // dS^T of the tile whose dQ products come next (two sets alternate)
   f32x16 s_a, dp_a, s_b, dp_b;  // scores of the query tiles 0 / 1
 #pragma unroll
   for (int h2 = 0; h2 < 2; ++h2) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) dsf[h2][e] = (__bf16)0.f;
+    for (int e = 0; e < 8; ++e) { dsf_x[h2][e] = (__bf16)0.f; dsf_y[h2][e] = (__bf16)0.f; }
 #pragma unroll
-    for (int i = 0; i < DT; ++i) ktr[h2][i] = dsf[h2];
+    for (int i = 0; i < DT; ++i) ktr[h2][i] = dsf_x[h2];
   }
 
   // Masks the scores of tile (kt, qt) of `block` just computed: on the wave's diagonal block
@@ -173,93 +203,150 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   };
 
   // One trip.  QP / QC / QN: query tile of the tile before / in the middle / after.  TR:
-  // behind their last use the transposed fragments are replaced by those of key tile `tr_kt`
-  // of the K tile at `tr_src`; ROW: likewise the row fragments, by those of key tile
-  // `row_kt` of the K / V tiles at `row_src`.  `part0`: first of the NLOAD / 4 loads of block
-  // `fetch_block` issued in this trip.  The order of the instructions below is the order they
-  // are issued in: a wave issues in order, and an MFMA that finds the matrix core busy holds
-  // back whatever follows it, so loads and elementwise work sit between the MFMAs.
-  auto trip = [&](auto qp_c, auto qc_c, auto qn_c, auto tr_c, auto row_c, const uint8_t* tr_src,
-                  int tr_kt, const uint8_t* row_src, int row_kt, int fetch_block, int part0,
-                  f32x16& s_c, f32x16& dp_c, f32x16& s_n, f32x16& dp_n) __attribute__((always_inline)) {
+  // behind their last use the transposed fragments are replaced by those of key tile TR_KT of
+  // the K tile whose address registers are b_tr; ROW: likewise the row fragments, by those of
+  // key tile ROW_KT of the K / V tiles whose address registers are b_row.  CALC: which address
+  // registers this trip works out behind its first MFMAs (1: b_tr and b_row from slot offset
+  // `o`; 2: b_row).  PART0: first of the NLOAD / 4 loads issued in this trip, to `dst`.  dS of
+  // the tile in the middle leaves in ds_out; the dQ products of the tile before read ds_in.
+  // The statements below are issued in the order they are written (MFMAs and elementwise
+  // instructions are volatile asm statements, LDS reads do not cross the MFMAs).  Of the
+  // elementwise work on a pair of elements,
+  //   dS = exp2(S sc - lse) (dP - delta),
+  // three MFMAs share the nine instructions so that each sees at most one exponential (16
+  // cycles, the others 4 to 8) and no instruction reads the result of the one before it.
+  auto trip = [&](auto qp_c, auto qc_c, auto qn_c, auto tr_c, auto row_c, auto tr_kt_c, auto row_kt_c,
+                  auto calc_c, auto part0_c, uint32_t o, uint32_t dst, uint32_t (&b_tr)[2],
+                  uint32_t (&b_row)[4], f32x16& s_c, f32x16& dp_c, f32x16& s_n, f32x16& dp_n,
+                  const bf16x8 (&ds_in)[2], bf16x8 (&ds_out)[2]) __attribute__((always_inline)) {
     constexpr int QP = decltype(qp_c)::value, QC = decltype(qc_c)::value,
                   QN = decltype(qn_c)::value;
     constexpr bool TR = decltype(tr_c)::value, ROW = decltype(row_c)::value;
+    constexpr int TR_KT = decltype(tr_kt_c)::value, ROW_KT = decltype(row_kt_c)::value;
+    constexpr int CALC = decltype(calc_c)::value, PART0 = decltype(part0_c)::value;
     constexpr int PARTS = NLOAD / 4;
-    // dQ products of the tile before
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2)
-#pragma unroll
-      for (int i = 0; i < DT; ++i) {
-        mfma_avv(dqacc[QP][i], ktr[h2][i], dsf[h2]);
-        if (TR) ktr[h2][i] = slab_frag_tr(tr_src, 64, i * 32, 2 * tr_kt + h2, lane);
-        if (h2 * DT + i < PARTS) fetch_part(fetch_block, part0 + h2 * DT + i);
-      }
-    // scores of the tile after, two MFMAs at a time, with dS of EPG elements of the tile in
-    // the middle behind each pair
+    constexpr int NSLOT = 2 * DT + 2 * KS;  // MFMAs of the trip
+    constexpr int STEPS = 24 / NSLOT;       // elementwise steps behind each (8 pairs of elements x 3)
+    const float sc_l = sc, lse_l = lse2[QC], dlt_l = dlt[QC];
+    float t0, t1, u0, u1, p0, p1, d0, d1;
     uint32_t dw[8];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      if (ks == 0) {
-        mfma_vva_first(s_n, kfr[0], qf[QN][0]);
-        mfma_vva_first(dp_n, vfr[0], dof[QN][0]);
+    auto arg = [&](float& t, int r) __attribute__((always_inline)) {
+      asm volatile("v_fma_f32 %0, %1, %2, -%3" : "=v"(t) : "v"(s_c[r]), "s"(sc_l), "v"(lse_l));
+    };
+    // step 3 g + ph of the elementwise work on elements 2 g, 2 g + 1
+    auto step = [&](int stp) __attribute__((always_inline)) {
+      const int g = stp / 3, ph = stp % 3, r = 2 * g;
+      if (ph == 0) {
+        asm volatile("v_exp_f32 %0, %1" : "=v"(p0) : "v"(t0));  // exp2(-inf) = 0 where masked
+        asm volatile("v_sub_f32 %0, %1, %2" : "=v"(u0) : "v"(dp_c[r]), "v"(dlt_l));
+        asm volatile("v_sub_f32 %0, %1, %2" : "=v"(u1) : "v"(dp_c[r + 1]), "v"(dlt_l));
+      } else if (ph == 1) {
+        asm volatile("v_exp_f32 %0, %1" : "=v"(p1) : "v"(t1));
+        if (g > 0) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dw[g - 1]) : "v"(d0), "v"(d1));
+        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(d0) : "v"(p0), "v"(u0));
       } else {
-        mfma_vva(s_n, kfr[ks], qf[QN][ks]);
-        mfma_vva(dp_n, vfr[ks], dof[QN][ks]);
+        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(d1) : "v"(p1), "v"(u1));
+        if (g < 7) { arg(t0, r + 2); arg(t1, r + 3); }
       }
-      if (ROW) {
-        kfr[ks] = slabs_frag<D>(row_src, row_kt * 32, ks, lane);
-        vfr[ks] = slabs_frag<D>(row_src + TILE, row_kt * 32, ks, lane);
+    };
+#pragma unroll
+    for (int m = 0; m < NSLOT; ++m) {
+      if (m < 2 * DT) {
+        // dQ products of the tile before
+        const int h2 = m / DT, i = m % DT;
+        mfma_avv(dqacc[QP][i], ktr[h2][i], ds_in[h2]);
+        if (m == 0) { arg(t0, 0); arg(t1, 1); }
+        // (slot offsets are multiples of 1024: adding them commutes with the XORs)
+        if (CALC == 1 && m == 0) {
+          b_tr[0] = a_tr + o;
+          b_tr[1] = b_tr[0] ^ 64;
+          asm volatile("" : "+v"(b_tr[0]), "+v"(b_tr[1]));
+        }
+        if (CALC != 0 && m == 1) {
+          b_row[0] = a_row + o;
+#pragma unroll
+          for (int k = 1; k < 4; ++k) b_row[k] = b_row[0] ^ (k << 5);
+          asm volatile("" : "+v"(b_row[0]), "+v"(b_row[1]), "+v"(b_row[2]), "+v"(b_row[3]));
+        }
+        if (TR) {
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(uintptr_t)(
+              b_tr[i & 1] + ((i >> 1) * 8192 + TR_KT * 4096 + h2 * 2048)));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(uintptr_t)(
+              b_tr[(i & 1) ^ 1] + ((i >> 1) * 8192 + TR_KT * 4096 + h2 * 2048 + 1024)));
+          ktr[h2][i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+        // (the loads go behind MFMAs that have no address work behind them)
+        if (m >= 2 * DT - PARTS) {
+          if (m == 2 * DT - PARTS) fetch_part(dst, std::integral_constant<int, PART0>{});
+          else fetch_part(dst, std::integral_constant<int, PART0 + PARTS - 1>{});
+        }
+      } else {
+        // scores of the tile after
+        const int ks = (m - 2 * DT) >> 1;
+        if ((m - 2 * DT) & 1) {
+          if (ks == 0) mfma_vva_first(dp_n, vfr[0], dof[QN][0]);
+          else mfma_vva(dp_n, vfr[ks], dof[QN][ks]);
+          if (ROW) vfr[ks] = *(lds_frag)(uintptr_t)(b_row[ks & 3] + (TILE + (ks >> 2) * 8192 + ROW_KT * 4096));
+        } else {
+          if (ks == 0) mfma_vva_first(s_n, kfr[0], qf[QN][0]);
+          else mfma_vva(s_n, kfr[ks], qf[QN][ks]);
+          if (ROW) kfr[ks] = *(lds_frag)(uintptr_t)(b_row[ks & 3] + ((ks >> 2) * 8192 + ROW_KT * 4096));
+        }
       }
 #pragma unroll
-      for (int r = ks * EPG; r < ks * EPG + EPG; r += 2) {
-        float s0 = s_c[r], s1 = s_c[r + 1], g0 = dp_c[r], g1 = dp_c[r + 1];
-        asm volatile("" : "+v"(s0), "+v"(s1), "+v"(g0), "+v"(g1));
-        const float p0 = fast_exp2(fmaf(s0, sc, -lse2[QC]));  // exp2(-inf) = 0 where masked
-        const float p1 = fast_exp2(fmaf(s1, sc, -lse2[QC]));
-        dw[r >> 1] = pack2(p0 * (g0 - dlt[QC]), p1 * (g1 - dlt[QC]));
-        asm volatile("" : "+v"(dw[r >> 1]));
-      }
+      for (int e = 0; e < STEPS; ++e) step(m * STEPS + e);
     }
+    asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dw[7]) : "v"(d0), "v"(d1));
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
       typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
       const u32x4 dv = {dw[4 * h2], dw[4 * h2 + 1], dw[4 * h2 + 2], dw[4 * h2 + 3]};
-      dsf[h2] = __builtin_bit_cast(bf16x8, dv);
+      ds_out[h2] = __builtin_bit_cast(bf16x8, dv);
     }
     // The compiler does not know that the asm statements above are MFMAs, whose results take
     // 11 issue slots to land: whatever it does with the new scores (copies included) has to
-    // wait behind this statement, which the elementwise work of the last MFMA pair (nine
-    // instructions and more, tied in front of it) and four idle slots keep clear.
-    asm volatile("s_nop 3" : "+v"(s_n), "+v"(dp_n));
+    // wait behind this statement, which the elementwise work behind the last MFMA (three
+    // instructions or more, and the one above) and eight idle slots keep clear.
+    asm volatile("s_nop 7" : "+v"(s_n), "+v"(dp_n));
   };
 
   using T = std::true_type;
   using F = std::false_type;
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
   constexpr int PARTS = NLOAD / 4;
+  static_assert(PARTS >= 1 && PARTS <= 2 && PARTS <= 2 * DT, "a trip issues one or two loads");
   // The four trips of block j (tiles a, b in s_a, s_b; then c, d).  TAIL: the scores computed
   // here may need the mask (the wave's last block and the one before it).
+  uint32_t b_tr[2] = {0, 0}, b_row[4] = {0, 0, 0, 0};
   auto block_trips = [&](auto tail, int j) __attribute__((always_inline)) {
     constexpr bool TAIL = decltype(tail)::value;
-    const uint8_t* sl = smem + (j & 3) * SLOT;
-    const uint8_t* sl1 = smem + ((j + 1) & 3) * SLOT;
+    // this block's slot (transposed fragments, row fragments of its second key tile), the next
+    // block's (row fragments of its first key tile), and where block j + 3 goes
+    uint32_t o0 = (uint32_t)(j & 3) * SLOT, o1 = (uint32_t)((j + 1) & 3) * SLOT;
+    uint32_t dst = lds_w + (uint32_t)((j + 3) & 3) * SLOT;
+    asm volatile("" : "+s"(o0), "+s"(o1), "+s"(dst));
     // a in the middle: dQ of d of the block before (its transposed fragments give way to
     // this block's first key tile), scores of b (the row fragments give way to the second
     // key tile's)
-    trip(I1{}, I0{}, I1{}, T{}, T{}, sl, 0, sl, 1, j + 3, 0 * PARTS, s_a, dp_a, s_b, dp_b);
+    trip(I1{}, I0{}, I1{}, T{}, T{}, I0{}, I1{}, I1{}, std::integral_constant<int, 0 * PARTS>{}, o0, dst,
+         b_tr, b_row, s_a, dp_a, s_b, dp_b, dsf_x, dsf_y);
     if (TAIL) mask(s_b, j, 0, 1);
     // b in the middle: dQ of a, scores of c
-    trip(I0{}, I1{}, I0{}, F{}, F{}, sl, 0, sl, 0, j + 3, 1 * PARTS, s_b, dp_b, s_a, dp_a);
+    trip(I0{}, I1{}, I0{}, F{}, F{}, I0{}, I0{}, I0{}, std::integral_constant<int, 1 * PARTS>{}, o0, dst,
+         b_tr, b_row, s_b, dp_b, s_a, dp_a, dsf_y, dsf_x);
     if (TAIL) mask(s_a, j, 1, 0);
     // c in the middle: dQ of b (transposed fragments: second key tile moves in), scores of d
     // (row fragments: the next block's first key tile moves in)
-    trip(I1{}, I0{}, I1{}, T{}, T{}, sl, 1, sl1, 0, j + 3, 2 * PARTS, s_a, dp_a, s_b, dp_b);
+    trip(I1{}, I0{}, I1{}, T{}, T{}, I1{}, I0{}, I2{}, std::integral_constant<int, 2 * PARTS>{}, o1, dst,
+         b_tr, b_row, s_a, dp_a, s_b, dp_b, dsf_x, dsf_y);
     if (TAIL) mask(s_b, j, 1, 1);
     // d in the middle: dQ of c, scores of the next block's a
-    trip(I0{}, I1{}, I0{}, F{}, F{}, sl, 0, sl, 0, j + 3, 3 * PARTS, s_b, dp_b, s_a, dp_a);
+    trip(I0{}, I1{}, I0{}, F{}, F{}, I0{}, I0{}, I0{}, std::integral_constant<int, 3 * PARTS>{}, o1, dst,
+         b_tr, b_row, s_b, dp_b, s_a, dp_a, dsf_y, dsf_x);
     if (TAIL) mask(s_a, j + 1, 0, 0);
+    fetch_advance();
   };
 
   dma_wait<NLOAD>();   // blocks 0 and 1 are in (block 2 may be on its way)
@@ -306,7 +393,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
-        for (int i = 0; i < DT; ++i) mfma_avv(dqacc[1][i], ktr[h2][i], dsf[h2]);
+        for (int i = 0; i < DT; ++i) mfma_avv(dqacc[1][i], ktr[h2][i], dsf_x[h2]);
     }
     block_end();
   }
@@ -314,10 +401,10 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
-      for (int i = 0; i < DT; ++i) mfma_avv(dqacc[1][i], ktr[h2][i], dsf[h2]);
+      for (int i = 0; i < DT; ++i) mfma_avv(dqacc[1][i], ktr[h2][i], dsf_x[h2]);
   }
   for (; j < nblk; ++j) {
-    fetch(j + 3);  // its share of the loads for the waves still at work
+    fetch((j + 3) & 3);  // its share of the loads for the waves still at work
     block_end();
   }
   dma_wait_all();
