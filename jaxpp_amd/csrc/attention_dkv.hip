@@ -59,12 +59,15 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
   // dQ kernel left them; the upper half of the wave repeats the lower one into the unused
   // part of the slot
   const uint32_t offst = (uint32_t)((lane & 31) * 16);
+  typedef __attribute__((address_space(3))) const bf16x8* lds_frag;
+  typedef __attribute__((address_space(3))) const f32x4* lds_f4;
+  typedef __attribute__((address_space(3))) s16x4* lds_s16x4;
 
   // Per-lane parts of the LDS addresses, in bytes from the start of a slot.
   // Row fragment (tile t, step ks) of this wave's 32 queries:
   //   t TILE + (ks >> 2) 8192 + (a_row ^ (ks & 3) << 5)
   // (the chunk 2 (ks & 3) + lane / 32 enters the swizzle by XOR, and 2 (ks & 3) has bit 0 clear)
-  const uint32_t a_row = (uint32_t)slab_off(qh * 32 + (lane & 31), lane >> 5);
+  const uint32_t a_row = lds0 + (uint32_t)slab_off(qh * 32 + (lane & 31), lane >> 5);
   // Transposed fragment (tile t, columns 32 ii.., steps 2 qh + h2, half hi) - slab_frag_tr()
   // with its address split into the lane's part and the rest:
   //   t TILE + (ii >> 1) 8192 + h2 2048 + hi 1024 + (a_tr ^ ((ii & 1) ^ hi) << 6)
@@ -73,11 +76,11 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     const int g = lane >> 4, s = lane & 15;
     const int k0 = qh * 32 + ((g >> 1) << 2) + (s >> 2);
     const int c0 = ((g & 1) << 1) + ((s & 3) >> 1);
-    a_tr = (uint32_t)(((s & 1) << 3) + slab_off(k0, c0));
+    a_tr = lds0 + (uint32_t)(((s & 1) << 3) + slab_off(k0, c0));
   }
   // Row statistics: the lane's rows 8 g + 4 (lane / 32) + 0..3 of its query half, four floats
   // per read:  2 TILE + [256 for lse] + 32 g + a_st
-  const uint32_t a_st = (uint32_t)(2 * TILE + (qh * 32 + (lane >> 5) * 4) * 4);
+  const uint32_t a_st = lds0 + (uint32_t)(2 * TILE + (qh * 32 + (lane >> 5) * 4) * 4);
 
   for (int seg = 0; seg < 2; ++seg) {
     const int kb = seg == 0 ? w.x : nkb - 1 - w.x;
@@ -105,37 +108,43 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
 
     const int total = grp * (nkb - kb);   // items; the last grp of them lie on the diagonal
 
-    // The fetch cursor walks the items - running pointers, advanced with selects (the trips of
+    // The fetch cursor walks the items - running addresses, advanced with selects (the trips of
     // the main loop are one basic block) - and stays on the last item once they are exhausted,
     // so every trip issues the same number of loads (the waits below count them).
-    const long head_back = (long)(grp - 1) * D;  // from the last head of a group to the first
-    const bf16_t* f_q = p.q + (row0 + (long)(nkb - 1) * 64) * p.ldq + (long)hk * grp * D;
-    const bf16_t* f_do = p.d_o + (row0 + (long)(nkb - 1) * 64) * p.lddo + (long)hk * grp * D;
-    const float* f_st = p.delta + 2 * (((long)b * p.n_heads + hk * grp) * p.seq + (long)(nkb - 1) * 64);
+    uint64_t f_q = uniform_u64((uint64_t)(p.q + (row0 + (long)(nkb - 1) * 64) * p.ldq + (long)hk * grp * D));
+    uint64_t f_do = uniform_u64((uint64_t)(p.d_o + (row0 + (long)(nkb - 1) * 64) * p.lddo + (long)hk * grp * D));
+    uint64_t f_st = uniform_u64((uint64_t)(p.delta + 2 * (((long)b * p.n_heads + hk * grp) * p.seq + (long)(nkb - 1) * 64)));
+    // bytes from one item to the next: the next head, or (from the last head of a group) the
+    // first head of the query block before
+    const int64_t step_qd = 2 * D, step_st = 8 * (int64_t)p.seq;
+    const int64_t wrap_q = -2 * ((int64_t)(grp - 1) * D + 64 * p.ldq);
+    const int64_t wrap_do = -2 * ((int64_t)(grp - 1) * D + 64 * p.lddo);
+    const int64_t wrap_st = -8 * ((int64_t)(grp - 1) * p.seq + 64);
     int f_h = 0, f_left = total;
-    // part j of an item's loads (NLOAD of them per wave: the Q tile's, the dO tile's, the row
-    // statistics); the last part moves the cursor on
-    auto fetch_part = [&](int slot, int j) __attribute__((always_inline)) {
-      const uint32_t dst = lds0 + slot * SLOT;
+    // part J of an item's loads (NLOAD of them per wave: the Q tile's, the dO tile's, the row
+    // statistics) into the slot at `dst` (this wave's share of it); the last part moves the
+    // cursor on
+    auto fetch_part = [&](uint32_t dst, auto j_c) __attribute__((always_inline)) {
+      constexpr int J = decltype(j_c)::value;
       constexpr int PER = Tile64::INSTS;  // loads per wave and 64-column slab
-      if (j < NLOAD - 1) {
-        const int t = j / (PER * (D / 64)), c = (j / PER) % (D / 64), k = j % PER;
-        dma_load16(uniform_ptr((t ? f_do : f_q) + c * 64), (t ? offdo : offq)[k],
-                   dst + t * TILE + c * 8192 + (wave * PER + k) * 1024);
-        return;
+      if constexpr (J < NLOAD - 1) {
+        constexpr int t = J / (PER * (D / 64)), c = (J / PER) % (D / 64), k = J % PER;
+        dma_load16_at<t * TILE + c * 8192 + k * 1024, c * 128>(t ? f_do : f_q, (t ? offdo : offq)[k], dst);
+      } else {
+        dma_load16_at<2 * TILE, 0>(f_st, offst, dst - wave * (PER * 1024));
+        const bool go = f_left > 1;
+        const bool wrap = go && f_h + 1 == grp;
+        f_left -= go ? 1 : 0;
+        f_h = wrap ? 0 : f_h + (go ? 1 : 0);
+        f_q += wrap ? wrap_q : (go ? step_qd : 0);
+        f_do += wrap ? wrap_do : (go ? step_qd : 0);
+        f_st += wrap ? wrap_st : (go ? step_st : 0);
       }
-      dma_load16(uniform_ptr((const bf16_t*)f_st), offst, dst + 2 * TILE);
-      const bool go = f_left > 1;
-      const bool wrap = go && f_h + 1 == grp;   // next: first head of the query block before
-      f_left -= go ? 1 : 0;
-      f_h = wrap ? 0 : f_h + (go ? 1 : 0);
-      f_q += wrap ? -(head_back + 64 * p.ldq) : (go ? D : 0);
-      f_do += wrap ? -(head_back + 64 * p.lddo) : (go ? D : 0);
-      f_st += wrap ? -2 * ((long)(grp - 1) * p.seq + 64) : (go ? 2 * (long)p.seq : 0);
     };
+    const uint32_t lds_w = lds0 + wave * (Tile64::INSTS * 1024);
     auto fetch = [&](int slot) __attribute__((always_inline)) {
-#pragma unroll
-      for (int j = 0; j < NLOAD; ++j) fetch_part(slot, j);
+      const uint32_t dst = lds_w + (uint32_t)slot * SLOT;
+      static_for<0, NLOAD>([&](auto j_c) __attribute__((always_inline)) { fetch_part(dst, j_c); });
     };
 
     // S and dP of an item (its tiles in `slot`) against this wave's keys
@@ -148,7 +157,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
       }
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const float4 nd = *(const float4*)(slot + a_st + 32 * g);
+        const f32x4 nd = *(lds_f4)(uintptr_t)(a_st + (uint32_t)(slot - smem) + 32 * g);
         dp[4 * g] = nd.x; dp[4 * g + 1] = nd.y; dp[4 * g + 2] = nd.z; dp[4 * g + 3] = nd.w;
       }
       // (the same statements as in the trips: compiler-chosen MFMAs would leave their results
@@ -209,16 +218,15 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
       constexpr int EPG = 16 / KS;  // elements of step 2 per MFMA pair of step 1
       uint32_t b_row[4], b_tr[2], b_stc, b_stn;  // this trip's address registers
       bf16x8 qfr[KS], dofr[KS];     // Q / dO fragments of item i + 1
-      float4 lse_r[4];              // lse of item i's rows
+      f32x4 lse_r[4];             // lse of item i's rows
       auto row_frag = [&](int t, int ks) __attribute__((always_inline)) {
-        return *(const bf16x8*)(smem + b_row[ks & 3] + (t * TILE + (ks >> 2) * 8192));
+        return *(lds_frag)(uintptr_t)(b_row[ks & 3] + (t * TILE + (ks >> 2) * 8192));
       };
       auto tr_frag = [&](int t, int ii, int h2) __attribute__((always_inline)) {
-        typedef __attribute__((address_space(3))) s16x4* lds_s16x4;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)JPP_LDS_PTR(
-            smem + b_tr[ii & 1] + (t * TILE + (ii >> 1) * 8192 + h2 * 2048)));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)JPP_LDS_PTR(
-            smem + b_tr[(ii & 1) ^ 1] + (t * TILE + (ii >> 1) * 8192 + h2 * 2048 + 1024)));
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(uintptr_t)(
+            b_tr[ii & 1] + (t * TILE + (ii >> 1) * 8192 + h2 * 2048)));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)(uintptr_t)(
+            b_tr[(ii & 1) ^ 1] + (t * TILE + (ii >> 1) * 8192 + h2 * 2048 + 1024)));
         const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         return __builtin_bit_cast(bf16x8, v);
       };
@@ -228,19 +236,31 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
           else qfr[n >> 1] = row_frag(0, n >> 1);
         } else if (n < KS + 4) {  // -delta of item i + 1's rows: where its dP products start from
           const int g = n - KS;
-          const float4 nd = *(const float4*)(smem + b_stn + 32 * g);
+          const f32x4 nd = *(lds_f4)(uintptr_t)(b_stn + 32 * g);
           dp_n[4 * g] = nd.x; dp_n[4 * g + 1] = nd.y; dp_n[4 * g + 2] = nd.z; dp_n[4 * g + 3] = nd.w;
         } else {
           const int g = n - KS - 4;
-          lse_r[g] = *(const float4*)(smem + b_stc + (256 + 32 * g));
+          lse_r[g] = *(lds_f4)(uintptr_t)(b_stc + (256 + 32 * g));
         }
       };
       // dV / dK products of item i - 1 from registers; behind each, the transposed fragments
       // of item i take over its operand's registers, and a share of: the reads for steps 1
       // and 2, the loads of item i + 3 into the slot item i - 1 has left
-#pragma unroll
-      for (int m = 0; m < NB; ++m) {
-        const int h2 = m / (2 * DT), ii = (m >> 1) % DT;
+      uint32_t dst = lds_w + (uint32_t)((i + 3) & 3) * SLOT;
+      asm volatile("" : "+s"(dst));
+      // The loads of item i + 3 (into the slot item i - 1 has left) go behind the MFMAs of step
+      // 3, evenly spread.  (Behind those of step 1 as well they cost 6 % of the kernel, and so
+      // did starting the four waves of a trip 16 cycles apart - tried because a CU's waves
+      // share one path to memory, 16 cycles per wave-level load, and wait for each other when
+      // they reach their loads together.)
+      auto dma_slot = [&](int m) __attribute__((always_inline)) {  // m: constant after unrolling
+        static_for<0, NLOAD>([&](auto j_c) __attribute__((always_inline)) {
+          if (decltype(j_c)::value * NB / NLOAD == m) fetch_part(dst, j_c);
+        });
+      };
+      static_for<0, NB>([&](auto m_c) __attribute__((always_inline)) {
+        constexpr int m = decltype(m_c)::value;
+        constexpr int h2 = m / (2 * DT), ii = (m >> 1) % DT;
         if (m & 1) mfma_avv(dkacc[ii], qtr[h2][ii], dsf[h2]);
         else mfma_avv(dvacc[ii], dotr[h2][ii], pf[h2]);
         if (m == 0) {
@@ -262,15 +282,14 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
         else dotr[h2][ii] = tr_frag(1, ii, h2);
 #pragma unroll
         for (int n = m * NR / NB; n < (m + 1) * NR / NB; ++n) early_read(n);
-#pragma unroll
-        for (int j = m * NLOAD / NB; j < (m + 1) * NLOAD / NB; ++j) fetch_part((i + 3) & 3, j);
-      }
+        dma_slot(m);
+      });
       // S and dP of item i + 1, with P and dS of EPG elements of item i behind each pair:
       // behind the first MFMA the exponentials (and the arguments of the next pair's), behind
       // the second the products and the packing to bf16.  No instruction reads the result of
       // the one before it.
       auto lse_of = [&](int r) __attribute__((always_inline)) {
-        const float4 l4 = lse_r[r >> 2];
+        const f32x4 l4 = lse_r[r >> 2];
         return (r & 3) == 0 ? l4.x : (r & 3) == 1 ? l4.y : (r & 3) == 2 ? l4.z : l4.w;
       };
       float t[EPG], tn[EPG], pe[EPG], de[EPG];
