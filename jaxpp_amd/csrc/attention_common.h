@@ -98,6 +98,9 @@ JPP_MFMA(mfma_vvv, "v", "v", "v")
 __device__ __forceinline__ void mfma_vva_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b) : "memory");
 }
+__device__ __forceinline__ void mfma_vvv_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b) : "memory");
+}
 __device__ __forceinline__ void mfma_vaa_first(f32x16& acc, const bf16x8& a, const bf16x8& b) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "a"(a), "a"(b) : "memory");
 }

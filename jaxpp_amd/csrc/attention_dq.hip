@@ -165,6 +165,23 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qf[qt][ks]), "+a"(dof[qt][ks]));
   settle(lse2[0]); settle(lse2[1]); settle(dlt[0]); settle(dlt[1]);
+  // dP - delta comes out of the matrix core: one more MFMA per tile adds, to every key's row
+  // of dP^T, the queries' -delta - as the product of a [keys x 16] operand of ones in three
+  // columns with a [16 x queries] operand that holds -delta in those three rows, split into
+  // three bf16 terms (24 bits of it)
+  bf16x8 ones_f, nd_f[2];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones_f[e] = (__bf16)((lane < 32 && e < 3) ? 1.f : 0.f);
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const float nd = -dlt[qt];
+    const __bf16 hi = (__bf16)nd;
+    const __bf16 mid = (__bf16)(nd - (float)hi);
+    const __bf16 lo = (__bf16)(nd - (float)hi - (float)mid);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) nd_f[qt][e] = (__bf16)0.f;
+    if (lane < 32) { nd_f[qt][0] = hi; nd_f[qt][1] = mid; nd_f[qt][2] = lo; }
+  }
 
   f32x16 dqacc[2][DT];
 #pragma unroll
@@ -207,7 +224,8 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
   // the K tile whose address registers are b_tr; ROW: likewise the row fragments, by those of
   // key tile ROW_KT of the K / V tiles whose address registers are b_row.  CALC: which address
   // registers this trip works out behind its first MFMAs (1: b_tr and b_row from slot offset
-  // `o`; 2: b_row).  PART0: first of the NLOAD / 4 loads issued in this trip, to `dst`.  dS of
+  // `o`; 2: b_row).  PART0: with NLOAD / 4 loads of the block to `dst` per trip, this trip's first
+  // (a trip without TR issues its own and those of the trip before it).  dS of
   // the tile in the middle leaves in ds_out; the dQ products of the tile before read ds_in.
   // The statements below are issued in the order they are written (MFMAs and elementwise
   // instructions are volatile asm statements, LDS reads do not cross the MFMAs).  Of the
@@ -225,27 +243,24 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     constexpr int TR_KT = decltype(tr_kt_c)::value, ROW_KT = decltype(row_kt_c)::value;
     constexpr int CALC = decltype(calc_c)::value, PART0 = decltype(part0_c)::value;
     constexpr int PARTS = NLOAD / 4;
-    constexpr int NSLOT = 2 * DT + 2 * KS;  // MFMAs of the trip
-    constexpr int STEPS = 24 / NSLOT;       // elementwise steps behind each (8 pairs of elements x 3)
-    const float sc_l = sc, lse_l = lse2[QC], dlt_l = dlt[QC];
-    float t0, t1, u0, u1, p0, p1, d0, d1;
+    constexpr int NSLOT = 2 * DT + 1 + 2 * KS;  // MFMAs of the trip
+    const float sc_l = sc, lse_l = lse2[QC];
+    float t0, t1, p0, p1, d0, d1;
     uint32_t dw[8];
     auto arg = [&](float& t, int r) __attribute__((always_inline)) {
       asm volatile("v_fma_f32 %0, %1, %2, -%3" : "=v"(t) : "v"(s_c[r]), "s"(sc_l), "v"(lse_l));
     };
-    // step 3 g + ph of the elementwise work on elements 2 g, 2 g + 1
+    // step 3 g + ph of the elementwise work on elements 2 g, 2 g + 1 (dp_c holds dP - delta)
     auto step = [&](int stp) __attribute__((always_inline)) {
       const int g = stp / 3, ph = stp % 3, r = 2 * g;
       if (ph == 0) {
         asm volatile("v_exp_f32 %0, %1" : "=v"(p0) : "v"(t0));  // exp2(-inf) = 0 where masked
-        asm volatile("v_sub_f32 %0, %1, %2" : "=v"(u0) : "v"(dp_c[r]), "v"(dlt_l));
-        asm volatile("v_sub_f32 %0, %1, %2" : "=v"(u1) : "v"(dp_c[r + 1]), "v"(dlt_l));
+        if (g > 0) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dw[g - 1]) : "v"(d0), "v"(d1));
       } else if (ph == 1) {
         asm volatile("v_exp_f32 %0, %1" : "=v"(p1) : "v"(t1));
-        if (g > 0) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dw[g - 1]) : "v"(d0), "v"(d1));
-        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(d0) : "v"(p0), "v"(u0));
+        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(d0) : "v"(p0), "v"(dp_c[r]));
       } else {
-        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(d1) : "v"(p1), "v"(u1));
+        asm volatile("v_mul_f32 %0, %1, %2" : "=v"(d1) : "v"(p1), "v"(dp_c[r + 1]));
         if (g < 7) { arg(t0, r + 2); arg(t1, r + 3); }
       }
     };
@@ -275,17 +290,21 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
               b_tr[(i & 1) ^ 1] + ((i >> 1) * 8192 + TR_KT * 4096 + h2 * 2048 + 1024)));
           ktr[h2][i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         }
-        // (the loads go behind MFMAs that have no address work behind them)
-        if (m >= 2 * DT - PARTS) {
-          if (m == 2 * DT - PARTS) fetch_part(dst, std::integral_constant<int, PART0>{});
-          else fetch_part(dst, std::integral_constant<int, PART0 + PARTS - 1>{});
-        }
+        // the block's loads go out in the trips that read nothing from LDS, half in each (3 %
+        // of the kernel against a quarter in every trip)
+        if constexpr (!TR) if (m < 2 * PARTS)
+          static_for<0, 2 * PARTS>([&](auto q_c) __attribute__((always_inline)) {
+            if (decltype(q_c)::value == m)
+              fetch_part(dst, std::integral_constant<int, PART0 - PARTS + decltype(q_c)::value>{});
+          });
+      } else if (m == 2 * DT) {
+        // -delta of the tile after's queries: where its dP products start from
+        mfma_vvv_first(dp_n, ones_f, nd_f[QN]);
       } else {
         // scores of the tile after
-        const int ks = (m - 2 * DT) >> 1;
-        if ((m - 2 * DT) & 1) {
-          if (ks == 0) mfma_vva_first(dp_n, vfr[0], dof[QN][0]);
-          else mfma_vva(dp_n, vfr[ks], dof[QN][ks]);
+        const int ks = (m - 2 * DT - 1) >> 1;
+        if ((m - 2 * DT - 1) & 1) {
+          mfma_vva(dp_n, vfr[ks], dof[QN][ks]);
           if (ROW) vfr[ks] = *(lds_frag)(uintptr_t)(b_row[ks & 3] + (TILE + (ks >> 2) * 8192 + ROW_KT * 4096));
         } else {
           if (ks == 0) mfma_vva_first(s_n, kfr[0], qf[QN][0]);
@@ -294,7 +313,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
         }
       }
 #pragma unroll
-      for (int e = 0; e < STEPS; ++e) step(m * STEPS + e);
+      for (int stp = m * 24 / NSLOT; stp < (m + 1) * 24 / NSLOT; ++stp) step(stp);
     }
     asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(dw[7]) : "v"(d0), "v"(d1));
 #pragma unroll
@@ -361,7 +380,8 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     for (int ks = 0; ks < KS; ++ks) {
       if (ks == 0) {
         mfma_vva_first(s_a, kfr[0], qf[0][0]);
-        mfma_vva_first(dp_a, vfr[0], dof[0][0]);
+        mfma_vvv_first(dp_a, ones_f, nd_f[0]);
+        mfma_vva(dp_a, vfr[0], dof[0][0]);
       } else {
         mfma_vva(s_a, kfr[ks], qf[0][ks]);
         mfma_vva(dp_a, vfr[ks], dof[0][ks]);
