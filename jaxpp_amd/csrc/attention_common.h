@@ -55,12 +55,13 @@ __device__ __forceinline__ void rope_back(f32x16 (&acc)[DT], const float* cos_ta
     }
 }
 
-// 8 consecutive accumulator registers -> one bf16 MFMA operand
+// 8 consecutive accumulator registers -> one bf16 MFMA operand (round to nearest even; two
+// elements per conversion instruction)
 __device__ __forceinline__ bf16x8 acc_to_frag(const f32x16& a, int base) {
-  bf16x8 f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) f[e] = (__bf16)a[base + e];
-  return f;
+  typedef float f32x8 __attribute__((ext_vector_type(8)));
+  const f32x8 v = {a[base], a[base + 1], a[base + 2], a[base + 3],
+                   a[base + 4], a[base + 5], a[base + 6], a[base + 7]};
+  return __builtin_convertvector(v, bf16x8);
 }
 
 // row-major operand fragment straight from HBM (lane: row = lane&31, 8

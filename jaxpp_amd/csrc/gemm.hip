@@ -116,10 +116,7 @@ __device__ __forceinline__ void swiglu_grad_f(float g, float u, float d, float& 
 // XCDs (8 of them, each with its own L2); give every XCD a contiguous range of
 // tiles, and inside a range walk GROUP tile-rows at a time so the B panels in
 // flight stay L2 resident.
-#ifndef JPP_COLUMN_SPLIT_ROWS
-#define JPP_COLUMN_SPLIT_ROWS 64
-#endif
-constexpr int kColumnSplitRows = JPP_COLUMN_SPLIT_ROWS;  // tile rows from which XCDs split by columns
+constexpr int kColumnSplitRows = 64;  // tile rows from which XCDs split by columns
 
 __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int nwg = tiles_m * tiles_n;
