@@ -44,14 +44,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   const int q0 = qb * 128 + wave * 32;
   const int qi = q0 + (lane & 31);  // this lane's query position
 
-  bf16x8 qf[KS];
-  {
-    const bf16_t* qbase = p.q + (row0 + q0) * p.ldq + h * D;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = global_frag(qbase, p.ldq, ks, lane);
-  }
-  settle(qf);
-
   f32x16 oacc[DT];
 #pragma unroll
   for (int i = 0; i < DT; ++i)
@@ -68,10 +60,26 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   Tile64::offsets(offv, p.ldv, wave, lane);
   const uint32_t lds0 = lds_address(smem);
 
+  // The workgroup's 128 rows of Q come through LDS like the K / V tiles (two tiles, in the
+  // stage the loop fills second): a fragment taken from HBM directly touches 32 rows with 32
+  // bytes each, and the CU's path to memory takes such a load line by line.
+  bf16x8 qf[KS];
+  {
+    Tile64::Offsets offq;
+    Tile64::offsets(offq, p.ldq, wave, lane);
+    const bf16_t* qbase = p.q + (row0 + (long)qb * 128) * p.ldq + h * D;
+    dma_tile<D>(qbase, offq, lds0 + STAGE, wave);
+    dma_tile<D>(qbase + 64 * p.ldq, offq, lds0 + STAGE + TILE, wave);
+  }
   dma_tile<D>(kbase, offk, lds0, wave);
   dma_tile<D>(vbase, offv, lds0 + TILE, wave);
   dma_wait_all();
   __syncthreads();
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    qf[ks] = slabs_frag<D>(smem + STAGE + (wave >> 1) * TILE, (wave & 1) * 32, ks, lane);
+  settle(qf);
+  __syncthreads();  // the stage is block 1's from the first trip on
 
   for (int blk = 0; blk < nblk; ++blk) {
     const int k0 = blk * 64;
@@ -166,16 +174,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.0f / l_tot;
-  bf16_t* orow = p.o + (row0 + qi) * p.ldo + h * D;
 #pragma unroll
   for (int i = 0; i < DT; ++i)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int dv = i * 32 + g * 8 + (lane >> 5) * 4;
-      *(uint2*)(orow + dv) =
-          make_uint2(pack_bf16x2(oacc[i][4 * g] * inv, oacc[i][4 * g + 1] * inv),
-                     pack_bf16x2(oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv));
-    }
+    for (int r = 0; r < 16; ++r) oacc[i][r] *= inv;
+  // (the K / V stages are idle: the loop ends behind a barrier)
+  store_tile_by_rows<D, DT>(oacc, lds0 + wave * (32 * D * 2), p.o + (row0 + q0) * p.ldo + h * D,
+                            p.ldo, lane);
   if (lane < 32)
     p.lse[((long)b * p.n_heads + h) * p.seq + qi] = m_run * p.scale + logf(l_tot);
 }
@@ -327,15 +332,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) dqacc[i][r] *= p.scale;
   if (p.rope_cos) rope_back<D, DT>(dqacc, p.rope_cos, p.rope_sin, qi, lane);
-  bf16_t* drow = p.dq + (row0 + qi) * p.lddq + h * D;
-#pragma unroll
-  for (int i = 0; i < DT; ++i)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int d = i * 32 + g * 8 + (lane >> 5) * 4;
-      *(uint2*)(drow + d) = make_uint2(pack_bf16x2(dqacc[i][4 * g], dqacc[i][4 * g + 1]),
-                                       pack_bf16x2(dqacc[i][4 * g + 2], dqacc[i][4 * g + 3]));
-    }
+  // (the K / V stages are idle: the loop ends behind a barrier)
+  store_tile_by_rows<D, DT>(dqacc, lds0 + wave * (32 * D * 2), p.dq + (row0 + q0) * p.lddq + h * D,
+                            p.lddq, lane);
 }
 
 // ---------------------------------------------------------------------------

@@ -113,6 +113,43 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
+// A wave's 32 x D result tile leaves through LDS by rows.  In the accumulators a lane holds,
+// of row lane & 31, the columns 32 i + 8 g + 4 (lane >> 5) + 0..3 in acc[i][4 g ..]: stored
+// from there, one instruction would touch 32 rows with 8 bytes each, and the CU's path to
+// memory takes such an instruction line by line.  So the tile is rounded to bf16 into `stage`
+// (32 * D * 2 bytes of LDS that only this wave uses; 16-byte units of a row XOR-ed with the
+// row index, which spreads a write over the banks) and read back with a lane owning 16
+// consecutive bytes of a row, 64 / (D / 8) whole rows per store instruction.  LDS operations
+// of one wave execute in order: no barrier.
+template <int D, int DT>
+__device__ __forceinline__ void store_tile_by_rows(const f32x16 (&acc)[DT], uint32_t stage,
+                                                   bf16_t* dst, long ld, int lane) {
+  static_assert(DT * 32 == D, "head of D elements in DT tiles of 32");
+  constexpr int UNITS = D / 8, RPI = 64 / UNITS;
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) u32x2* lds_u2;
+  typedef __attribute__((address_space(3))) const u32x4* lds_u4;
+  const int row = lane & 31, hh = lane >> 5;
+  const uint32_t wbase = stage + row * (D * 2) + hh * 8;
+#pragma unroll
+  for (int i = 0; i < DT; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int u = i * 4 + g;
+      *(lds_u2)(uintptr_t)(wbase + (uint32_t)((u ^ (row & (UNITS - 1))) << 4)) =
+          u32x2{pack2(acc[i][4 * g], acc[i][4 * g + 1]), pack2(acc[i][4 * g + 2], acc[i][4 * g + 3])};
+    }
+  const int r0 = lane / UNITS, U = lane % UNITS;
+#pragma unroll
+  for (int k = 0; k < 32 / RPI; ++k) {
+    const int r = k * RPI + r0;
+    const u32x4 v = *(lds_u4)(uintptr_t)(stage + r * (D * 2) + (uint32_t)((U ^ (r & (UNITS - 1))) << 4));
+    *(u32x4*)(dst + (long)r * ld + U * 8) = v;
+  }
+}
+
+
 // f(integral_constant<int, I>) for I = FROM .. TO - 1
 template <int FROM, int TO, class F>
 __device__ __forceinline__ void static_for(F&& f) {

@@ -86,20 +86,17 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     const int kb = seg == 0 ? w.x : nkb - 1 - w.x;
     const int k0 = kb * 64 + ksb * 32;
 
+    // The key block's K and V tiles come through LDS like every other tile (into the slot the
+    // ring uses last): a fragment taken from HBM directly touches 32 rows with 32 bytes each,
+    // and the CU's path to memory takes such a load line by line.
     bf16x8 kf[KS], vf[KS];
     {
-      const bf16_t* kbase = p.k + (row0 + k0) * p.ldk + hk * D;
-      const bf16_t* vbase = p.v + (row0 + k0) * p.ldv + hk * D;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        kf[ks] = global_frag(kbase, p.ldk, ks, lane);
-        vf[ks] = global_frag(vbase, p.ldv, ks, lane);
-      }
+      Tile64::Offsets offk, offv;
+      Tile64::offsets(offk, p.ldk, wave, lane);
+      Tile64::offsets(offv, p.ldv, wave, lane);
+      dma_tile<D>(p.k + (row0 + (long)kb * 64) * p.ldk + hk * D, offk, lds0 + 3 * SLOT, wave);
+      dma_tile<D>(p.v + (row0 + (long)kb * 64) * p.ldv + hk * D, offv, lds0 + 3 * SLOT + TILE, wave);
     }
-    // (waits for the loads here, and names where the fragments live: the accumulation
-    // registers, where the MFMAs of the trips read them)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(kf[ks]), "+a"(vf[ks]));
     f32x16 dkacc[DT], dvacc[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i)
@@ -346,6 +343,18 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     fetch(0);
     fetch(1);
     fetch(2);
+    dma_wait<3 * NLOAD>();  // the K / V tiles are in
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      kf[ks] = slabs_frag<D>(smem + 3 * SLOT, ksb * 32, ks, lane);
+      vf[ks] = slabs_frag<D>(smem + 3 * SLOT + TILE, ksb * 32, ks, lane);
+    }
+    // (names where the fragments live: the accumulation registers, where the MFMAs of the
+    // trips read them)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(kf[ks]), "+a"(vf[ks]));
+    lds_wait_all();  // the slot is item 3's from the first trip on
     dma_wait<NLOAD>();
     __syncthreads();
     f32x16 s_a, dp_a, s_b, dp_b;
@@ -383,8 +392,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
     __syncthreads();
     if (qh == 0) {
       const int ki = k0 + (lane_e & 31);
-      bf16_t* dkrow = p.dk + (row0 + ki) * p.lddk + hk * D;
-      bf16_t* dvrow = p.dv + (row0 + ki) * p.lddv + hk * D;
 #pragma unroll
       for (int i = 0; i < DT; ++i)
 #pragma unroll
@@ -393,17 +400,11 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkv_kernel(AttnParams p) {
           dvacc[i][r] += xch[((DT + i) * 16 + r) * 64];
         }
       if (p.rope_cos) rope_back<D, DT>(dkacc, p.rope_cos, p.rope_sin, ki, lane_e);
-#pragma unroll
-      for (int i = 0; i < DT; ++i) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int d = i * 32 + g * 8 + (lane_e >> 5) * 4;
-          *(uint2*)(dkrow + d) = make_uint2(pack_bf16x2(dkacc[i][4 * g], dkacc[i][4 * g + 1]),
-                                            pack_bf16x2(dkacc[i][4 * g + 2], dkacc[i][4 * g + 3]));
-          *(uint2*)(dvrow + d) = make_uint2(pack_bf16x2(dvacc[i][4 * g], dvacc[i][4 * g + 1]),
-                                            pack_bf16x2(dvacc[i][4 * g + 2], dvacc[i][4 * g + 3]));
-        }
-      }
+      // (staged in ring memory behind the exchange area; the ring is idle until the barrier below)
+      constexpr uint32_t XCH = 2 * (2 * DT * 16 * 64 * 4);
+      const uint32_t stage = lds0 + XCH + wave * (2 * 32 * D * 2);
+      store_tile_by_rows<D, DT>(dkacc, stage, p.dk + (row0 + k0) * p.lddk + hk * D, p.lddk, lane_e);
+      store_tile_by_rows<D, DT>(dvacc, stage + 32 * D * 2, p.dv + (row0 + k0) * p.lddv + hk * D, p.lddv, lane_e);
     }
     __syncthreads();  // the exchange area is slot memory of the next key block
   }

@@ -448,20 +448,11 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     for (int qt = 0; qt < 2; ++qt)
       rope_back<D, DT>(dqacc[qt], p.rope_cos, p.rope_sin, q0 + qt * 32 + (lane & 31), lane);
   }
+  // (the ring is free: every wave has left the loop behind its last barrier)
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
-    const int qi = q0 + qt * 32 + (lane & 31);
-    bf16_t* drow = p.dq + (row0 + qi) * p.lddq + h * D;
-#pragma unroll
-    for (int i = 0; i < DT; ++i)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int d = i * 32 + g * 8 + (lane >> 5) * 4;
-        *(uint2*)(drow + d) =
-            make_uint2(pack_bf16x2(dqacc[qt][i][4 * g], dqacc[qt][i][4 * g + 1]),
-                       pack_bf16x2(dqacc[qt][i][4 * g + 2], dqacc[qt][i][4 * g + 3]));
-      }
-  }
+  for (int qt = 0; qt < 2; ++qt)
+    store_tile_by_rows<D, DT>(dqacc[qt], lds0 + (wave * 2 + qt) * (32 * D * 2),
+                              p.dq + (row0 + q0 + qt * 32) * p.lddq + h * D, p.lddq, lane);
 }
 
 }  // namespace
