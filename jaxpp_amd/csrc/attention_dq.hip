@@ -101,34 +101,69 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     static_for<0, NLOAD>([&](auto j_c) __attribute__((always_inline)) { fetch_part(dst, j_c); });
     fetch_advance();
   };
+  // This wave's Q and dO as MFMA operands (accumulation registers), and per query tile the
+  // row's log-sum-exp (exp2 domain) and delta = sum_d dO * O: a lane holds half of its row of
+  // dO (the chunks the fragments give it) and the same half of O, the other half is with
+  // lane ^ 32.  The wave's 64 rows of Q, dO and O come through LDS, one after the other
+  // through 64 * D * 2 bytes that only this wave uses (half of the ring's last slot, or of a
+  // slot's worth of LDS behind the ring), as the swizzled slabs slabs_frag() reads: a fragment
+  // taken from HBM directly touches 32 rows with 32 bytes each, and the CU's path to memory
+  // takes such a load line by line (the three tensors that way: 19 k cycles per workgroup).
+  // One load instruction brings 8 rows x 128 bytes; which 16 bytes a lane brings depends on
+  // the row's swizzle, which differs between even and odd groups of 8 rows by chunk bit 2.
+  const uint32_t stg_off = (wave < 2 ? 3 * SLOT : 4 * SLOT) + (wave & 1) * (SLOT / 2);
+  auto stage_rows = [&](const bf16_t* base, long ld) __attribute__((always_inline)) {
+    const int r8 = lane >> 3, c_e = (lane & 7) ^ slab_swz(r8);
+    const uint32_t off_e = (uint32_t)(r8 * ld * 2 + (c_e << 4)), off_o = (uint32_t)(r8 * ld * 2 + ((c_e ^ 4) << 4));
+    uint64_t src = uniform_u64((uint64_t)base);
+    const uint64_t step = (uint64_t)ld * 16;  // 8 rows
+    static_for<0, 8>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      static_for<0, D / 64>([&](auto c_c) __attribute__((always_inline)) {
+        constexpr int c = decltype(c_c)::value;
+        dma_load16_at<c * 8192 + i * 1024, c * 128>(src, (i & 1) ? off_o : off_e, lds0 + stg_off);
+      });
+      src += step;
+    });
+  };
+  auto staged_frag = [&](int qt, int ks) __attribute__((always_inline)) {
+    return slabs_frag<D>(smem + stg_off, qt * 32, ks, lane);
+  };
+  bf16x8 qf[2][KS], dof[2][KS];
+  uint4 ov[2][KS];
+  float lse2[2] = {0.f, 0.f}, dlt[2] = {0.f, 0.f};
+  const long rows = row0 + q0;
+  if (active) {
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+      lse2[qt] = p.lse[((long)b * p.n_heads + h) * p.seq + q0 + qt * 32 + (lane & 31)];
+    stage_rows(p.q + rows * p.ldq + h * D, p.ldq);
+  }
   // the first three key blocks are on their way while this wave's own operands arrive
   fetch(0);
   fetch(1);
   fetch(2);
-
-  // This wave's Q and dO as MFMA operands (accumulation registers), and per query tile the
-  // row's log-sum-exp (exp2 domain) and delta = sum_d dO * O:
-  // a lane holds half of its row of dO (the chunks the fragments give it) and reads the same
-  // half of O, the other half is with lane ^ 32.  All loads are issued before the first of
-  // them is waited for.
-  bf16x8 qf[2][KS], dof[2][KS];
-  uint4 ov[2][KS];
-  float lse2[2] = {0.f, 0.f}, dlt[2] = {0.f, 0.f};
   if (active) {
+    dma_wait<3 * NLOAD>();  // Q is in (loads complete in order)
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      const long r = row0 + q0 + qt * 32;
-      const bf16_t* qbase = p.q + r * p.ldq + h * D;
-      const bf16_t* dobase = p.d_o + r * p.lddo + h * D;
-      const bf16_t* obase = p.o + r * p.ldo + h * D;
+    for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        qf[qt][ks] = global_frag(qbase, p.ldq, ks, lane);
-        dof[qt][ks] = global_frag(dobase, p.lddo, ks, lane);
-        ov[qt][ks] = *(const uint4*)(obase + (long)(lane & 31) * p.ldo + ks * 16 + (lane >> 5) * 8);
-      }
-      lse2[qt] = p.lse[((long)b * p.n_heads + h) * p.seq + q0 + qt * 32 + (lane & 31)];
-    }
+      for (int ks = 0; ks < KS; ++ks) qf[qt][ks] = staged_frag(qt, ks);
+    lds_wait_all();
+    stage_rows(p.d_o + rows * p.lddo + h * D, p.lddo);
+    dma_wait_all();
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) dof[qt][ks] = staged_frag(qt, ks);
+    lds_wait_all();
+    stage_rows(p.o + rows * p.ldo + h * D, p.ldo);
+    dma_wait_all();
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ov[qt][ks] = __builtin_bit_cast(uint4, staged_frag(qt, ks));
+    lds_wait_all();  // (the ring's last slot is block 3's from the first trips on)
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
       const long stat = ((long)b * p.n_heads + h) * p.seq + q0 + qt * 32 + (lane & 31);
@@ -462,7 +497,7 @@ int launch_dq(hipStream_t stream, const AttnParams& p, int head_dim, bool causal
   const dim3 grid((p.seq + 255) / 256, p.n_heads, p.batch);
 #define JPP_DQ(D_, C_)                                                                  \
   do {                                                                                  \
-    constexpr int LDS = 4 * 2 * D_ * 128;                                               \
+    constexpr int LDS = 5 * 2 * D_ * 128;  /* the ring, and a slot's worth for the prologue */ \
     if (int rc = set_smem(attn_bwd_dq_kernel<D_, C_>, LDS)) return rc;                  \
     hipLaunchKernelGGL((attn_bwd_dq_kernel<D_, C_>), grid, dim3(256), LDS, stream, p);  \
   } while (0)
