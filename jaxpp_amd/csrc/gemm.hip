@@ -310,7 +310,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   // of A, each fragment read while the block before it computes.
   // Waits count requests from the youngest (vmcnt is in order): at the wait point of K-step
   // t the copies of K-steps t+2 .. t+NS-1 and the accumulator rows requested during the last
-  // NS-1 K-steps may stay in flight.
+  // NS-1 K-steps may stay in flight (where a stage's refill is split over two K-steps, see
+  // LATE below, its second half is the youngest request and everything is waited for).
   constexpr int OPB = IA + IB;  // operand copies per wave and K-step
   bf16x8 fw[2][TN], fx[2][TMH];
   if (kt_n > 0) {
@@ -330,6 +331,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
 
   int st = 0;   // stage of K-step kt: kt % NS
   int cbi = 0;  // accumulator-row buffer of K-step kt: kt % (NS + 1)
+  // The refill of a retired stage is 8 wave-level copies per wave, 64 per workgroup, and the
+  // CU's path to memory takes one in 16 cycles: issued all behind the barrier, under the last
+  // MFMA block, they kept that block waiting on the path (a wave issues in order) for twice
+  // the time its MFMAs need.  With two stages the 256 x 256 tile therefore issues LATE of
+  // its four parts under the first MFMA block of the next K-step instead (still three blocks
+  // ahead of the wait for them): 4 - 6 % per K-step by timestamps inside the loop, 0.2 - 1 %
+  // of the Llama-3-8B-shaped step depending on the device.  (3 or 4 parts late: slower again,
+  // the copies land too late.)
+  constexpr int LATE = (NS == 2 && BM == 256 && BN == 256 && NW == 8) ? 2 : 0;
+  constexpr bool SPLIT = LATE > 0;
+  const bf16_t* ga_late = nullptr;
+  const bf16_t* gb_late = nullptr;
+  int st_late = 0;
   for (int kt = 0; kt < kt_n; ++kt) {
     const int nst = st + 1 == NS ? 0 : st + 1;
     const uint8_t* sa = smem + st * STAGE;
@@ -358,7 +372,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
           int cin = 0;
           if (EPI == JPP_EPI_ACC_F32 && stream_c)
             cin = max(0, min(kt - 1, NBT - 1) - max(0, kt + 1 - NS) + 1);
-          if (cin <= 0) dma_wait<(NS - 2) * OPB>();
+          if (SPLIT || cin <= 0) dma_wait<(NS - 2) * OPB>();
           else if (cin == 1) dma_wait<(NS - 2) * OPB + 1>();
           else if (cin == 2) dma_wait<(NS - 2) * OPB + 2>();
           else dma_wait<(NS - 2) * OPB + 3>();
@@ -402,7 +416,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
       static_assert(TMH % 2 == 0 && TN % 2 == 0, "2x2 groups of MFMA tiles");
 #pragma unroll
       for (int ib = 0; ib < TMH / 2; ++ib) {
-        if (ks == NB - 1) {
+        if (!SPLIT && ks == NB - 1) {
 #pragma unroll
           for (int i = 2 * ib; i < 2 * ib + 2; ++i)
             if (i % (TMH / PARTS) == 0) {
@@ -410,6 +424,24 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
               TileB::template issue_part<IB / PARTS>(i / (TMH / PARTS), gb, offb,
                                                      lds0 + st * STAGE + A_BYTES, wave);
             }
+        }
+        if constexpr (SPLIT) {
+          static_assert(!SPLIT || (PARTS == 4 && TMH == 4 && LATE <= 4), "four parts, two per block");
+          // parts 0 .. 3 - LATE in the last block (spread from its end), the others one per
+          // pair of MFMA rows from the start of the next K-step on
+          const int slot = ks * 2 + ib;           // pair of MFMA rows within the K-step
+          if (ks == NB - 1) {
+            const int part = slot - (2 * NB - (4 - LATE));
+            if (part >= 0) {
+              TileA::template issue_part<IA / PARTS>(part, ga, offa, lds0 + st * STAGE, wave);
+              TileB::template issue_part<IB / PARTS>(part, gb, offb, lds0 + st * STAGE + A_BYTES, wave);
+            }
+          } else if (slot < LATE && kt > 0) {
+            const int part = 4 - LATE + slot;
+            TileA::template issue_part<IA / PARTS>(part, ga_late, offa, lds0 + st_late * STAGE, wave);
+            TileB::template issue_part<IB / PARTS>(part, gb_late, offb,
+                                                   lds0 + st_late * STAGE + A_BYTES, wave);
+          }
         }
         // a walk over the 2 x TN tiles of this pair of rows, the next pair taking the columns in
         // the opposite direction
@@ -433,6 +465,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
         dma_load16(uniform_ptr((const bf16_t*)p.c), c_off0 + (uint32_t)(kt * NW * p.ldc * 4),
                    lds0 + C_LDS + (cbi * NW + wave) * C_PITCH);
     }
+    ga_late = ga; gb_late = gb; st_late = st;
     st = nst;
     cbi = cbi + 1 == NS + 1 ? 0 : cbi + 1;
   }
