@@ -462,7 +462,10 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     fetch((j + 3) & 3);  // its share of the loads for the waves still at work
     block_end();
   }
+  // every wave's loads have landed before the ring serves as the output's staging space (the
+  // last trips fetch the last block again, into slots the staging may share)
   dma_wait_all();
+  __syncthreads();
   if (!active) return;
 
   // (the MFMAs above are asm statements: their results are settled before the compiler's
@@ -483,7 +486,6 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_kernel(AttnParams p) {
     for (int qt = 0; qt < 2; ++qt)
       rope_back<D, DT>(dqacc[qt], p.rope_cos, p.rope_sin, q0 + qt * 32 + (lane & 31), lane);
   }
-  // (the ring is free: every wave has left the loop behind its last barrier)
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt)
     store_tile_by_rows<D, DT>(dqacc[qt], lds0 + (wave * 2 + qt) * (32 * D * 2),
