@@ -13,8 +13,17 @@ stage-level 1e-3 (the worst of them 4 x the bound, as everywhere).  That is what
 arithmetic does at this depth: evaluated twice on the sweep's six-layer BERT pipeline, with
 float32 and with float64 accumulation, it disagrees with itself on 2.5e-3 of the first layer's
 QKV weight gradient, by up to 2.5 x (tests/test_oracle_stage.py,
-test_bf16_sensitivity_of_a_six_layer_pipeline).  How good the bf16 results are is held
-separately: no farther from the float32 computation than the bf16 oracle's own
+test_bf16_sensitivity_of_a_six_layer_pipeline).  At eight layers a fixed figure stops being one:
+a further draw of this sweep (offset 200000, seed 4: BERT, 4 stages of 2 layers) has 4.65e-3 of
+that tensor outside the bound while the device is as close to the float32 run as the bf16 oracle
+is (0.99 x in the Frobenius norm) and the float32 run itself has 2.4e-2 of its elements outside
+the same bound around the bf16 oracle.  (A four-layer one of the same sweep, seed 5, has 1.5e-3 against the
+stage-level 1e-3 in the same way.)  So where the float32 run exists, a gradient is also
+granted half of that run's own count: the device may disagree with the bf16 oracle on half as
+many elements as the unrounded computation does (seen: a fifth at most), and its worst element
+may be 1.5 x as far outside the bound as that run's worst is (of 400 further draws one six-layer
+pipeline had an element at 4.1 x, with the float32 run's worst of that tensor at 4.0 x; the
+float32 run's worst elements sit at 3 - 7 x, the device's at 0.5 - 1.0 of them).  How good the bf16 results are is held separately: no farther from the float32 computation than the bf16 oracle's own
 (parity.close_to_truth).  The sweep is for dataflow errors - a wrong slot, a microbatch counted
 twice, a stage out of order - which put whole tensors off by their own magnitude."""
 import os
@@ -77,6 +86,11 @@ def draw(seed):
 # fraction of a tensor's elements granted outside the elementwise bound: the stage-level
 # figure, and what pipelines of more than four layers get (see the module's text)
 DEEP_BAD_FRAC = 4e-3
+# ... and what any gradient gets of the count of the float32 run's elements outside the same bound
+# around the bf16 oracle
+DEEP_TRUTH_SHARE = 0.5
+# ... and how far outside it the worst element may be, in units of that run's worst
+TRUTH_EXCESS = 1.5
 
 
 @pytest.mark.parametrize("seed", range(40))
@@ -129,7 +143,14 @@ def test_random_train_step_matches_sequential_loop(seed):
         for li in range(per):
             for k, v in want_acc[s][li].items():
                 got = np.asarray(grad["layers"][s * per + li][k], np.float32)
-                parity.close(got, v.reshape(got.shape), 2e-2, f"grad {s}/{li}/{k}", BAD_FRAC, EXCESS)
+                frac, excess = BAD_FRAC, EXCESS
+                if truth:
+                    t_bad, t_n, t_worst = parity.violations(
+                        np.asarray(truth[1][s][li][k], np.float32).reshape(got.shape),
+                        np.asarray(v, np.float32).reshape(got.shape), 2e-2)
+                    frac = max(frac, DEEP_TRUTH_SHARE * t_bad / max(t_n, 1))
+                    excess = max(excess, TRUTH_EXCESS * t_worst)
+                parity.close(got, v.reshape(got.shape), 2e-2, f"grad {s}/{li}/{k}", frac, excess)
                 if truth:
                     parity.close_to_truth(got, v, truth[1][s][li][k], f"grad {s}/{li}/{k}")
     train_step.close()
