@@ -21,7 +21,7 @@ the same bound around the bf16 oracle.  (A four-layer one of the same sweep, see
 stage-level 1e-3 in the same way.)  So where the float32 run exists, a gradient is also
 granted half of that run's own count: the device may disagree with the bf16 oracle on half as
 many elements as the unrounded computation does (seen: a fifth at most), and its worst element
-may be 1.5 x as far outside the bound as that run's worst is (of 400 further draws one six-layer
+may be 1.5 x as far outside the bound as that run's worst is (of 360 further draws one six-layer
 pipeline had an element at 4.1 x, with the float32 run's worst of that tensor at 4.0 x; the
 float32 run's worst elements sit at 3 - 7 x, the device's at 0.5 - 1.0 of them).  How good the bf16 results are is held separately: no farther from the float32 computation than the bf16 oracle's own
 (parity.close_to_truth).  The sweep is for dataflow errors - a wrong slot, a microbatch counted
