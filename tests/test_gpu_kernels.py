@@ -237,6 +237,9 @@ def test_gemm_with_rotary_epilogue(batch, seq, heads, rot_heads, d, k, tile):
     (64, 1, 16, 8, 1, 1024),
     # eight query heads per key-value head (the 70B-shaped layer's grouping)
     (128, 1, 16, 2, 1, 512), (128, 1, 64, 8, 1, 256),
+    # head 128 with an odd number of 128-query blocks: the last workgroup of the dQ kernel is half
+    # empty, and its last loads go to the slot its first waves stage their output through
+    (128, 1, 8, 2, 1, 640),
 ])
 def test_attention_fwd_bwd(d, causal, hq, hkv, batch, seq):
     print(f"attention d={d} causal={causal} hq={hq} hkv={hkv} b={batch} s={seq}", flush=True)
