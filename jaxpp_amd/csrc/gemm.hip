@@ -87,12 +87,33 @@ struct GemmArgs<true> {
   GemmProblem more[3];   // problems 1..3; `first` past the grid for those not in use
 };
 
+// erf(u / sqrt 2) and exp(-u^2 / 2) for the exact GELU and its derivative: the rational
+// approximation 7.1.26 of Abramowitz & Stegun (one reciprocal, one exponential, five fused
+// multiply-adds; absolute error 6e-7 in fp32, that of a float erf 1e-7 - either is three
+// orders below half a bf16 ulp of the results, and on bf16-valued N(0, 1.5) inputs as many
+// of the rounded results differ from a float64 evaluation's as with the library's erff: 2e-3
+// of gelu's - tiny values of the negative tail -, 4e-4 of its derivative's).  The library
+// call costs about 35 instructions, and an epilogue of a 256 x 256 tile makes 128 of them per
+// lane: 17 - 23 us of a 52 - 58 us GEMM at 4096 x 4096 x 1024.
+__device__ __forceinline__ void erf_and_gauss(float u, float& erf_x, float& gauss) {
+  const float ax = fabsf(u) * 0.7071067811865476f;
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, ax, 1.0f));
+  gauss = __expf(-ax * ax);
+  float poly = fmaf(1.061405429f, t, -1.453152027f);
+  poly = fmaf(poly, t, 1.421413741f);
+  poly = fmaf(poly, t, -0.284496736f);
+  poly = fmaf(poly, t, 0.254829592f);
+  erf_x = copysignf(fmaf(-poly * t, gauss, 1.0f), u);
+}
+
 __device__ __forceinline__ float gelu_f(float u, int tanh_form) {
   if (tanh_form) {
     float t = tanhf(0.7978845608028654f * (u + 0.044715f * u * u * u));
     return 0.5f * u * (1.0f + t);
   }
-  return 0.5f * u * (1.0f + erff(u * 0.7071067811865476f));
+  float e, g;
+  erf_and_gauss(u, e, g);
+  return 0.5f * u * (1.0f + e);
 }
 
 __device__ __forceinline__ float gelu_grad_f(float u, int tanh_form) {
@@ -101,8 +122,9 @@ __device__ __forceinline__ float gelu_grad_f(float u, int tanh_form) {
     return 0.5f * (1.0f + t) +
            0.5f * u * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 0.134145f * u * u);
   }
-  return 0.5f * (1.0f + erff(u * 0.7071067811865476f)) +
-         u * __expf(-0.5f * u * u) * 0.3989422804014327f;
+  float e, g;
+  erf_and_gauss(u, e, g);
+  return 0.5f * (1.0f + e) + u * g * 0.3989422804014327f;
 }
 
 __device__ __forceinline__ float swiglu_f(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
