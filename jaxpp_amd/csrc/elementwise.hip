@@ -468,7 +468,7 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restric
     unpack8(*(const uint4*)(gu + t * 2 * f + gate_col(c, f, il)), a);
     unpack8(*(const uint4*)(gu + t * 2 * f + up_col(c, f, il)), b);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) a[e] = a[e] / (1.0f + __expf(-a[e])) * b[e];
+    for (int e = 0; e < 8; ++e) a[e] = a[e] * __builtin_amdgcn_rcpf(1.0f + __expf(-a[e])) * b[e];  // as the GEMM epilogue's
     *(uint4*)(s + t * f + c * 8) = pack8(a);
   }
 }
@@ -489,7 +489,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restric
     unpack8(*(const uint4*)(ds + t * f + c * 8), d);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float sg = 1.0f / (1.0f + __expf(-a[e]));
+      const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-a[e]));
       const float da = d[e] * b[e] * sg * (1.0f + a[e] * (1.0f - sg));
       const float db = d[e] * a[e] * sg;
       a[e] = da;
