@@ -216,8 +216,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
     bid -= JPP_PICK(0, first);
 #undef JPP_PICK
   }
-  using TileA = DmaTile<BM, TA, NW>;
-  using TileB = DmaTile<BN, TB, NW>;
+  // Which waves issue the HBM -> LDS copies.  With two waves per SIMD the older one is served
+  // first whenever it has an instruction ready, so it runs ahead and then waits at the
+  // K-step's barrier for the younger one, whose K-step is therefore what a tile's time is made
+  // of - and a wave issues in order: every copy it issues (16 cycles of the CU's path to
+  // memory, longer when other waves' copies are queued) holds back its next MFMA.  So the four
+  // older waves issue all copies (twice as many each) in the time they would wait anyway, and
+  // the younger ones only read fragments and multiply: 2.4 - 3.3 % of the step on the Llama-
+  // and Mixtral-shaped stages, 2 % on the BERT-large-shaped one (single GEMMs: TN -5 %,
+  // NN / NT -2.5 % at 4096 x 28672 x 4096; two shapes of twelve +1 - 2 %).
+  constexpr int DW = NW == 8 ? 4 : NW;
+  using TileA = DmaTile<BM, TA, DW>;
+  using TileB = DmaTile<BN, TB, DW>;
   constexpr int A_BYTES = TileA::BYTES, STAGE = TileA::BYTES + TileB::BYTES;
   constexpr int WN = NW / 2;                        // waves: 2 along m, NW/2 along n
   // 16x16 MFMA tiles per wave.  A K-step runs them in 2 HS blocks of TMH x TN (32 contraction
@@ -227,7 +237,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   constexpr int NB = 2 * HS;
   extern __shared__ __align__(1024) uint8_t smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // (wave-uniform where the waves differ in what they do: a scalar branch around the copies)
+  const int wave = DW == NW ? tid >> 6 : __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool dma_wave = wave < DW;
   const int wm = wave / WN, wn = wave % WN;
   int tm, tn;
   const int tiles = p.tiles_m * p.tiles_n;
@@ -344,8 +357,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       const int k = min(s, kt_n - 1);
-      TileA::template issue<0, IA>(uniform_ptr(a_at(k)), offa, lds0 + s * STAGE, wave);
-      TileB::template issue<0, IB>(uniform_ptr(b_at(k)), offb, lds0 + s * STAGE + A_BYTES, wave);
+      if (dma_wave) {
+        TileA::template issue<0, IA>(uniform_ptr(a_at(k)), offa, lds0 + s * STAGE, wave);
+        TileB::template issue<0, IB>(uniform_ptr(b_at(k)), offb, lds0 + s * STAGE + A_BYTES, wave);
+      }
     }
     dma_wait<(NS - 1) * OPB>();  // stage 0 has landed; the others may still be in flight
   }
@@ -445,7 +460,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
         if (!SPLIT && ks == NB - 1) {
 #pragma unroll
           for (int i = 2 * ib; i < 2 * ib + 2; ++i)
-            if (i % (TMH / PARTS) == 0) {
+            if (i % (TMH / PARTS) == 0 && dma_wave) {
               TileA::template issue_part<IA / PARTS>(i / (TMH / PARTS), ga, offa, lds0 + st * STAGE, wave);
               TileB::template issue_part<IB / PARTS>(i / (TMH / PARTS), gb, offb,
                                                      lds0 + st * STAGE + A_BYTES, wave);
@@ -458,11 +473,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
           const int slot = ks * 2 + ib;           // pair of MFMA rows within the K-step
           if (ks == NB - 1) {
             const int part = slot - (2 * NB - (4 - LATE));
-            if (part >= 0) {
+            if (part >= 0 && dma_wave) {
               TileA::template issue_part<IA / PARTS>(part, ga, offa, lds0 + st * STAGE, wave);
               TileB::template issue_part<IB / PARTS>(part, gb, offb, lds0 + st * STAGE + A_BYTES, wave);
             }
-          } else if (slot < LATE && kt > 0) {
+          } else if (slot < LATE && kt > 0 && dma_wave) {
             const int part = 4 - LATE + slot;
             TileA::template issue_part<IA / PARTS>(part, ga_late, offa, lds0 + st_late * STAGE, wave);
             TileB::template issue_part<IB / PARTS>(part, gb_late, offb,
