@@ -467,7 +467,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
             }
         }
         if constexpr (SPLIT) {
-          static_assert(!SPLIT || (PARTS == 4 && TMH == 4 && LATE <= 4), "four parts, two per block");
+          static_assert(!SPLIT || (PARTS == 4 && TMH == 4 && LATE >= 2 && LATE <= 4),
+                        "four parts, at most two of them in the last block (it has two slots)");
           // parts 0 .. 3 - LATE in the last block (spread from its end), the others one per
           // pair of MFMA rows from the start of the next K-step on
           const int slot = ks * 2 + ib;           // pair of MFMA rows within the K-step
