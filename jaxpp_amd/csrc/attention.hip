@@ -306,6 +306,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
             dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[ks], dof[ks], dp, 0, 0, 0);
           }
         }
+        // (wave priority by phase as in the forward kernel: -3 % at the BERT-large shape)
+        __builtin_amdgcn_s_setprio(2);
         bf16x8 ktr[2][DT];  // K^T fragments arrive under the elementwise arithmetic
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2)
@@ -324,6 +326,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
           const float pr = fast_exp2(fmaf(s[r], sc, -lse2));  // exp2(-inf) = 0 where masked
           s[r] = pr * (dp[r] - dlt);  // (the softmax scale is applied to dQ at the end)
         }
+        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
           const bf16x8 dsf = acc_to_frag(s, h2 * 8);
@@ -331,6 +334,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(AttnParams p) {
           for (int i = 0; i < DT; ++i)
             dqacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr[h2][i], dsf, dqacc[i], 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
       }
     }
     dma_wait_all();
@@ -449,6 +453,8 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
                                                             vf[ks], dp[u], 0, 0, 0);
           }
         }
+        // (wave priority by phase as in the forward kernel: -2 % at the BERT-large shape)
+        __builtin_amdgcn_s_setprio(2);
 #pragma unroll
         for (int u = 0; u < TB; ++u) {
           const int t = t0 + u;
@@ -469,6 +475,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
             }
           }
         }
+        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int u = 0; u < TB; ++u) {
           const int t = t0 + u;
@@ -485,6 +492,7 @@ __global__ __launch_bounds__(256, (D > 64 ? 1 : 2)) void attn_bwd_dkv_wide_kerne
             }
           }
         }
+        __builtin_amdgcn_s_setprio(0);
       }
     }
     park((it + 1) & 1);
