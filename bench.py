@@ -160,12 +160,15 @@ def default_wgrad_group(wl, two_streams: bool) -> int:
     fours (73 GB); 70B-shaped 4579-4584 / 4545-4552 / 4543-4554 ms (197 / 215 / 251 GB), so
     pairs there.  The Mixtral-shaped stage 2671-2699 ms ungrouped, 2615-2627 in pairs (206 /
     236 GB; the experts' grouped contraction takes the pairs' own row groups): pairs, fours do
-    not fit.  Narrow layers run two streams: ungrouped."""
-    if two_streams or wl.layer.family not in ("llama", "mixtral") or wl.layer.hidden < 4096:
+    not fit.  BERT-large-shaped stage: a layer's four weight gradients are 192 tiles, three
+    quarters of one round of the 256 CUs; four microbatches' are three full rounds - 52.5 ms
+    ungrouped, 51.5 in pairs, 51.0 in fours on one stream, 52.0 / 52.0 / 51.0 with the weight
+    gradients on a second stream."""
+    if wl.dtype != "bf16":
         return 1
-    if wl.layer.family == "mixtral":
+    if wl.layer.family == "mixtral" or wl.layer.hidden >= 8192:
         return 2
-    return 4 if wl.layer.hidden < 8192 else 2
+    return 4
 
 
 def cpu_baseline(wl, budget_layers: int = 1):
@@ -219,12 +222,12 @@ def main():
                          "rocprofv3 --pmc, which serialises every dispatch; not the headline)")
     ap.add_argument("--unfused-accumulate", action="store_true",
                     help="bf16 weight gradient + separate fp32 accumulate pass")
-    ap.add_argument("--two-streams", choices=["auto", "on", "off"], default="auto",
+    ap.add_argument("--two-streams", choices=["on", "off"], default="off",
                     help="weight gradients on the stage's second stream and the forward of a "
-                         "fused entry beside its backward.  auto: on when the layers are too "
-                         "narrow for one kernel to fill the chip (hidden < 2048: +7%% at cfg2), off "
-                         "otherwise (-1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
-                         "include the other stream's kernels)")
+                         "fused entry beside its backward.  Measured: 52.0 ms against 52.5 at "
+                         "cfg2 with ungrouped weight gradients, no difference with groups of "
+                         "four (51.0); -1%% at cfg3, -2%% at cfg5, and per-kernel timings then "
+                         "include the other stream's kernels")
     ap.add_argument("--wgrad-group", type=int, default=None,
                     help="weight gradients of this many consecutive microbatches as one product "
                          "per weight (1: per microbatch; default: see default_wgrad_group)")
@@ -279,9 +282,9 @@ def main():
     if args.n_mubatches:
         import dataclasses
         wl = dataclasses.replace(wl, n_mubatches=args.n_mubatches)
-    two = wl.layer.hidden < 2048 if args.two_streams == "auto" else args.two_streams == "on"
+    two = args.two_streams == "on"
     group = args.wgrad_group if args.wgrad_group is not None else default_wgrad_group(wl, two)
-    if args.unfused_accumulate or two:
+    if args.unfused_accumulate:
         group = 1
     use_graph = args.graph == "on" or (args.graph == "auto" and wl.layer.hidden < 2048)
     wb = Workbench(wl, fused=not args.unfused_accumulate, two_streams=two, wgrad_group=group)
@@ -421,8 +424,8 @@ def side_run(wl, name: str, wgrad_group: int | None = None, steps: int = 3, warm
     settings the bench would choose for it; the executor is freed afterwards."""
     import gc
     gc.collect()
-    two = wl.layer.hidden < 2048
-    group = 1 if two else (wgrad_group if wgrad_group is not None else default_wgrad_group(wl, two))
+    two = False
+    group = wgrad_group if wgrad_group is not None else default_wgrad_group(wl, two)
     wb = Workbench(wl, fused=True, two_streams=two, wgrad_group=group)
     ms, _ = timed_steps(wb, steps, warmup, use_graph=wl.layer.hidden < 2048, cls=None)
     flops = wb.step_flops()

@@ -453,7 +453,9 @@ typedef struct {
                             arriving in between sends what is pending ahead as a shorter
                             product (same sums, other rounding).  If a grouped launch fails
                             the stage is unusable: every later task and join returns
-                            JPP_ERR_STATE.  One stream, bf16, fused_wgrad_accum only. */
+                            JPP_ERR_STATE.  bf16 and fused_wgrad_accum only.  With
+                            two_streams a group runs on the stage's second stream, behind
+                            the input-gradient half of its last member. */
 } jpp_stage_desc;
 
 

@@ -630,7 +630,7 @@ int layer_bwd_w_group(jpp_stage* s, hipStream_t st, int chunk, int li, int n, ui
     return run_wgrads(s, st, wb);
   }
   if (s->d.family == JPP_FAMILY_MIXTRAL) {
-    float* partial = s->S<float>(s->s_partial);
+    float* partial = s->S<float>(st == s->side && s->side ? s->s_partial_side : s->s_partial);
     const int E = s->d.n_experts;
     // the experts' weight gradients over all n microbatches at once where the grouped
     // contraction takes several operand pairs (each with its own row groups: the routing
@@ -698,8 +698,27 @@ int run_pending_w(jpp_stage* s, hipStream_t st, int chunk) {
   const int n = (int)pend.size();
   for (int i = 0; i < n; ++i) slots[i] = s->slots[pend[i].second];
   int rc = JPP_OK;
+  hipStream_t ws = st;
+  if (s->side) {
+    // the group runs on the second stream, behind everything the caller's stream holds so
+    // far (the input-gradient halves that wrote the cotangents in the slots)
+    JPP_CHECK_HIP(hipEventRecord(s->ev_fork, st));
+    JPP_CHECK_HIP(hipStreamWaitEvent(s->side, s->ev_fork, 0));
+    ws = s->side;
+  }
   for (int li = s->d.layers_per_chunk - 1; li >= 0 && rc == JPP_OK; --li)
-    rc = layer_bwd_w_group(s, st, chunk, li, n, slots);
+    rc = layer_bwd_w_group(s, ws, chunk, li, n, slots);
+  if (s->side && rc == JPP_OK) {
+    // a forward that takes one of these slots next waits for the group to have read it
+    for (auto& e : pend) {
+      if (hipEventRecord(s->ev_slot[e.second], s->side) != hipSuccess)
+        rc = jpp_set_error(JPP_ERR_HIP, "run_task: hipEventRecord on the second stream failed");
+      s->slot_pending[e.second] = 1;
+    }
+    if (hipEventRecord(s->ev_tail, s->side) != hipSuccess)
+      rc = jpp_set_error(JPP_ERR_HIP, "run_task: hipEventRecord on the second stream failed");
+    s->tail_pending = true;
+  }
   for (auto& e : pend) {
     const auto key = std::make_pair(chunk, e.first);
     s->free_slots.push_back(e.second);
@@ -842,9 +861,8 @@ int jpp_stage_create(const jpp_stage_desc* d, jpp_stage** out) {
 
   JPP_REQUIRE(d->wgrad_group >= 0 && d->wgrad_group <= 4, "stage_create: wgrad_group must be 0..4");
   if (d->wgrad_group > 1)
-    JPP_REQUIRE(!d->two_streams && d->fused_wgrad_accum && d->dtype == JPP_DTYPE_BF16,
-                "stage_create: grouped weight gradients need one stream, bf16 and accumulation "
-                "in the GEMM");
+    JPP_REQUIRE(d->fused_wgrad_accum && d->dtype == JPP_DTYPE_BF16,
+                "stage_create: grouped weight gradients need bf16 and accumulation in the GEMM");
 
   jpp_stage* s = new jpp_stage();
   s->d = *d;

@@ -395,7 +395,8 @@ def test_mixtral_8x7b_layer_on_a_dualpipev_row_matches_oracle():
 def test_bench_row_equals_sequential_order(name, peak):
     """The rows bench.py times, at full size and with its own device state (bench.Workbench):
     cfg3 = Interleaved1F1B(8, 4) rank 0, 32 microbatches, 2 x 4 Llama-3-8B-shaped layers;
-    cfg2 = Std1F1B(4) rank 0, 16 microbatches, 6 BERT-large layers, two streams.  No oracle at
+    cfg2 = Std1F1B(4) rank 0, 16 microbatches, 6 BERT-large layers (its ungrouped passes with the
+    weight gradients on the stage's second stream, which bench.py offers as an option).  No oracle at
     this size; instead the reference's own invariant (tests/test_transformations.py:187-191):
     the scheduled row must give bit-identical results to the same work in sequential order
     (every microbatch forward then backward, chunk by chunk) - every task's output and every
@@ -470,13 +471,13 @@ def test_bench_row_equals_sequential_order(name, peak):
             for pname, v in gd.items():
                 np.testing.assert_array_equal(g[i][pname], v, err_msg=f"{what}: grad {i}/{pname}")
     ex.close()
-    group = bench.default_wgrad_group(wl, two)
+    group = bench.default_wgrad_group(wl, False)
     if group > 1:
         # the mode the bench runs by default: weight gradients of `group` microbatches as one
         # product per weight.  Outputs bit-identical; accumulators equal up to f32
         # reassociation; a microbatch held back keeps its slot, so the peak is higher.
         del wb, outs_sched, outs_loop, grads_sched, grads_loop
-        wb = bench.Workbench(wl, fused=True, two_streams=two, wgrad_group=group)
+        wb = bench.Workbench(wl, fused=True, two_streams=False, wgrad_group=group)
         ex = wb.ex
         ex.zero_grads()
         for b in outs.values():

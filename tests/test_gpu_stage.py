@@ -242,6 +242,16 @@ def test_grouped_weight_gradients(name, spec, sched, n, rank):
                 if not (spec.family == "mixtral" and pname in ("Wr", "Wgu", "Wd")):
                     want = acc_w[st][0][pname].reshape(v.shape)
                     parity.close_stage(got[2][st][0][pname], want, 2e-2, f"group {group}: grad {st}/{pname}")
+        # the groups on the stage's second stream, the row queued without host waits: the same
+        # launches in the same order per accumulator, so bit for bit the one-stream result
+        side = run_on_gpu(spec, plan, 1, params, two_streams=True, wgrad_group=group)
+        for i in (0, 1):
+            for k, v in got[i].items():
+                np.testing.assert_array_equal(side[i][k], v, err_msg=f"group {group}, two streams: {i}/{k}")
+        for st in plan.stages:
+            for pname, v in got[2][st][0].items():
+                np.testing.assert_array_equal(side[2][st][0][pname], v,
+                                              err_msg=f"group {group}, two streams: grad {st}/{pname}")
 
 
 def test_grouped_weight_gradients_do_not_depend_on_task_order():
@@ -301,8 +311,8 @@ def test_grouped_weight_gradients_hold_their_slots():
     assert ex.live_slots() == 0
     rt.sync()
     ex.close()
-    with pytest.raises(rt.JppError, match="grouped weight gradients need one stream"):
-        rt.StageExecutor(spec, 1, 1, 1, False, True, True, wgrad_group=2)
+    with pytest.raises(rt.JppError, match="grouped weight gradients need bf16 and accumulation"):
+        rt.StageExecutor(spec, 1, 1, 1, False, False, False, wgrad_group=2)
 
 
 def test_routing_readback():
