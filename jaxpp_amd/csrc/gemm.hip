@@ -58,6 +58,9 @@ struct GemmParams {
   int n_seg, group_mode;
   int64_t group_rows;
   long stride_b, stride_c;
+  // JPP_GROUP_M as two launches (see group_head_rows): 1 = the 256x256 tiles of the rows
+  // before the split, 2 = smaller tiles over the rows behind it, 0 = one launch for all rows
+  int tail_split;
   // rotary embedding in the bf16 epilogue of the forward kernels (NULL: none): columns
   // [0, rope_cols) are heads of rope_hd elements, row r is position (rope_row0 + r) % rope_seq
   const float* rope_cos;
@@ -182,6 +185,16 @@ __device__ __forceinline__ const bf16_t* part_ptr(const bf16_t* p0, const bf16_t
   const int start = part == 0 ? 0 : part == 1 ? c1 : part == 2 ? c2 : c3;
   return base + (long)(kt - start) * step;
 }
+// Row-grouped products know the number of rows in use (`rows`, a multiple of 256) on the
+// device only; the grid covers the buffer's capacity.  When the 256x256 tiles of those rows
+// end in a round that fills at most half of the 256 CUs, the tile rows of that round are
+// left to a second launch of 128x128 tiles (four times as many tiles, a round of which takes
+// about a third of the time): returns the first row of that part, `rows` when there is none.
+__device__ __forceinline__ long group_head_rows(int rows, int n) {
+  const int tm = rows / 256, tn = n / 256, total = tm * tn, rest = total % 256;
+  const bool split = total > 256 && rest > 0 && rest <= 128 && rest % tn == 0;
+  return split ? (long)(tm - rest / tn) * 256 : (long)rows;
+}
 // K-steps that hold data of row group e of a grouped contraction
 __device__ __forceinline__ int group_steps(const int* seg, const int* seg_rows, int e) {
   const int rows = seg_rows ? min(seg_rows[e], seg[e + 1] - seg[e]) : seg[e + 1] - seg[e];
@@ -245,7 +258,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   int tm, tn;
   const int tiles = p.tiles_m * p.tiles_n;
   tile_of_block(p.group_mode == JPP_GROUP_K ? bid % tiles : bid, p.tiles_m, p.tiles_n, tm, tn);
-  const long m0 = (long)tm * BM, n0 = (long)tn * BN;
+  long m0 = (long)tm * BM;
+  const long n0 = (long)tn * BN;
+  if (p.group_mode == JPP_GROUP_M && p.tail_split) {
+    const long head = group_head_rows(p.seg[p.n_seg], p.n);
+    if (p.tail_split == 1) {
+      if (m0 >= head) return;
+    } else {
+      m0 += head;
+    }
+  }
 
   const long a_off = TA ? m0 : m0 * p.lda, b_off = TB ? n0 : n0 * p.ldb;
   const bf16_t* a_src = p.a + a_off;
@@ -747,6 +769,7 @@ int launch(hipStream_t stream, GemmParams& p) {
                     : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;
   double am = p.m, ak = (double)p.k * (p.k_parts > 1 ? p.k_parts : 1), copies = 1;
   if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
+  if (p.tail_split == 2) am = 0;   // the launch over the rows before the split carries the product's work
   if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
   const double b_bytes = 2.0 * p.n * ak * (p.group_mode == JPP_GROUP_M ? p.n_seg : 1);
   ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW, NS>(), 2.0 * am * p.n * ak,
@@ -925,6 +948,7 @@ int prepare(const jpp_gemm_args* a, GemmParams& p) {
   p.gelu_tanh = a->gelu_tanh;
   p.seg = a->seg; p.seg_rows = a->seg_rows; p.n_seg = a->n_seg; p.group_mode = a->group_mode;
   p.group_rows = a->group_rows;
+  p.tail_split = 0;
   p.stride_b = a->stride_b; p.stride_c = a->stride_c;
   p.k_parts = a->k_parts > 1 ? a->k_parts : 1;
   p.kt_part = (int)(a->k / 64);
@@ -1032,6 +1056,20 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
         const int rc = dispatch(stream, a, head, 4);
         return rc != JPP_OK ? rc : dispatch(stream, a, tail, 3);
       }
+    }
+  }
+  // Row groups: how many rows are in use is known on the device only, so the same split is
+  // made there (group_head_rows) - the second launch is always enqueued and its workgroups
+  // leave at once when the first one's tiles cover every row.
+  if (tile == 4 && a->tile == 0 && a->group_mode == JPP_GROUP_M && a->epilogue == JPP_EPI_BF16) {
+    const long tm = a->m / 256, tn = a->n / 256;
+    if (tm * tn > 256 && tn <= 128) {
+      GemmParams head = p, tail = p;
+      head.tail_split = 1;
+      tail.tail_split = 2;
+      tail.m = (int)std::min<long>(a->m, 128 / tn * 256);   // at most 128 tiles of 256x256
+      const int rc = dispatch(stream, a, head, 4);
+      return rc != JPP_OK ? rc : dispatch(stream, a, tail, 1);
     }
   }
   return dispatch(stream, a, p, tile);

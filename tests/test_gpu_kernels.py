@@ -641,6 +641,49 @@ def test_grouped_gemm():
                 n_seg=E, group_mode=2, stride_c=h * f, tile=4, more=[(d_xp_b.ptr, d_dy_b.ptr)])
 
 
+@pytest.mark.parametrize("trans_b", [1, 0], ids=["nn", "nt"])
+@pytest.mark.parametrize("counts,h", [
+    ([520, 300, 256, 1100, 700, 300, 255, 513], 128),    # 20 tile rows x 16: last round 64 tiles -> 4 rows split off
+    ([520, 300, 256, 1100, 700, 300, 255, 513], 2048),   # ... with the deeper prefetch of a long contraction
+    ([512, 512, 512, 512, 512, 512, 512, 512], 128),     # 16 x 16 = one full round: nothing to split
+    ([1024, 512, 512, 512, 512, 512, 512, 600], 128),    # 19 x 16: 48 tiles -> 3 rows split off
+    ([2048, 512, 512, 512, 512, 512, 512, 1300], 128),   # 26 x 16: 160 tiles in the last round: no split
+    ([256, 0, 0, 0, 0, 0, 0, 1], 128),                   # 2 x 16: less than a round: no split
+], ids=["rest64", "rest64-long", "full", "rest48", "rest160", "small"])
+def test_grouped_gemm_last_round(counts, h, trans_b):
+    """Row-grouped products whose 256x256 tiles end in a round that fills at most half of the
+    CUs run that round's rows as 128x128 tiles in a second launch; where the split falls is
+    decided on the device from the rows in use.  Bit for bit the single launch on 256x256
+    tiles (the caller's choice of tile switches the split off), and right against numpy."""
+    rng = np.random.default_rng(sum(counts) + trans_b)
+    E, f = 8, 4096
+    seg = np.zeros(E + 1, np.int32)
+    for e, c in enumerate(counts):
+        seg[e + 1] = seg[e] + (c + 255) // 256 * 256
+    cap = int(seg[E]) + 768                       # the grid covers the capacity, not the rows in use
+    xp = np.zeros((cap, h), np.float32)
+    for e, c in enumerate(counts):
+        xp[seg[e]:seg[e] + c] = rnd(rng, c, h)
+    w = rnd(rng, E, h, f, scale=0.1 if h < 1024 else 0.03)
+    wd = np.ascontiguousarray(w.transpose(0, 2, 1)) if not trans_b else w     # [E, f, h] for nt
+    b_seg, b_xp, b_w = rt.DeviceBuffer.from_numpy(seg), dev_bf16(xp), dev_bf16(wd)
+    outs = []
+    for tile in (0, 4):
+        out = rt.DeviceBuffer(cap * f * 2)
+        out.zero()
+        print(f"grouped product, counts {counts}, h {h}, trans_b {trans_b}, tile {tile}", flush=True)
+        rt.gemm(b_xp.ptr, b_w.ptr, out.ptr, cap, f, h, h, f if trans_b else h, f, 0, trans_b,
+                rt.EPI_BF16, seg=b_seg.ptr, n_seg=E, group_mode=1, stride_b=h * f, tile=tile)
+        rt.sync()
+        outs.append(out.download_bf16((cap, f)))
+    np.testing.assert_array_equal(outs[0], outs[1])
+    xb = xp
+    for e in range(E):
+        if counts[e]:
+            close(outs[0][seg[e]:seg[e + 1]], xb[seg[e]:seg[e + 1]] @ w[e], 1e-2, f"group {e}")
+    assert not outs[0][seg[E]:].any(), "rows past the last group must not be written"
+
+
 @pytest.mark.parametrize("tile,m,f,k", [(1, 128, 128, 64), (2, 256, 256, 128), (4, 512, 256, 192),
                                         (3, 384, 256, 128),
                                         # split into 256x256 + 128x256 launches: the forward at
