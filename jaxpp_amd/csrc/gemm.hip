@@ -58,15 +58,16 @@ struct GemmParams {
   int n_seg, group_mode;
   int64_t group_rows;
   long stride_b, stride_c;
-  // JPP_GROUP_M as two launches (see group_head_rows): 1 = the 256x256 tiles of the rows
-  // before the split, 2 = smaller tiles over the rows behind it, 0 = one launch for all rows
-  int tail_split;
   // rotary embedding in the bf16 epilogue of the forward kernels (NULL: none): columns
   // [0, rope_cols) are heads of rope_hd elements, row r is position (rope_row0 + r) % rope_seq
   const float* rope_cos;
   const float* rope_sin;
   int rope_cols, rope_seq, rope_hd;
   long rope_row0;
+  // JPP_GROUP_M with a bf16 epilogue as two launches (see group_head_rows): 1 = the 256x256
+  // tiles of the rows before the split, 2 = smaller tiles over the rows behind it, 0 = one
+  // launch for all rows
+  int tail_split;
 };
 
 // One more problem of a launch that covers several independent products of one kind (same
@@ -260,12 +261,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   tile_of_block(p.group_mode == JPP_GROUP_K ? bid % tiles : bid, p.tiles_m, p.tiles_n, tm, tn);
   long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
-  if (p.group_mode == JPP_GROUP_M && p.tail_split) {
-    const long head = group_head_rows(p.seg[p.n_seg], p.n);
-    if (p.tail_split == 1) {
-      if (m0 >= head) return;
-    } else {
-      m0 += head;
+  if constexpr (EPI == JPP_EPI_BF16 && !KP && !MP) {   // (the launcher splits these only)
+    if (p.group_mode == JPP_GROUP_M && p.tail_split) {
+      const long head = group_head_rows(p.seg[p.n_seg], p.n);
+      if (p.tail_split == 1 && m0 >= head) return;
+      if (p.tail_split == 2) m0 += head;
     }
   }
 
