@@ -151,9 +151,10 @@ typedef struct {
    * offsets of the expert groups in the token-permuted buffers, multiples of 256.
    *   JPP_GROUP_M: rows of A and C are grouped; group e multiplies b + e * stride_b.
    *                m is the capacity of the permuted buffer; tiles past seg[n_seg] exit.
-   *                With tile = 0 and JPP_EPI_BF16 the product is two launches: when the
-   *                256x256 tiles of the seg[n_seg] rows in use end in a round that fills at
-   *                most half of the CUs, that round's rows are 128x128 tiles (same bits).
+   *                With tile = 0 and JPP_EPI_BF16 the product is up to three launches: when
+   *                the 256x256 tiles of the seg[n_seg] rows in use end in a round that fills
+   *                at most half of the CUs, that round's rows are 128x128 or 128x256 tiles
+   *                (same bits).
    *   JPP_GROUP_K: (weight gradients) C_e = c + e * stride_c gets the product over the
    *                rows seg[e] .. seg[e+1] (multiples of 64) of A and B; k is ignored.  Also
    *                the way to split one long contraction over workgroups: equal ranges, an

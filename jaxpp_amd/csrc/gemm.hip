@@ -64,9 +64,9 @@ struct GemmParams {
   const float* rope_sin;
   int rope_cols, rope_seq, rope_hd;
   long rope_row0;
-  // JPP_GROUP_M with a bf16 epilogue as two launches (see group_head_rows): 1 = the 256x256
-  // tiles of the rows before the split, 2 = smaller tiles over the rows behind it, 0 = one
-  // launch for all rows
+  // JPP_GROUP_M with a bf16 epilogue as three launches (see group_head_rows): 1 = the 256x256
+  // tiles of the rows before the split, 2 / 3 = 128x128 / 128x256 tiles over the rows behind
+  // it (one of the two finds work), 0 = one launch for all rows
   int tail_split;
 };
 
@@ -189,11 +189,14 @@ __device__ __forceinline__ const bf16_t* part_ptr(const bf16_t* p0, const bf16_t
 // Row-grouped products know the number of rows in use (`rows`, a multiple of 256) on the
 // device only; the grid covers the buffer's capacity.  When the 256x256 tiles of those rows
 // end in a round that fills at most half of the 256 CUs, the tile rows of that round are
-// left to a second launch of 128x128 tiles (four times as many tiles, a round of which takes
-// about a third of the time): returns the first row of that part, `rows` when there is none.
-__device__ __forceinline__ long group_head_rows(int rows, int n) {
+// left to a second launch of smaller tiles: 128x128 when the round holds at most 64 tiles
+// (at most one round of the small tiles, about 0.43 of the time), 128x256 when it holds up to
+// 128 (one round again, about 0.6).  Returns the first row of that part (`rows` when there
+// is none) and which of the two launches it belongs to (tail_split values 2 and 3).
+__device__ __forceinline__ long group_head_rows(int rows, int n, int& tail_kind) {
   const int tm = rows / 256, tn = n / 256, total = tm * tn, rest = total % 256;
   const bool split = total > 256 && rest > 0 && rest <= 128 && rest % tn == 0;
+  tail_kind = rest <= 64 ? 2 : 3;
   return split ? (long)(tm - rest / tn) * 256 : (long)rows;
 }
 // K-steps that hold data of row group e of a grouped contraction
@@ -263,9 +266,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   const long n0 = (long)tn * BN;
   if constexpr (EPI == JPP_EPI_BF16 && !KP && !MP) {   // (the launcher splits these only)
     if (p.group_mode == JPP_GROUP_M && p.tail_split) {
-      const long head = group_head_rows(p.seg[p.n_seg], p.n);
-      if (p.tail_split == 1 && m0 >= head) return;
-      if (p.tail_split == 2) m0 += head;
+      int tail_kind;
+      const long head = group_head_rows(p.seg[p.n_seg], p.n, tail_kind);
+      if (p.tail_split == 1 ? m0 >= head : p.tail_split != tail_kind) return;
+      if (p.tail_split != 1) m0 += head;
     }
   }
 
@@ -769,7 +773,7 @@ int launch(hipStream_t stream, GemmParams& p) {
                     : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;
   double am = p.m, ak = (double)p.k * (p.k_parts > 1 ? p.k_parts : 1), copies = 1;
   if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
-  if (p.tail_split == 2) am = 0;   // the launch over the rows before the split carries the product's work
+  if (p.tail_split >= 2) am = 0;   // the launch over the rows before the split carries the product's work
   if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
   const double b_bytes = 2.0 * p.n * ak * (p.group_mode == JPP_GROUP_M ? p.n_seg : 1);
   ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW, NS>(), 2.0 * am * p.n * ak,
@@ -1059,17 +1063,20 @@ extern "C" int jpp_gemm_bf16(void* stream_, const jpp_gemm_args* a) {
     }
   }
   // Row groups: how many rows are in use is known on the device only, so the same split is
-  // made there (group_head_rows) - the second launch is always enqueued and its workgroups
-  // leave at once when the first one's tiles cover every row.
+  // made there (group_head_rows) - the launches of small tiles are always enqueued and the
+  // workgroups of those that find no rows of theirs leave at once.
   if (tile == 4 && a->tile == 0 && a->group_mode == JPP_GROUP_M && a->epilogue == JPP_EPI_BF16) {
     const long tm = a->m / 256, tn = a->n / 256;
     if (tm * tn > 256 && tn <= 128) {
-      GemmParams head = p, tail = p;
+      GemmParams head = p, small = p, wide = p;
       head.tail_split = 1;
-      tail.tail_split = 2;
-      tail.m = (int)std::min<long>(a->m, 128 / tn * 256);   // at most 128 tiles of 256x256
-      const int rc = dispatch(stream, a, head, 4);
-      return rc != JPP_OK ? rc : dispatch(stream, a, tail, 1);
+      small.tail_split = 2;
+      small.m = (int)std::min<long>(a->m, 64 / tn * 256);    // at most 64 tiles of 256x256
+      wide.tail_split = 3;
+      wide.m = (int)std::min<long>(a->m, 128 / tn * 256);    // at most 128
+      int rc = dispatch(stream, a, head, 4);
+      if (rc == JPP_OK && small.m > 0) rc = dispatch(stream, a, small, 1);
+      return rc != JPP_OK ? rc : dispatch(stream, a, wide, 3);
     }
   }
   return dispatch(stream, a, p, tile);

@@ -4,6 +4,8 @@
 // prefix sums in token order, reductions run in a fixed order.
 #include <math.h>
 
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
@@ -258,17 +260,22 @@ __global__ __launch_bounds__(256) void scatter_dy_kernel(const El* __restrict__ 
   }
 }
 
-// dx[t] = dxp[row_of[t,0]] + dxp[row_of[t,1]] + dlogits[t] Wr^T
+// dx[t] = dxp[row_of[t,0]] + dxp[row_of[t,1]] + dlogits[t] Wr^T.  A thread owns 8 columns and
+// keeps their 8 x 8 router weights in registers; the workgroup walks tokens together, so a
+// token's rows and logit gradients are the same address for every lane (scalar loads) and
+// the vector memory path carries the two expert rows and the result only.
 template <typename El>
 __global__ __launch_bounds__(256) void combine_bwd_kernel(const El* __restrict__ dxp,
                                                           const int* __restrict__ row_of,
                                                           const float* __restrict__ dlogits,
                                                           const El* __restrict__ wr, long T,
                                                           int h, El* __restrict__ dx) {
-  const int hc = h / 8;
-  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < T * hc; i += (long)gridDim.x * 256) {
-    const long t = i / hc;
-    const int c = (int)(i - t * hc);
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= h / 8) return;
+  float w[8][kE];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) load8(wr + (long)(c * 8 + j) * kE, w[j]);
+  for (long t = blockIdx.x; t < T; t += gridDim.x) {
     float a[8], b[8], dl[kE];
     load8(dxp + (long)row_of[t * 2] * h + c * 8, a);
     load8(dxp + (long)row_of[t * 2 + 1] * h + c * 8, b);
@@ -276,11 +283,9 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const El* __restrict__
     for (int e = 0; e < kE; ++e) dl[e] = dlogits[t * kE + e];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      float w[8];
-      load8(wr + (long)(c * 8 + j) * kE, w);
       float r = 0.f;
 #pragma unroll
-      for (int e = 0; e < kE; ++e) r += dl[e] * w[e];
+      for (int e = 0; e < kE; ++e) r += dl[e] * w[j][e];
       a[j] = (a[j] + b[j]) + r;
     }
     store8(dx + t * h + c * 8, a);
@@ -293,25 +298,39 @@ template <typename El>
 __global__ __launch_bounds__(256) void wr_partial_kernel(const El* __restrict__ x,
                                                          const float* __restrict__ dlogits, long T,
                                                          int h, float* __restrict__ partial) {
-  const int j = blockIdx.y * 256 + threadIdx.x;
-  if (j >= h) return;
-  float acc[kE];
+  // a thread owns 8 columns (one 16-byte piece of a bf16 row per token); a column's terms are
+  // added in token order
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= h / 8) return;
+  float acc[8][kE];
 #pragma unroll
-  for (int e = 0; e < kE; ++e) acc[e] = 0.f;
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int e = 0; e < kE; ++e) acc[j][e] = 0.f;
+  // (few workgroups for this much data: 16 row pieces per lane in flight keep memory busy)
+#pragma unroll 16
   for (long t = blockIdx.x; t < T; t += gridDim.x) {
-    const float xv = to_f32(x[t * h + j]);
+    float xv[8], dl[kE];
+    load8(x + t * h + c * 8, xv);
 #pragma unroll
-    for (int e = 0; e < kE; ++e) acc[e] += xv * dlogits[t * kE + e];
+    for (int e = 0; e < kE; ++e) dl[e] = dlogits[t * kE + e];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < kE; ++e) acc[j][e] += xv[j] * dl[e];
   }
-  float* dst = partial + ((long)blockIdx.x * h + j) * kE;
+  float* dst = partial + ((long)blockIdx.x * h + c * 8) * kE;
 #pragma unroll
-  for (int e = 0; e < kE; ++e) dst[e] = acc[e];
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int e = 0; e < kE; ++e) dst[j * kE + e] = acc[j][e];
 }
 __global__ __launch_bounds__(256) void wr_reduce_kernel(const float* __restrict__ partial, int nb,
                                                         long n, float* __restrict__ acc) {
   const long i = (long)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = 0.f;
+#pragma unroll 16
   for (int b = 0; b < nb; ++b) s += partial[(long)b * n + i];
   acc[i] += s;
 }
@@ -434,12 +453,15 @@ int jpp_moe_combine_bwd(void* stream, const jpp_moe_args* a, const void* dxp,
   JPP_REQUIRE(a && dxp && dlogits && dx, "moe_combine_bwd: null operand");
   ProbeScope probe((hipStream_t)stream, "moe_combine_bwd", 0,
                    (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden * (a->top_k + 1));
+  // 256 threads cover 2048 columns; about 16 tokens per workgroup
+  const dim3 cgrid((unsigned)std::min<long>((a->tokens + 15) / 16, 4096),
+                   (unsigned)((a->hidden / 8 + 255) / 256));
   if (a->dtype == JPP_DTYPE_F32) {
-    hipLaunchKernelGGL(combine_bwd_kernel<float>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
+    hipLaunchKernelGGL(combine_bwd_kernel<float>, cgrid, dim3(256), 0,
                        (hipStream_t)stream, (const float*)dxp, a->row_of, dlogits,
                        (const float*)a->wr, (long)a->tokens, (int)a->hidden, (float*)dx);
   } else {
-    hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, dim3(grid_for(a->tokens * (a->hidden / 8))), dim3(256), 0,
+    hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, cgrid, dim3(256), 0,
                        (hipStream_t)stream, (const bf16_t*)dxp, a->row_of, dlogits,
                        (const bf16_t*)a->wr, (long)a->tokens, (int)a->hidden, (bf16_t*)dx);
   }
@@ -454,10 +476,10 @@ int jpp_moe_router_wgrad(void* stream, const jpp_moe_args* a, const void* x, con
   ProbeScope probe(st, "moe_router_wgrad", 0, (a->dtype == JPP_DTYPE_F32 ? 4.0 : 2.0) * a->tokens * a->hidden);
   const int nb = 64;
   if (a->dtype == JPP_DTYPE_F32) {
-    hipLaunchKernelGGL(wr_partial_kernel<float>, dim3(nb, (unsigned)((a->hidden + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL(wr_partial_kernel<float>, dim3(nb, (unsigned)((a->hidden / 8 + 255) / 256)), dim3(256), 0,
                        st, (const float*)x, dlogits, (long)a->tokens, (int)a->hidden, partial);
   } else {
-    hipLaunchKernelGGL(wr_partial_kernel<bf16_t>, dim3(nb, (unsigned)((a->hidden + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL(wr_partial_kernel<bf16_t>, dim3(nb, (unsigned)((a->hidden / 8 + 255) / 256)), dim3(256), 0,
                        st, (const bf16_t*)x, dlogits, (long)a->tokens, (int)a->hidden, partial);
   }
   const long n = (long)a->hidden * kE;

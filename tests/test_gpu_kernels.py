@@ -647,13 +647,16 @@ def test_grouped_gemm():
     ([520, 300, 256, 1100, 700, 300, 255, 513], 2048),   # ... with the deeper prefetch of a long contraction
     ([512, 512, 512, 512, 512, 512, 512, 512], 128),     # 16 x 16 = one full round: nothing to split
     ([1024, 512, 512, 512, 512, 512, 512, 600], 128),    # 19 x 16: 48 tiles -> 3 rows split off
+    ([1024, 512, 512, 512, 512, 512, 512, 1300], 128),   # 22 x 16: 96 tiles -> 6 rows split off, as 128x256 tiles
+    ([1024, 512, 512, 512, 512, 512, 512, 1300], 2048),
     ([2048, 512, 512, 512, 512, 512, 512, 1300], 128),   # 26 x 16: 160 tiles in the last round: no split
     ([256, 0, 0, 0, 0, 0, 0, 1], 128),                   # 2 x 16: less than a round: no split
-], ids=["rest64", "rest64-long", "full", "rest48", "rest160", "small"])
+], ids=["rest64", "rest64-long", "full", "rest48", "rest96", "rest96-long", "rest160", "small"])
 def test_grouped_gemm_last_round(counts, h, trans_b):
     """Row-grouped products whose 256x256 tiles end in a round that fills at most half of the
-    CUs run that round's rows as 128x128 tiles in a second launch; where the split falls is
-    decided on the device from the rows in use.  Bit for bit the single launch on 256x256
+    CUs run that round's rows as 128x128 tiles (up to 64 tiles of 256x256) or 128x256 tiles (up
+    to 128) in launches of their own; where the split falls is decided on the device from the
+    rows in use.  Bit for bit the single launch on 256x256
     tiles (the caller's choice of tile switches the split off), and right against numpy."""
     rng = np.random.default_rng(sum(counts) + trans_b)
     E, f = 8, 4096
