@@ -651,7 +651,12 @@ def test_grouped_gemm():
     ([1024, 512, 512, 512, 512, 512, 512, 1300], 2048),
     ([2048, 512, 512, 512, 512, 512, 512, 1300], 128),   # 26 x 16: 160 tiles in the last round: no split
     ([256, 0, 0, 0, 0, 0, 0, 1], 128),                   # 2 x 16: less than a round: no split
-], ids=["rest64", "rest64-long", "full", "rest48", "rest96", "rest96-long", "rest160", "small"])
+    # 69 tile rows in groups of 8 - 10 (72 with the capacity: the XCDs split the tile columns and
+    # walk them group by group); 80 tiles in the last round -> 5 rows split off
+    ([2300, 2048, 1900, 2200, 2100, 2500, 1800, 2000], 128),
+    ([5000, 0, 300, 6100, 2100, 40, 1800, 2000], 128),   # groups of 20, 0, 2, 24, 9, 1, 8, 8 tile rows
+], ids=["rest64", "rest64-long", "full", "rest48", "rest96", "rest96-long", "rest160", "small",
+        "tall", "tall-uneven"])
 def test_grouped_gemm_last_round(counts, h, trans_b):
     """Row-grouped products whose 256x256 tiles end in a round that fills at most half of the
     CUs run that round's rows as 128x128 tiles (up to 64 tiles of 256x256) or 128x256 tiles (up
