@@ -148,6 +148,7 @@ __device__ __forceinline__ void swiglu_grad_f(float g, float u, float d, float& 
 // flight stay L2 resident.
 constexpr int kColumnSplitRows = 64;  // tile rows from which XCDs split by columns
 
+template <bool WGRAD = false>
 __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int nwg = tiles_m * tiles_n;
   if ((tiles_n & 7) == 0 && tiles_m >= kColumnSplitRows) {
@@ -166,7 +167,12 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     return;
   }
   if ((nwg & 7) == 0) pid = (pid & 7) * (nwg >> 3) + (pid >> 3);
-  constexpr int GROUP = 8;
+  // Tile rows an XCD walks at a time.  Weight gradients (both operands activations, a panel
+  // 8 MiB and more) whose output is at most 16 tiles high or wide take 4: measured, A/B on
+  // one box, -0.7 % on the weight-gradient launches of the Llama-3-8B- and Mixtral-shaped
+  // stages (-0.2 % step time); 4 for every weight gradient cost the 70B-shaped stage 0.6 %
+  // (32 x 40 .. 32 x 224 tiles), 16 for every product cost 1.8 %.
+  const int GROUP = WGRAD && (tiles_m <= 16 || tiles_n <= 16) ? 4 : 8;
   const int width = GROUP * tiles_n;
   const int group = pid / width;
   const int first = group * GROUP;
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs<MP> args) {
   const int wm = wave / WN, wn = wave % WN;
   int tm, tn;
   const int tiles = p.tiles_m * p.tiles_n;
-  tile_of_block(p.group_mode == JPP_GROUP_K ? bid % tiles : bid, p.tiles_m, p.tiles_n, tm, tn);
+  tile_of_block<TA && TB>(p.group_mode == JPP_GROUP_K ? bid % tiles : bid, p.tiles_m, p.tiles_n, tm, tn);
   long m0 = (long)tm * BM;
   const long n0 = (long)tn * BN;
   if constexpr (EPI == JPP_EPI_BF16 && !KP && !MP) {   // (the launcher splits these only)
