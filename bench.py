@@ -126,7 +126,7 @@ class Workbench:
 # of this script (the counters scaled by what they read for copy kernels of known size), keyed by
 # (workload, kernel class, microbatches per weight-gradient launch): a launch over four
 # microbatches reads four operand pairs and the accumulator once
-MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8_multi", 4): 1.3326e10,  # a layer per launch
+MEASURED_TRAFFIC = {("cfg3", "gemm_tn_accf32_256x256w8_multi", 4): 1.2677e10,  # a layer per launch
                     ("cfg3", "gemm_tn_accf32_256x256w8", 4): 2.879e9,
                     ("cfg3", "gemm_tn_accf32_256x256w8", 1): 1.005e9}  # one weight per launch
 

@@ -779,11 +779,15 @@ int launch(hipStream_t stream, GemmParams& p) {
                     : EPI == JPP_EPI_F32 ? 4 : EPI == JPP_EPI_SWIGLU ? 3 : 2;
   double am = p.m, ak = (double)p.k * (p.k_parts > 1 ? p.k_parts : 1), copies = 1;
   if (p.group_mode == JPP_GROUP_M && p.group_rows) am = p.group_rows;
-  if (p.tail_split >= 2) am = 0;   // the launch over the rows before the split carries the product's work
   if (p.group_mode == JPP_GROUP_K) { ak = p.group_rows; copies = p.n_seg; }
   const double b_bytes = 2.0 * p.n * ak * (p.group_mode == JPP_GROUP_M ? p.n_seg : 1);
-  ProbeScope probe(stream, class_name<BM, BN, TA, TB, EPI, NW, NS>(), 2.0 * am * p.n * ak,
-                   2.0 * am * ak + b_bytes + copies * am * p.n * cb);
+  // (the small-tile launches of a row-grouped product's last round add their time to the class
+  // of its 256x256 launch, which declares the whole product's work)
+  const bool tail = p.tail_split >= 2;
+  ProbeScope probe(stream, tail ? class_name<256, 256, TA, TB, EPI, 8, 2>()
+                                : class_name<BM, BN, TA, TB, EPI, NW, NS>(),
+                   tail ? 0.0 : 2.0 * am * p.n * ak,
+                   tail ? 0.0 : 2.0 * am * ak + b_bytes + copies * am * p.n * cb);
   auto kern = gemm_kernel<BM, BN, TA, TB, EPI, NW, NS, KP>;
   static_assert(SMEM <= 160 * 1024, "LDS of one CU");
   // the LDS limit of a kernel is sticky: set once per instantiation, by whichever host
