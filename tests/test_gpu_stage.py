@@ -382,8 +382,9 @@ def test_lifetime_errors():
         rt.StageExecutor(LayerSpec("bert", 128, 4, 256, 128, 1), 1, 1, 1)
 
 
-@pytest.mark.parametrize("two_streams,group", [(False, 0), (True, 0), (False, 2)],
-                         ids=["one-stream", "two-streams", "weight-gradients-in-pairs"])
+@pytest.mark.parametrize("two_streams,group", [(False, 0), (True, 0), (False, 2), (True, 2)],
+                         ids=["one-stream", "two-streams", "weight-gradients-in-pairs",
+                              "pairs-on-the-second-stream"])
 @pytest.mark.parametrize("spec,sched,n,rank", [(LLAMA, S.Interleaved1F1B(4, 2), 4, 0),
                                                (MIXTRAL, S.DualPipeV(4, 2), 4, 0)],
                          ids=["llama-interleaved", "mixtral-dualpipev"])
